@@ -1,0 +1,50 @@
+"""Shared test helpers: seeded synthetic inputs and the activation tolerance."""
+import numpy as np
+
+# Activation tolerance stated by the project goal for fp16 results.
+MAX_ABS = 2e-2
+MEAN_REL = 1e-3
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def randn_h(r, shape, std=1.0):
+    return (r.standard_normal(shape) * std).astype(np.float16)
+
+
+def check_close(got, want, max_abs=MAX_ABS, mean_rel=MEAN_REL, what=""):
+    """max |got-want| <= max_abs and mean|got-want| / mean|want| <= mean_rel"""
+    g = np.asarray(got, dtype=np.float64)
+    w = np.asarray(want, dtype=np.float64)
+    assert g.shape == w.shape, (g.shape, w.shape)
+    assert np.isfinite(g).all(), f"{what}: non-finite values in result"
+    d = np.abs(g - w)
+    ma = d.max() if d.size else 0.0
+    mr = d.mean() / max(np.abs(w).mean(), 1e-30) if d.size else 0.0
+    assert ma <= max_abs, f"{what}: max-abs {ma:.3e} > {max_abs}"
+    assert mr <= mean_rel, f"{what}: mean-rel {mr:.3e} > {mean_rel}"
+    return ma, mr
+
+
+def make_tile_linear(r, N, K, sparsity, seed, std=0.02, bias_std=0.0, oracle=None):
+    """dense W ~ N(0,std) -> seeded tile_mat via the oracle's generator"""
+    import oracle.et_oracle as orc
+
+    W = randn_h(r, (N, K), std)
+    row_ptr, row_offset = orc.gen_sparse_tile_mat(N, K, sparsity, seed)
+    data = orc.tile_pack(W, row_ptr, row_offset)
+    bias = randn_h(r, (N,), bias_std) if bias_std else np.zeros(N, np.float16)
+    return dict(W=W, row_ptr=row_ptr, row_offset=row_offset, data=data, bias=bias, N=N, K=K)
+
+
+def dense_masked(lin):
+    """dense float64 weight with pruned tiles zeroed (built without the oracle's pack)"""
+    N, K = lin["N"], lin["K"]
+    Wm = np.zeros((N, K), np.float64)
+    rp, ro = lin["row_ptr"], lin["row_offset"]
+    for bn in range(N // 16):
+        for i in range(rp[bn], rp[bn + 1]):
+            Wm[bn * 16:(bn + 1) * 16, ro[i]:ro[i] + 16] = lin["W"][bn * 16:(bn + 1) * 16, ro[i]:ro[i] + 16]
+    return Wm
