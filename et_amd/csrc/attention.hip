@@ -1,0 +1,592 @@
+// Fused multi-head self-attention for gfx950: on-the-fly (scores never leave
+// the CU), attention-aware pruned (compact Q/K/V column sets per head) and the
+// score-matrix-in-memory variant, all from one key-tiled online-softmax kernel.
+//
+// Reference math (kernels/attention.cu:51-120): Qs = half(Q*scale),
+// S = Qs K^T + mask, P = softmax_base2(S), Z = P V, per head, per 16-row query
+// block, with the whole 16 x seq_len score block in shared memory.  Here the
+// keys are walked in tiles of 64 with a running max / running sum, so LDS use
+// is independent of seq_len and no S x S block exists anywhere.
+//
+// Layout trick: both contractions are issued TRANSPOSED.
+//   S^T(keys x queries) = K_tile * Qs^T : A = K rows from LDS, B = Q fragment
+//     held in registers for the whole kernel.  A lane (c = lane%16, g =
+//     lane/16) then holds, for ONE query c, four consecutive keys 4g..4g+3 of
+//     each 16-key subtile, so row max / row sum need only two cross-lane steps
+//     (xor 16, xor 32) and the running statistics are per-lane scalars.
+//   O^T(d x queries) = V^T * P^T : the P values a lane already holds are, as
+//     they stand, the B operand (8 k-slots = 4 keys of subtile 2kk + 4 keys
+//     of subtile 2kk+1); the matching A operand is read from a V tile that was
+//     transposed while being staged into LDS.  P never goes through LDS and
+//     the O accumulator's query index is again the lane's c, so the online
+//     rescale is a per-lane multiply.
+#include "common.h"
+
+#include <cmath>
+
+namespace et {
+
+constexpr int AT_THREADS = 256;
+constexpr int AT_WAVES = 4;
+constexpr int AT_KT = 64; // keys per tile
+
+struct AttnArgs {
+    f16 *out;
+    const f16 *Q, *K, *V, *QK, *mask;
+    const int *seq_lens, *cu_seqlens;
+    const int *qk_head_ptr, *v_col_id, *v_head_ptr;
+    int ldq, ldv, ldo, seq_len, nhead, batch, nqb, total, per_xcd;
+    float log2_scale, scale;
+};
+
+__device__ __forceinline__ f16x8 load8_guard(const f16 *p, int d0, int n) {
+    f16x8 v;
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+        v[j] = (d0 + j < n) ? p[d0 + j] : (f16)0;
+    return v;
+}
+
+__device__ __forceinline__ float xor_max_16_32(float v) {
+    v = fmaxf(v, __shfl_xor(v, 16, WAVE));
+    v = fmaxf(v, __shfl_xor(v, 32, WAVE));
+    return v;
+}
+
+template <int HD, int QS, bool PRUNED, bool SHAREDQK>
+__global__ void __launch_bounds__(AT_THREADS) attention_kernel(const AttnArgs a) {
+    constexpr int DK = HD / 32;   // k-steps of Q K^T
+    constexpr int DV = HD / 16;   // 16-wide column subtiles of the output
+    constexpr int LDK = HD + 8;   // halves per staged K row
+    constexpr int LDV = AT_KT + 8; // halves per staged V^T row
+    constexpr int QB = AT_WAVES * 16 * QS; // queries per workgroup
+    constexpr int LDO = HD + 8;
+    constexpr int SM_KV = AT_KT * LDK + HD * LDV;
+    constexpr int SM_O = QB * LDO;
+    constexpr int SM = SM_KV > SM_O ? SM_KV : SM_O;
+    __shared__ __attribute__((aligned(16))) f16 smem[SM];
+    f16 *ks = smem;
+    f16 *vt = smem + AT_KT * LDK;
+
+    const int pid = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3);
+    if (pid >= a.total)
+        return;
+    const int qb = pid % a.nqb;
+    const int bh = pid / a.nqb;
+    const int h = bh % a.nhead;
+    const int b = bh / a.nhead;
+
+    int row0, len, rows_alloc; // first row, valid rows, rows that exist for this sequence
+    if (a.cu_seqlens) {
+        row0 = a.cu_seqlens[b];
+        len = a.cu_seqlens[b + 1] - row0;
+        rows_alloc = len;
+    } else {
+        row0 = b * a.seq_len;
+        len = a.seq_lens ? a.seq_lens[b] : a.seq_len;
+        rows_alloc = a.seq_len;
+    }
+    len = min(max(len, 0), a.seq_len);
+    const int q0 = qb * QB;
+    if (q0 >= rows_alloc)
+        return;
+
+    int qc0 = h * HD, nqk = HD, vc0 = h * HD, nv = HD;
+    if (PRUNED) {
+        if (a.qk_head_ptr) {
+            qc0 = a.qk_head_ptr[h];
+            nqk = min(a.qk_head_ptr[h + 1] - qc0, HD);
+        }
+        if (a.v_head_ptr) {
+            vc0 = a.v_head_ptr[h];
+            nv = min(a.v_head_ptr[h + 1] - vc0, HD);
+        }
+    }
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int c16 = lane & 15;
+    const int g4 = lane >> 4;
+    f16 *obase = a.out + (size_t)row0 * a.ldo + h * HD;
+
+    if (q0 < len) {
+        // ---- Q fragments (B operand of S^T), scaled in half like the reference
+        f16x8 qf[QS][DK];
+        const f16 sc = (f16)a.scale;
+#pragma unroll
+        for (int qs = 0; qs < QS; qs++) {
+            const int q = q0 + (wave * QS + qs) * 16 + c16;
+#pragma unroll
+            for (int s = 0; s < DK; s++) {
+                f16x8 v = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (!SHAREDQK && q < len) {
+                    const f16 *qrow = a.Q + (size_t)(row0 + q) * a.ldq + qc0;
+                    if (PRUNED)
+                        v = load8_guard(qrow, s * 32 + g4 * 8, nqk);
+                    else
+                        v = *reinterpret_cast<const f16x8 *>(qrow + s * 32 + g4 * 8);
+                }
+                qf[qs][s] = v * sc;
+            }
+        }
+
+        f32x4 ot[DV][QS];
+        float m_run[QS], l_run[QS];
+#pragma unroll
+        for (int qs = 0; qs < QS; qs++) {
+            m_run[qs] = -INFINITY;
+            l_run[qs] = 0.f;
+#pragma unroll
+            for (int d = 0; d < DV; d++)
+                ot[d][qs] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        const bool mask_vec = a.mask && ((a.seq_len & 3) == 0) &&
+                              ((reinterpret_cast<uintptr_t>(a.mask) & 7u) == 0);
+        const bool qk_vec = SHAREDQK && ((a.seq_len & 3) == 0) &&
+                            ((reinterpret_cast<uintptr_t>(a.QK) & 7u) == 0);
+
+        for (int kb = 0; kb < len; kb += AT_KT) {
+            __syncthreads(); // previous tile fully consumed
+            if (!SHAREDQK) { // stage K tile, row-major [key][d]
+                constexpr int CPR = HD / 8;
+                for (int idx = tid; idx < AT_KT * CPR; idx += AT_THREADS) {
+                    const int key = idx / CPR, dc = idx % CPR;
+                    f16x8 v = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                    if (kb + key < len) {
+                        const f16 *krow = a.K + (size_t)(row0 + kb + key) * a.ldq + qc0;
+                        if (PRUNED)
+                            v = load8_guard(krow, dc * 8, nqk);
+                        else
+                            v = *reinterpret_cast<const f16x8 *>(krow + dc * 8);
+                    }
+                    *reinterpret_cast<f16x8 *>(ks + key * LDK + dc * 8) = v;
+                }
+            }
+            { // stage V tile transposed, [d][key]; rows at or beyond len as zeros
+                constexpr int DQ = HD / 4;
+                for (int w = tid; w < (AT_KT / 4) * DQ; w += AT_THREADS) {
+                    const int dq = w % DQ, kq = w / DQ;
+                    f16x4 r4[4];
+#pragma unroll
+                    for (int kk = 0; kk < 4; kk++) {
+                        const int key = kb + kq * 4 + kk;
+                        f16x4 v = f16x4{0, 0, 0, 0};
+                        if (key < len) {
+                            const f16 *vrow = a.V + (size_t)(row0 + key) * a.ldv + vc0;
+                            if (PRUNED) {
+#pragma unroll
+                                for (int e = 0; e < 4; e++)
+                                    v[e] = (dq * 4 + e < nv) ? vrow[dq * 4 + e] : (f16)0;
+                            } else {
+                                v = *reinterpret_cast<const f16x4 *>(vrow + dq * 4);
+                            }
+                        }
+                        r4[kk] = v;
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const f16x4 t = f16x4{r4[0][e], r4[1][e], r4[2][e], r4[3][e]};
+                        *reinterpret_cast<f16x4 *>(vt + (dq * 4 + e) * LDV + kq * 4) = t;
+                    }
+                }
+            }
+            __syncthreads();
+
+            // ---- scores, transposed: st[ksub][qs][r] = S[q = c16][key = 16 ksub + 4 g4 + r]
+            f32x4 st[4][QS];
+            if (!SHAREDQK) {
+#pragma unroll
+                for (int ksub = 0; ksub < 4; ksub++) {
+#pragma unroll
+                    for (int qs = 0; qs < QS; qs++)
+                        st[ksub][qs] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s = 0; s < DK; s++) {
+                        const f16x8 kf = *reinterpret_cast<const f16x8 *>(
+                            ks + (ksub * 16 + c16) * LDK + s * 32 + g4 * 8);
+#pragma unroll
+                        for (int qs = 0; qs < QS; qs++)
+                            st[ksub][qs] = mfma16x16x32(kf, qf[qs][s], st[ksub][qs]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int qs = 0; qs < QS; qs++) {
+                    const int q = q0 + (wave * QS + qs) * 16 + c16;
+#pragma unroll
+                    for (int ksub = 0; ksub < 4; ksub++) {
+                        const int key = kb + ksub * 16 + g4 * 4;
+                        f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+                        if (q < len) {
+                            const f16 *src = a.QK + ((size_t)bh * a.seq_len + q) * a.seq_len + key;
+                            if (qk_vec && key + 3 < len) {
+                                const f16x4 t = *reinterpret_cast<const f16x4 *>(src);
+#pragma unroll
+                                for (int r = 0; r < 4; r++)
+                                    v[r] = (float)t[r];
+                            } else {
+#pragma unroll
+                                for (int r = 0; r < 4; r++)
+                                    if (key + r < len)
+                                        v[r] = (float)src[r];
+                            }
+                        }
+                        st[ksub][qs] = v;
+                    }
+                }
+            }
+
+            // ---- mask, online softmax, pack P
+            f16x8 pf[QS][2];
+#pragma unroll
+            for (int qs = 0; qs < QS; qs++) {
+                const int q = q0 + (wave * QS + qs) * 16 + c16;
+                float mx = -INFINITY;
+#pragma unroll
+                for (int ksub = 0; ksub < 4; ksub++) {
+                    const int key = kb + ksub * 16 + g4 * 4;
+                    float mk[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (a.mask && q < len) {
+                        const f16 *mrow = a.mask + (size_t)q * a.seq_len + key;
+                        if (mask_vec && key + 3 < len) {
+                            const f16x4 t = *reinterpret_cast<const f16x4 *>(mrow);
+#pragma unroll
+                            for (int r = 0; r < 4; r++)
+                                mk[r] = (float)t[r];
+                        } else {
+#pragma unroll
+                            for (int r = 0; r < 4; r++)
+                                if (key + r < len)
+                                    mk[r] = (float)mrow[r];
+                        }
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        float s = (st[ksub][qs][r] + mk[r]) * a.log2_scale;
+                        if (key + r >= len)
+                            s = -INFINITY;
+                        st[ksub][qs][r] = s;
+                        mx = fmaxf(mx, s);
+                    }
+                }
+                mx = xor_max_16_32(mx);
+                const float m_new = fmaxf(m_run[qs], mx);
+                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+                const float alpha = __builtin_amdgcn_exp2f(m_run[qs] - m_use);
+                m_run[qs] = m_new;
+                float psum = 0.f;
+                f16 ph[16];
+#pragma unroll
+                for (int ksub = 0; ksub < 4; ksub++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const float p = __builtin_amdgcn_exp2f(st[ksub][qs][r] - m_use);
+                        psum += p;
+                        ph[ksub * 4 + r] = (f16)p;
+                    }
+                l_run[qs] = l_run[qs] * alpha + psum;
+#pragma unroll
+                for (int d = 0; d < DV; d++)
+                    ot[d][qs] *= alpha;
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++)
+                    pf[qs][kk] = f16x8{ph[kk * 8 + 0], ph[kk * 8 + 1], ph[kk * 8 + 2], ph[kk * 8 + 3],
+                                       ph[kk * 8 + 4], ph[kk * 8 + 5], ph[kk * 8 + 6], ph[kk * 8 + 7]};
+            }
+
+            // ---- O^T += V^T P^T
+#pragma unroll
+            for (int d = 0; d < DV; d++) {
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++) {
+                    const f16 *vrow = vt + (d * 16 + c16) * LDV + kk * 32 + g4 * 4;
+                    const f16x4 v0 = *reinterpret_cast<const f16x4 *>(vrow);
+                    const f16x4 v1 = *reinterpret_cast<const f16x4 *>(vrow + 16);
+                    const f16x8 vf = f16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+                    for (int qs = 0; qs < QS; qs++)
+                        ot[d][qs] = mfma16x16x32(vf, pf[qs][kk], ot[d][qs]);
+                }
+            }
+        }
+
+        // ---- normalise and stage the output block in LDS
+        __syncthreads();
+        f16 *os = smem;
+        if (PRUNED) { // columns that no kept V column maps to must read as zero
+            for (int i = tid; i < SM_O / 8; i += AT_THREADS)
+                reinterpret_cast<f16x8 *>(os)[i] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            __syncthreads();
+        }
+#pragma unroll
+        for (int qs = 0; qs < QS; qs++) {
+            float l = l_run[qs];
+            l += __shfl_xor(l, 16, WAVE);
+            l += __shfl_xor(l, 32, WAVE);
+            const float inv = l > 0.f ? 1.0f / l : 0.f;
+            const int ql = (wave * QS + qs) * 16 + c16;
+#pragma unroll
+            for (int d = 0; d < DV; d++) {
+                f16x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    o[r] = (f16)(ot[d][qs][r] * inv);
+                if (PRUNED) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int j = d * 16 + g4 * 4 + r;
+                        if (j < nv) {
+                            const int col = (a.v_col_id ? a.v_col_id[vc0 + j] : vc0 + j) - h * HD;
+                            if (col >= 0 && col < HD)
+                                os[ql * LDO + col] = o[r];
+                        }
+                    }
+                } else {
+                    *reinterpret_cast<f16x4 *>(os + ql * LDO + d * 16 + g4 * 4) = o;
+                }
+            }
+        }
+        __syncthreads();
+        constexpr int CPR = HD / 8;
+        for (int idx = tid; idx < QB * CPR; idx += AT_THREADS) {
+            const int ql = idx / CPR, dc = idx % CPR;
+            const int q = q0 + ql;
+            if (q < rows_alloc) {
+                f16x8 v = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (q < len)
+                    v = *reinterpret_cast<const f16x8 *>(os + ql * LDO + dc * 8);
+                *reinterpret_cast<f16x8 *>(obase + (size_t)q * a.ldo + dc * 8) = v;
+            }
+        }
+    } else {
+        // whole query block is padding: rows exist (padded layout) and read as zero
+        constexpr int CPR = HD / 8;
+        for (int idx = tid; idx < QB * CPR; idx += AT_THREADS) {
+            const int ql = idx / CPR, dc = idx % CPR;
+            const int q = q0 + ql;
+            if (q < rows_alloc)
+                *reinterpret_cast<f16x8 *>(obase + (size_t)q * a.ldo + dc * 8) =
+                    f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+    }
+}
+
+// scaled Q K^T written to memory, [(b*nhead+h)][q][k]; one wave per 16 queries
+// x 64 keys, transposed product so a lane owns 4 consecutive keys of one query.
+template <int HD>
+__global__ void __launch_bounds__(256)
+qk_scores_kernel(f16 *__restrict__ QK, const f16 *__restrict__ Q, const f16 *__restrict__ K,
+                 int seq_len, int d_model, int nhead, float scale) {
+    constexpr int DK = HD / 32;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, c16 = lane & 15, g4 = lane >> 4;
+    const int bh = blockIdx.z, h = bh % nhead, b = bh / nhead;
+    const int q0 = blockIdx.y * 16;
+    const int k0 = (blockIdx.x * 4 + wave) * 64;
+    if (k0 >= seq_len)
+        return;
+    const size_t row0 = (size_t)b * seq_len;
+    const int q = q0 + c16;
+    f16x8 qf[DK];
+#pragma unroll
+    for (int s = 0; s < DK; s++) {
+        qf[s] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (q < seq_len)
+            qf[s] = *reinterpret_cast<const f16x8 *>(Q + (row0 + q) * d_model + h * HD + s * 32 + g4 * 8);
+    }
+#pragma unroll
+    for (int ksub = 0; ksub < 4; ksub++) {
+        const int key = k0 + ksub * 16 + c16;
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < DK; s++) {
+            f16x8 kf = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (key < seq_len)
+                kf = *reinterpret_cast<const f16x8 *>(K + (row0 + key) * d_model + h * HD + s * 32 + g4 * 8);
+            acc = mfma16x16x32(kf, qf[s], acc);
+        }
+        if (q < seq_len) {
+            f16 *dst = QK + ((size_t)bh * seq_len + q) * seq_len + k0 + ksub * 16 + g4 * 4;
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                if (k0 + ksub * 16 + g4 * 4 + r < seq_len)
+                    dst[r] = (f16)(acc[r] * scale);
+        }
+    }
+}
+
+template <int HD, bool PRUNED, bool SHAREDQK>
+static void attn_launch_qs(int qs, const AttnArgs &a, hipStream_t st) {
+    if (qs == 2)
+        hipLaunchKernelGGL((attention_kernel<HD, 2, PRUNED, SHAREDQK>), dim3(a.per_xcd * 8),
+                           dim3(AT_THREADS), 0, st, a);
+    else
+        hipLaunchKernelGGL((attention_kernel<HD, 1, PRUNED, SHAREDQK>), dim3(a.per_xcd * 8),
+                           dim3(AT_THREADS), 0, st, a);
+}
+
+static float head_scale(int hd) {
+    // half(sqrt(1/head_dim)), kernels/attention.cu:126
+    return (float)(f16)sqrtf(1.0f / (float)hd);
+}
+
+static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedqk,
+                              hipStream_t st, const char *who) {
+    ET_REQUIRE(a.out && a.V, ET_ERR_INVALID_ARG, "%s: null pointer", who);
+    ET_REQUIRE(sharedqk ? a.QK != nullptr : (a.Q && a.K), ET_ERR_INVALID_ARG, "%s: null pointer", who);
+    ET_REQUIRE(a.seq_len > 0 && d_model > 0 && a.nhead > 0 && a.batch > 0, ET_ERR_INVALID_ARG,
+               "%s: seq_len=%d d_model=%d nhead=%d batch=%d", who, a.seq_len, d_model, a.nhead, a.batch);
+    ET_REQUIRE(d_model % a.nhead == 0, ET_ERR_INVALID_ARG, "%s: d_model %% nhead != 0", who);
+    const int hd = d_model / a.nhead;
+    ET_REQUIRE(hd == 32 || hd == 64 || hd == 128, ET_ERR_UNSUPPORTED,
+               "%s: head_dim %d not in {32,64,128}", who, hd);
+    ET_REQUIRE(aligned16(a.out) && aligned16(a.Q) && aligned16(a.K) && aligned16(a.V),
+               ET_ERR_ALIGNMENT, "%s: out/Q/K/V must be 16-byte aligned", who);
+    if (!pruned) {
+        ET_REQUIRE(a.ldq % 8 == 0 && a.ldv % 8 == 0, ET_ERR_ALIGNMENT,
+                   "%s: d_model must be a multiple of 8", who);
+    }
+    a.ldo = d_model;
+    a.scale = head_scale(hd);
+    // queries per workgroup: 128 when that still fills the chip, else 64
+    int qs = 2;
+    {
+        const long wg128 = (long)((a.seq_len + 127) / 128) * a.nhead * a.batch;
+        if (wg128 < 512 || hd == 128)
+            qs = 1;
+    }
+    const int QB = AT_WAVES * 16 * qs;
+    a.nqb = (a.seq_len + QB - 1) / QB;
+    a.total = a.nqb * a.nhead * a.batch;
+    a.per_xcd = (a.total + 7) / 8;
+#define ET_ATTN_CASE(HDV)                                                                         \
+    if (hd == HDV) {                                                                              \
+        if (sharedqk) attn_launch_qs<HDV, false, true>(qs, a, st);                                \
+        else if (pruned) attn_launch_qs<HDV, true, false>(qs, a, st);                             \
+        else attn_launch_qs<HDV, false, false>(qs, a, st);                                        \
+    }
+    ET_ATTN_CASE(32)
+    ET_ATTN_CASE(64)
+    ET_ATTN_CASE(128)
+#undef ET_ATTN_CASE
+    return launch_status(who);
+}
+
+} // namespace et
+
+extern "C" int et_OTF_attention(void *out, const void *Q, const void *K, const void *V,
+                                const void *mask, int seq_len, int d_model, int nhead, int batch,
+                                const int *seq_lens, float log2_scale, void *stream) {
+    using namespace et;
+    AttnArgs a = {};
+    a.out = static_cast<f16 *>(out);
+    a.Q = static_cast<const f16 *>(Q);
+    a.K = static_cast<const f16 *>(K);
+    a.V = static_cast<const f16 *>(V);
+    a.mask = static_cast<const f16 *>(mask);
+    a.seq_lens = seq_lens;
+    a.ldq = a.ldv = d_model;
+    a.seq_len = seq_len;
+    a.nhead = nhead;
+    a.batch = batch;
+    a.log2_scale = log2_scale;
+    return attention_dispatch(a, d_model, false, false, static_cast<hipStream_t>(stream),
+                              "et_OTF_attention");
+}
+
+extern "C" int et_OTF_attention_varlen(void *out, const void *Q, const void *K, const void *V,
+                                       const void *mask, const int *cu_seqlens, int max_seq_len,
+                                       int d_model, int nhead, int batch, float log2_scale,
+                                       void *stream) {
+    using namespace et;
+    ET_REQUIRE(cu_seqlens, ET_ERR_INVALID_ARG, "et_OTF_attention_varlen: null cu_seqlens");
+    AttnArgs a = {};
+    a.out = static_cast<f16 *>(out);
+    a.Q = static_cast<const f16 *>(Q);
+    a.K = static_cast<const f16 *>(K);
+    a.V = static_cast<const f16 *>(V);
+    a.mask = static_cast<const f16 *>(mask);
+    a.cu_seqlens = cu_seqlens;
+    a.ldq = a.ldv = d_model;
+    a.seq_len = max_seq_len;
+    a.nhead = nhead;
+    a.batch = batch;
+    a.log2_scale = log2_scale;
+    return attention_dispatch(a, d_model, false, false, static_cast<hipStream_t>(stream),
+                              "et_OTF_attention_varlen");
+}
+
+extern "C" int et_Prune_attention(void *out, const void *Q, const void *K, const void *V,
+                                  const int *qk_head_ptr, int ldqk, const int *v_col_id,
+                                  const int *v_head_ptr, int ldv, const void *mask, int seq_len,
+                                  int d_model, int nhead, int batch, const int *seq_lens,
+                                  float log2_scale, void *stream) {
+    using namespace et;
+    AttnArgs a = {};
+    a.out = static_cast<f16 *>(out);
+    a.Q = static_cast<const f16 *>(Q);
+    a.K = static_cast<const f16 *>(K);
+    a.V = static_cast<const f16 *>(V);
+    a.mask = static_cast<const f16 *>(mask);
+    a.seq_lens = seq_lens;
+    a.qk_head_ptr = qk_head_ptr;
+    a.v_col_id = v_col_id;
+    a.v_head_ptr = v_head_ptr;
+    a.ldq = qk_head_ptr ? ldqk : d_model;
+    a.ldv = v_head_ptr ? ldv : d_model;
+    ET_REQUIRE(a.ldq > 0 && a.ldv > 0, ET_ERR_INVALID_ARG, "et_Prune_attention: ldqk=%d ldv=%d", ldqk, ldv);
+    ET_REQUIRE(!v_col_id || v_head_ptr, ET_ERR_INVALID_ARG,
+               "et_Prune_attention: v_col_id given without v_head_ptr");
+    a.seq_len = seq_len;
+    a.nhead = nhead;
+    a.batch = batch;
+    a.log2_scale = log2_scale;
+    return attention_dispatch(a, d_model, true, false, static_cast<hipStream_t>(stream),
+                              "et_Prune_attention");
+}
+
+extern "C" int et_sharedQK_attention(void *out, const void *QK, const void *V, const void *mask,
+                                     int seq_len, int d_model, int nhead, int batch,
+                                     const int *seq_lens, float log2_scale, void *stream) {
+    using namespace et;
+    AttnArgs a = {};
+    a.out = static_cast<f16 *>(out);
+    a.QK = static_cast<const f16 *>(QK);
+    a.V = static_cast<const f16 *>(V);
+    a.mask = static_cast<const f16 *>(mask);
+    a.seq_lens = seq_lens;
+    a.ldq = a.ldv = d_model;
+    a.seq_len = seq_len;
+    a.nhead = nhead;
+    a.batch = batch;
+    a.log2_scale = log2_scale;
+    return attention_dispatch(a, d_model, false, true, static_cast<hipStream_t>(stream),
+                              "et_sharedQK_attention");
+}
+
+extern "C" int et_qk_scores(void *QK, const void *Q, const void *K, int seq_len, int d_model,
+                            int nhead, int batch, void *stream) {
+    using namespace et;
+    ET_REQUIRE(QK && Q && K, ET_ERR_INVALID_ARG, "et_qk_scores: null pointer");
+    ET_REQUIRE(seq_len > 0 && d_model > 0 && nhead > 0 && batch > 0 && d_model % nhead == 0,
+               ET_ERR_INVALID_ARG, "et_qk_scores: bad sizes");
+    const int hd = d_model / nhead;
+    ET_REQUIRE(hd == 32 || hd == 64 || hd == 128, ET_ERR_UNSUPPORTED,
+               "et_qk_scores: head_dim %d not in {32,64,128}", hd);
+    ET_REQUIRE(aligned16(Q) && aligned16(K) && d_model % 8 == 0, ET_ERR_ALIGNMENT,
+               "et_qk_scores: Q/K must be 16-byte aligned");
+    // scale = half(1/sqrt(head_dim)), encoder/encoder.cu:113
+    const float scale = (float)(f16)(1.0f / sqrtf((float)hd));
+    const dim3 grid((seq_len + 255) / 256, (seq_len + 15) / 16, batch * nhead), block(256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    f16 *o = static_cast<f16 *>(QK);
+    const f16 *q = static_cast<const f16 *>(Q), *k = static_cast<const f16 *>(K);
+    if (hd == 32)
+        hipLaunchKernelGGL(qk_scores_kernel<32>, grid, block, 0, st, o, q, k, seq_len, d_model, nhead, scale);
+    else if (hd == 64)
+        hipLaunchKernelGGL(qk_scores_kernel<64>, grid, block, 0, st, o, q, k, seq_len, d_model, nhead, scale);
+    else
+        hipLaunchKernelGGL(qk_scores_kernel<128>, grid, block, 0, st, o, q, k, seq_len, d_model, nhead, scale);
+    return launch_status("et_qk_scores");
+}

@@ -1,0 +1,77 @@
+// Shared device/host helpers for the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/et_amd.h"
+
+namespace et {
+
+// ---- error plumbing -------------------------------------------------------
+void set_error(const char *fmt, ...);
+int hip_fail(hipError_t e, const char *what);
+
+#define ET_HIP(call)                                                           \
+    do {                                                                       \
+        hipError_t e__ = (call);                                               \
+        if (e__ != hipSuccess)                                                 \
+            return ::et::hip_fail(e__, #call);                                 \
+    } while (0)
+
+#define ET_REQUIRE(cond, code, ...)                                            \
+    do {                                                                       \
+        if (!(cond)) {                                                         \
+            ::et::set_error(__VA_ARGS__);                                      \
+            return (code);                                                     \
+        }                                                                      \
+    } while (0)
+
+static inline bool aligned16(const void *p) {
+    return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+static inline int launch_status(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+        return hip_fail(e, what);
+    return ET_OK;
+}
+
+// ---- vector types -----------------------------------------------------------
+typedef _Float16 f16;
+typedef f16 f16x2 __attribute__((ext_vector_type(2)));
+typedef f16 f16x4 __attribute__((ext_vector_type(4)));
+typedef f16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int WAVE = 64;
+
+// D(16x16,f32) += A(16x32,f16) * B(32x16,f16).
+// Register layout (wave64), g = lane/16, c = lane%16:
+//   a[j] = A[c][8g+j], b[j] = B[8g+j][c], d[r] = D[4g+r][c].
+// Only the pairing of a[j] with b[j] inside the same lane group matters for
+// the contraction, so any consistent assignment of k to (g,j) works.
+__device__ __forceinline__ f32x4 mfma16x16x32(f16x8 a, f16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
+
+// ---- wave64 reductions (all lanes receive the result) -----------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1)
+        v += __shfl_xor(v, m, WAVE);
+    return v;
+}
+
+__device__ __forceinline__ float f16_bits_to_float(uint16_t b) {
+    return (float)__builtin_bit_cast(f16, b);
+}
+
+} // namespace et

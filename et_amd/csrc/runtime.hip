@@ -1,0 +1,212 @@
+// Error reporting, device-memory plumbing and the small data-movement kernels
+// of the sequence-length-aware path.
+#include "common.h"
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstring>
+
+namespace et {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int hip_fail(hipError_t e, const char *what) {
+    set_error("%s: %s", what, hipGetErrorString(e));
+    return ET_ERR_HIP;
+}
+
+// one workgroup per (sequence, position), 16-byte copies
+__global__ void __launch_bounds__(128)
+pack_rows_kernel(f16 *__restrict__ packed, const f16 *__restrict__ padded,
+                 const int *__restrict__ cu, int seq_len, int width) {
+    const int b = blockIdx.y, t = blockIdx.x;
+    const int start = cu[b], len = cu[b + 1] - start;
+    if (t >= len)
+        return;
+    const int nch = width >> 3;
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(padded + ((size_t)b * seq_len + t) * width);
+    u32x4 *dst = reinterpret_cast<u32x4 *>(packed + (size_t)(start + t) * width);
+    for (int c = threadIdx.x; c < nch; c += blockDim.x)
+        dst[c] = src[c];
+}
+
+__global__ void __launch_bounds__(128)
+unpack_rows_kernel(f16 *__restrict__ padded, const f16 *__restrict__ packed,
+                   const int *__restrict__ cu, int seq_len, int width) {
+    const int b = blockIdx.y, t = blockIdx.x;
+    const int start = cu[b], len = cu[b + 1] - start;
+    const int nch = width >> 3;
+    u32x4 *dst = reinterpret_cast<u32x4 *>(padded + ((size_t)b * seq_len + t) * width);
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(packed + (size_t)(start + t) * width);
+    for (int c = threadIdx.x; c < nch; c += blockDim.x)
+        dst[c] = (t < len) ? src[c] : u32x4{0u, 0u, 0u, 0u};
+}
+
+// one workgroup per row; the inverse column map (dst column -> source column
+// or -1) is built in LDS
+__global__ void __launch_bounds__(256)
+scatter_cols_kernel(f16 *__restrict__ out, const f16 *__restrict__ in,
+                    const int *__restrict__ col_id, int n, int ld_in, int width) {
+    extern __shared__ int inv[];
+    for (int c = threadIdx.x; c < width; c += blockDim.x)
+        inv[c] = -1;
+    __syncthreads();
+    for (int j = threadIdx.x; j < n; j += blockDim.x)
+        inv[col_id[j]] = j;
+    __syncthreads();
+    const size_t r = blockIdx.x;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        const int j = inv[c];
+        out[r * width + c] = j >= 0 ? in[r * ld_in + j] : (f16)0;
+    }
+}
+
+__global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t nwords) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nwords;
+         i += (size_t)gridDim.x * blockDim.x)
+        p[i] = 0u;
+}
+
+} // namespace et
+
+extern "C" {
+
+const char *et_strerror(int code) {
+    switch (code) {
+    case ET_OK: return "ok";
+    case ET_ERR_INVALID_ARG: return "invalid argument";
+    case ET_ERR_ALIGNMENT: return "misaligned pointer or leading dimension";
+    case ET_ERR_UNSUPPORTED: return "unsupported shape";
+    case ET_ERR_HIP: return "HIP runtime error";
+    case ET_ERR_FORMAT: return "malformed pruned-weight format";
+    default: return "unknown error";
+    }
+}
+
+const char *et_last_error(void) { return et::g_err; }
+int et_abi_version(void) { return 1; }
+
+int et_malloc(void **ptr, size_t bytes) {
+    ET_REQUIRE(ptr, ET_ERR_INVALID_ARG, "et_malloc: null out pointer");
+    *ptr = nullptr;
+    ET_HIP(hipMalloc(ptr, bytes ? bytes : 16));
+    return ET_OK;
+}
+int et_free(void *ptr) {
+    if (ptr)
+        ET_HIP(hipFree(ptr));
+    return ET_OK;
+}
+int et_memcpy_h2d(void *dst, const void *src, size_t bytes) {
+    if (bytes)
+        ET_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return ET_OK;
+}
+int et_memcpy_d2h(void *dst, const void *src, size_t bytes) {
+    if (bytes)
+        ET_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return ET_OK;
+}
+int et_memcpy_d2d_async(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes)
+        ET_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
+    return ET_OK;
+}
+int et_fill_zero(void *dst, size_t bytes, void *stream) {
+    using namespace et;
+    ET_REQUIRE(dst || bytes == 0, ET_ERR_INVALID_ARG, "et_fill_zero: null pointer");
+    ET_REQUIRE(bytes % 4 == 0 && (reinterpret_cast<uintptr_t>(dst) & 3u) == 0, ET_ERR_ALIGNMENT,
+               "et_fill_zero: needs 4-byte granularity");
+    if (!bytes)
+        return ET_OK;
+    const size_t nw = bytes / 4;
+    const int grid = (int)std::min<size_t>((nw + 255) / 256, 4096);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<uint32_t *>(dst), nw);
+    return launch_status("et_fill_zero");
+}
+int et_stream_create(void **stream) {
+    ET_REQUIRE(stream, ET_ERR_INVALID_ARG, "et_stream_create: null out pointer");
+    hipStream_t s;
+    ET_HIP(hipStreamCreate(&s));
+    *stream = s;
+    return ET_OK;
+}
+int et_stream_destroy(void *stream) {
+    if (stream)
+        ET_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+    return ET_OK;
+}
+int et_stream_synchronize(void *stream) {
+    ET_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    return ET_OK;
+}
+int et_device_synchronize(void) {
+    ET_HIP(hipDeviceSynchronize());
+    return ET_OK;
+}
+int et_device_cu_count(void) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess)
+        return 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        return 0;
+    return n;
+}
+
+static int pack_check(const void *packed, const void *padded, const int *cu, int batch,
+                      int seq_len, int width, const char *who) {
+    using namespace et;
+    ET_REQUIRE(packed && padded && cu, ET_ERR_INVALID_ARG, "%s: null pointer", who);
+    ET_REQUIRE(batch > 0 && seq_len > 0 && width > 0, ET_ERR_INVALID_ARG, "%s: bad sizes", who);
+    ET_REQUIRE(width % 8 == 0 && aligned16(packed) && aligned16(padded), ET_ERR_ALIGNMENT,
+               "%s: width must be a multiple of 8 and pointers 16-byte aligned", who);
+    return ET_OK;
+}
+
+int et_pack_rows(void *packed, const void *padded, const int *cu_seqlens, int batch, int seq_len,
+                 int width, void *stream) {
+    using namespace et;
+    const int rc = pack_check(packed, padded, cu_seqlens, batch, seq_len, width, "et_pack_rows");
+    if (rc != ET_OK)
+        return rc;
+    hipLaunchKernelGGL(pack_rows_kernel, dim3(seq_len, batch), dim3(128), 0,
+                       static_cast<hipStream_t>(stream), static_cast<f16 *>(packed),
+                       static_cast<const f16 *>(padded), cu_seqlens, seq_len, width);
+    return launch_status("et_pack_rows");
+}
+
+int et_unpack_rows(void *padded, const void *packed, const int *cu_seqlens, int batch, int seq_len,
+                   int width, void *stream) {
+    using namespace et;
+    const int rc = pack_check(packed, padded, cu_seqlens, batch, seq_len, width, "et_unpack_rows");
+    if (rc != ET_OK)
+        return rc;
+    hipLaunchKernelGGL(unpack_rows_kernel, dim3(seq_len, batch), dim3(128), 0,
+                       static_cast<hipStream_t>(stream), static_cast<f16 *>(padded),
+                       static_cast<const f16 *>(packed), cu_seqlens, seq_len, width);
+    return launch_status("et_unpack_rows");
+}
+
+int et_scatter_cols(void *out, const void *in, const int *col_id, int rows, int n, int ld_in,
+                    int width, void *stream) {
+    using namespace et;
+    ET_REQUIRE(out && in && col_id, ET_ERR_INVALID_ARG, "et_scatter_cols: null pointer");
+    ET_REQUIRE(rows >= 0 && n >= 0 && n <= ld_in && n <= width && width > 0 && width <= 16384,
+               ET_ERR_INVALID_ARG, "et_scatter_cols: bad sizes");
+    if (rows == 0)
+        return ET_OK;
+    hipLaunchKernelGGL(scatter_cols_kernel, dim3(rows), dim3(256), width * sizeof(int),
+                       static_cast<hipStream_t>(stream), static_cast<f16 *>(out),
+                       static_cast<const f16 *>(in), col_id, n, ld_in, width);
+    return launch_status("et_scatter_cols");
+}
+
+} // extern "C"

@@ -1,0 +1,132 @@
+// Fused skip connection + LayerNorm for gfx950.
+//
+// Math of kernels/skip_layernorm.cu:4-43 (reference v1): x = half(a + skip),
+// fp32 mean and biased two-pass variance over the row, rstd =
+// rsqrt(var + 1e-6), y = (x-mean)*rstd*gamma + beta rounded to half, in place
+// on `a`.  Pure streaming op: 3 x size x 2 bytes per row, so the layout aims
+// at HBM bandwidth only — one wave64 per row, 16-byte loads per lane, the row
+// kept in registers between the passes, shuffle reductions, no LDS.
+#include "common.h"
+
+namespace et {
+
+// One wave per row; the row is held as NCH chunks of 8 halves per lane.
+template <int NCH>
+__global__ void __launch_bounds__(256)
+skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip,
+                          const f16 *__restrict__ gamma,
+                          const f16 *__restrict__ beta, int num, int size) {
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const long row = (long)blockIdx.x * 4 + wave;
+    if (row >= num)
+        return;
+    const int nchunk = size >> 3;
+    f16x8 *a = reinterpret_cast<f16x8 *>(in_out + row * size);
+    const f16x8 *s = reinterpret_cast<const f16x8 *>(skip + row * size);
+    const f16x8 *g = reinterpret_cast<const f16x8 *>(gamma);
+    const f16x8 *b = reinterpret_cast<const f16x8 *>(beta);
+
+    f16x8 x[NCH];
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = lane + i * 64;
+        if (c < nchunk) {
+            x[i] = a[c] + __builtin_nontemporal_load(&s[c]); // half add, one rounding
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                sum += (float)x[i][j];
+        }
+    }
+    const float mean = wave_sum(sum) / (float)size;
+    float var = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = lane + i * 64;
+        if (c < nchunk) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float d = (float)x[i][j] - mean;
+                var += d * d;
+            }
+        }
+    }
+    const float rstd = rsqrtf(wave_sum(var) / (float)size + 1e-6f);
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = lane + i * 64;
+        if (c < nchunk) {
+            const f16x8 gg = g[c], bb = b[c];
+            f16x8 y;
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                y[j] = (f16)(((float)x[i][j] - mean) * rstd * (float)gg[j] + (float)bb[j]);
+            a[c] = y;
+        }
+    }
+}
+
+// Any size, any alignment: one wave per row, three passes over memory.
+__global__ void __launch_bounds__(256)
+skip_layernorm_generic_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip,
+                              const f16 *__restrict__ gamma,
+                              const f16 *__restrict__ beta, int num, int size) {
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const long row = (long)blockIdx.x * 4 + wave;
+    if (row >= num)
+        return;
+    f16 *a = in_out + row * size;
+    const f16 *s = skip + row * size;
+    float sum = 0.f;
+    for (int c = lane; c < size; c += 64) {
+        const f16 x = a[c] + s[c];
+        a[c] = x; // same lane re-reads it below
+        sum += (float)x;
+    }
+    const float mean = wave_sum(sum) / (float)size;
+    float var = 0.f;
+    for (int c = lane; c < size; c += 64) {
+        const float d = (float)a[c] - mean;
+        var += d * d;
+    }
+    const float rstd = rsqrtf(wave_sum(var) / (float)size + 1e-6f);
+    for (int c = lane; c < size; c += 64)
+        a[c] = (f16)(((float)a[c] - mean) * rstd * (float)gamma[c] + (float)beta[c]);
+}
+
+} // namespace et
+
+extern "C" int et_skip_layernorm(void *in_out, const void *skip, const void *gamma,
+                                 const void *beta, int num, int size, void *stream) {
+    using namespace et;
+    ET_REQUIRE(in_out && skip && gamma && beta, ET_ERR_INVALID_ARG,
+               "et_skip_layernorm: null pointer");
+    ET_REQUIRE(num >= 0 && size > 0, ET_ERR_INVALID_ARG,
+               "et_skip_layernorm: num=%d size=%d", num, size);
+    if (num == 0)
+        return ET_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    f16 *a = static_cast<f16 *>(in_out);
+    const f16 *s = static_cast<const f16 *>(skip);
+    const f16 *g = static_cast<const f16 *>(gamma);
+    const f16 *b = static_cast<const f16 *>(beta);
+    const dim3 grid((num + 3) / 4), block(256);
+    const bool vec = (size % 8 == 0) && size <= 4096 && aligned16(in_out) &&
+                     aligned16(skip) && aligned16(gamma) && aligned16(beta);
+    if (!vec) {
+        hipLaunchKernelGGL(skip_layernorm_generic_kernel, grid, block, 0, st, a, s, g, b, num, size);
+    } else {
+        const int nch = (size / 8 + 63) / 64;
+        if (nch <= 1)
+            hipLaunchKernelGGL(skip_layernorm_vec_kernel<1>, grid, block, 0, st, a, s, g, b, num, size);
+        else if (nch <= 2)
+            hipLaunchKernelGGL(skip_layernorm_vec_kernel<2>, grid, block, 0, st, a, s, g, b, num, size);
+        else if (nch <= 4)
+            hipLaunchKernelGGL(skip_layernorm_vec_kernel<4>, grid, block, 0, st, a, s, g, b, num, size);
+        else
+            hipLaunchKernelGGL(skip_layernorm_vec_kernel<8>, grid, block, 0, st, a, s, g, b, num, size);
+    }
+    return launch_status("et_skip_layernorm launch");
+}

@@ -1,0 +1,198 @@
+"""Linear_tile / Linear_row / Encoder_* — the reference's encoder objects
+(encoder/Linear.h, encoder/encoder.h) over the C ABI in include/et_encoder.h.
+
+Constructor arguments keep the reference's order and meaning: weights, index
+arrays, LayerNorm parameters and the mask are HOST arrays (numpy) copied at
+construction; activations and the workspace are DEVICE tensors (torch).
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+import torch
+
+from ._lib import check, lib
+
+ENCODER_TILE, ENCODER_PRUNE, ENCODER_LENGTH = 0, 1, 2
+
+
+def _np(a, dt):
+    a = np.ascontiguousarray(a, dtype=dt)
+    return a
+
+
+def _hp(a):
+    return None if a is None else a.ctypes.data
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dp(t):
+    assert t.is_cuda and t.is_contiguous() and t.dtype == torch.float16
+    return t.data_ptr()
+
+
+class Linear_tile:
+    """encoder/Linear.h:4-46"""
+
+    def __init__(self, in_feat, out_feat, size, ntile, data, row_ptr, row_offset, bias, is_gelu=False):
+        self.in_feat, self.out_feat, self.size, self.is_gelu = in_feat, out_feat, size, bool(is_gelu)
+        data = _np(data, np.float16)
+        row_ptr, row_offset, bias = _np(row_ptr, np.int32), _np(row_offset, np.int32), _np(bias, np.float16)
+        assert data.size == ntile * 256 and row_offset.size == ntile and bias.size == out_feat
+        h = C.c_void_p()
+        check(lib().et_linear_tile_create(C.byref(h), in_feat, out_feat, size, ntile, _hp(data), _hp(row_ptr),
+                                          _hp(row_offset), _hp(bias), int(is_gelu)))
+        self._h = h
+
+    def run(self, x, out=None, rows=None):
+        rows = x.shape[0] if rows is None else rows
+        out = out if out is not None else torch.empty((x.shape[0], self.out_feat), dtype=torch.float16, device=x.device)
+        check(lib().et_linear_tile_run_rows(self._h, _dp(out), _dp(x), rows, _stream()))
+        return out
+
+    def _release(self):  # ownership moved into an encoder
+        self._h = None
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().et_linear_tile_destroy(self._h)
+            self._h = None
+
+
+def run_multi(linears, x, outs=None):
+    """several Linear_tile over the same input in one launch"""
+    n = len(linears)
+    outs = outs or [torch.empty((x.shape[0], l.out_feat), dtype=torch.float16, device=x.device) for l in linears]
+    hs = (C.c_void_p * n)(*[l._h for l in linears])
+    ys = (C.c_void_p * n)(*[_dp(o) for o in outs])
+    check(lib().et_linear_tile_run_multi(hs, ys, n, _dp(x), x.shape[0], _stream()))
+    return outs
+
+
+class Linear_row:
+    """encoder/Linear.h:48-72"""
+
+    def __init__(self, in_feat, out_feat, size, weight, row_id, nrow, bias, nhead):
+        weight, row_id, bias = _np(weight, np.float16), _np(row_id, np.int32), _np(bias, np.float16)
+        assert weight.size == nrow * in_feat and row_id.size == nrow and bias.size == nrow
+        self.in_feat, self.out_feat, self.size, self.nhead = in_feat, out_feat, size, nhead
+        h = C.c_void_p()
+        check(lib().et_linear_row_create(C.byref(h), in_feat, out_feat, size, _hp(weight), _hp(row_id), nrow,
+                                         _hp(bias), nhead))
+        self._h = h
+        a, b = C.c_int(), C.c_int()
+        check(lib().et_linear_row_query(h, C.byref(a), C.byref(b), None, None))
+        self.nrow, self.row_id_size = a.value, b.value
+
+    def run(self, x, out=None):
+        out = out if out is not None else torch.empty((x.shape[0], self.nrow), dtype=torch.float16, device=x.device)
+        assert x.shape[0] == self.size
+        check(lib().et_linear_row_run(self._h, _dp(out), _dp(x), _stream()))
+        return out
+
+    def _release(self):
+        self._h = None
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().et_linear_row_destroy(self._h)
+            self._h = None
+
+
+class _Encoder:
+    kind = None
+
+    def __init__(self, d_model, seq_len, nheads, buffer, Q_linear, K_linear, V_linear, O_linear, MLP1_linear,
+                 MLP2_linear, ln_gamma_1, ln_beta_1, ln_gamma_2, ln_beta_2, mask, batch=1):
+        self.d_model, self.seq_len, self.nheads, self.batch = d_model, seq_len, nheads, batch
+        need = self.buffer_size(d_model, seq_len, nheads, batch)
+        assert buffer.is_cuda and buffer.numel() * buffer.element_size() >= need, "workspace too small"
+        self.buffer = buffer
+        ln = [_np(t, np.float16) for t in (ln_gamma_1, ln_beta_1, ln_gamma_2, ln_beta_2)]
+        assert all(t.size == d_model for t in ln)
+        mask = None if mask is None else _np(mask, np.float16)
+        assert mask is None or mask.size == seq_len * seq_len
+        lin = [Q_linear, K_linear, V_linear, O_linear, MLP1_linear, MLP2_linear]
+        h = C.c_void_p()
+        check(lib().et_encoder_create(C.byref(h), self.kind, d_model, seq_len, nheads, batch, buffer.data_ptr(),
+                                      *[l._h for l in lin], *[_hp(t) for t in ln], _hp(mask)))
+        for l in lin:
+            l._release()
+        self._h = h
+
+    @classmethod
+    def buffer_size(cls, d_model, seq_len, nheads, batch=1):
+        return lib().et_encoder_buffer_size(cls.kind, d_model, seq_len, nheads, batch)
+
+    def run(self, out, inp):
+        """out, inp: [batch*seq_len, d_model] device tensors; out may be inp"""
+        check(lib().et_encoder_set_stream(self._h, _stream()))
+        check(lib().et_encoder_run(self._h, _dp(out), _dp(inp)))
+        return out
+
+    def set_log2_scale(self, v):
+        check(lib().et_encoder_set_log2_scale(self._h, float(v)))
+
+    def set_seq_lens(self, lens):
+        if lens is None:
+            check(lib().et_encoder_set_seq_lens(self._h, None))
+        else:
+            lens = _np(lens, np.int32)
+            assert lens.size == self.batch
+            check(lib().et_encoder_set_seq_lens(self._h, _hp(lens)))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().et_encoder_destroy(self._h)
+            self._h = None
+
+
+class Encoder_tile(_Encoder):
+    """encoder/encoder.h:56-77"""
+    kind = ENCODER_TILE
+
+
+class Encoder_prune(_Encoder):
+    """encoder/encoder.h:79-100; V_linear is a Linear_row"""
+    kind = ENCODER_PRUNE
+
+
+class Encoder_length(_Encoder):
+    """encoder/encoder.h:102-134"""
+    kind = ENCODER_LENGTH
+
+    def set_shared_qk(self, on):
+        check(lib().et_encoder_set_shared_qk(self._h, int(bool(on))))
+
+
+class Encoder_stack:
+    """N Encoder_length layers run on packed rows (variable-length batches)."""
+
+    def __init__(self, layers, d_model, seq_len, batch):
+        self.layers = list(layers)
+        n = len(self.layers)
+        hs = (C.c_void_p * n)(*[l._h for l in self.layers])
+        h = C.c_void_p()
+        check(lib().et_encoder_stack_create(C.byref(h), hs, n, d_model, seq_len, batch))
+        self._h = h
+        self.act = None
+        self.shape = (batch * seq_len, d_model)
+
+    def set_seq_lens(self, lens):
+        for l in self.layers:
+            l.set_seq_lens(lens)
+
+    def run(self, out, inp):
+        if self.act is None or self.act.device != inp.device:
+            self.act = torch.empty(self.shape, dtype=torch.float16, device=inp.device)
+        check(lib().et_encoder_stack_run(self._h, _dp(out), _dp(inp), _dp(self.act), _stream()))
+        return out
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().et_encoder_stack_destroy(self._h)
+            self._h = None

@@ -1,0 +1,103 @@
+// Pruned-weight linear operators.  Same names, constructor arguments and run()
+// meaning as encoder/Linear.h of the reference; the device work goes through
+// the C ABI (et_amd.h).
+#pragma once
+#include <utility>
+#include <vector>
+
+#include "utils.h"
+
+// Tensor-tile pruned linear: Y = X W^T + b with W as tile_mat
+// (encoder/Linear.h:4-46).  All constructor pointers are HOST memory.
+class Linear_tile {
+  private:
+    int in_feat;
+    int out_feat;
+    int size; // rows of X this operator is applied to (batch * seq_len)
+    et_tile_plan *plan;
+
+  public:
+    const bool is_gelu;
+    Linear_tile(int in_feat_, int out_feat_, int size_, int ntile, half *data_, int *row_ptr_,
+                int *row_offset_, half *bias_, bool is_gelu_ = false)
+        : in_feat(in_feat_), out_feat(out_feat_), size(size_), plan(nullptr), is_gelu(is_gelu_) {
+        etChk(et_tile_plan_create(&plan, in_feat_, out_feat_, ntile, data_, row_ptr_, row_offset_, bias_));
+    }
+    Linear_tile(const Linear_tile &) = delete;
+    Linear_tile &operator=(const Linear_tile &) = delete;
+    Linear_tile(Linear_tile &&other) noexcept
+        : in_feat(other.in_feat), out_feat(other.out_feat), size(other.size), plan(other.plan),
+          is_gelu(other.is_gelu) {
+        other.plan = nullptr;
+    }
+    ~Linear_tile() { et_tile_plan_destroy(plan); }
+
+    // encoder/Linear.h:36-45; `stream` is a hipStream_t (NULL = default stream)
+    void run(half *out, half *in, void *stream) const {
+        etChk(et_tile_plan_run(plan, out, in, size, is_gelu ? 1 : 0, stream));
+    }
+    // same operator on a different row count (variable-length batches)
+    void run_rows(half *out, half *in, int rows, void *stream) const {
+        etChk(et_tile_plan_run(plan, out, in, rows, is_gelu ? 1 : 0, stream));
+    }
+    // several linears over the same input in one launch (Q, K, V)
+    static void run_multi(const Linear_tile *const *lin, half *const *outs, int n, half *in, int rows,
+                          void *stream) {
+        const et_tile_plan *plans[4];
+        void *ys[4];
+        for (int i = 0; i < n && i < 4; i++) {
+            plans[i] = lin[i]->plan;
+            ys[i] = outs[i];
+        }
+        etChk(et_tile_plan_run_multi(plans, ys, n, in, rows, stream));
+    }
+    int rows() const { return size; }
+    int in_features() const { return in_feat; }
+    int out_features() const { return out_feat; }
+};
+
+// Row-pruned linear on compacted rows (encoder/Linear.h:48-72,
+// encoder/Linear.cu:60-91).  Output is compact: [size x nrow].
+class Linear_row {
+  public:
+    int in_feat;
+    int out_feat;
+    int size;
+    int nhead;
+    Weight<half> weight; // [nrow x in_feat], rows beyond row_id_size are zero
+    Weight<int> row_id;  // sorted outside
+    Weight<int> head_ptr;
+    int nrow;        // row_id_size rounded up to a multiple of 16
+    int row_id_size; // surviving rows
+    Weight<half> bias;
+
+    static int multiple_16(int x) { return ((x + 15) / 16) * 16; }
+
+    // weight_: HOST [row_id_size_ x in_feat_]; row_id_: HOST, ascending; bias_: HOST [row_id_size_]
+    Linear_row(int in_feat_, int out_feat_, int size_, half *weight_, int *row_id_, int row_id_size_,
+               half *bias_, int nhead_)
+        : in_feat(in_feat_), out_feat(out_feat_), size(size_), nhead(nhead_),
+          weight(in_feat_ * multiple_16(row_id_size_)), row_id(row_id_, row_id_size_ > 0 ? row_id_size_ : 1),
+          head_ptr(nhead_ + 1), nrow(multiple_16(row_id_size_)), row_id_size(row_id_size_),
+          bias(multiple_16(row_id_size_)) {
+        // padded rows must contribute nothing: zero the buffers first
+        etChk(et_fill_zero(weight.get(), sizeof(half) * (size_t)in_feat * nrow, nullptr));
+        etChk(et_fill_zero(bias.get(), sizeof(half) * (size_t)nrow, nullptr));
+        etChk(et_device_synchronize());
+        etChk(et_memcpy_h2d(weight.get(), weight_, sizeof(half) * (size_t)in_feat * row_id_size));
+        etChk(et_memcpy_h2d(bias.get(), bias_, sizeof(half) * (size_t)row_id_size));
+        std::vector<int> h_head_ptr(nhead + 1);
+        etChk(et_head_ptr(row_id_, row_id_size, nhead, out_feat / nhead, h_head_ptr.data()));
+        head_ptr.set(h_head_ptr.data());
+    }
+    Linear_row(Linear_row &&) noexcept = default;
+    Linear_row(const Linear_row &) = delete;
+
+    // encoder/Linear.h:68-71; the cuBLAS handle becomes a stream
+    void run(half *out, half *in, void *stream) const {
+        etChk(et_row_spmm_add_bias(out, in, weight.get(), bias.get(), size, nrow, in_feat, stream));
+    }
+    void run_rows(half *out, half *in, int rows, void *stream) const {
+        etChk(et_row_spmm_add_bias(out, in, weight.get(), bias.get(), rows, nrow, in_feat, stream));
+    }
+};

@@ -1,0 +1,275 @@
+// Encoder layer orchestration.  Same class names, constructor arguments and
+// run() meaning as encoder/encoder.h of the reference.  Differences, all
+// additive: an optional trailing `batch` (the reference binds one sequence per
+// encoder), a caller-settable stream, an exponent-base switch for the softmax,
+// optional per-sequence lengths.  One stream, no host synchronisation inside
+// run() (the reference blocks the host three times per layer,
+// encoder/encoder.cu:27-29), Q/K/V projected by one launch.
+#pragma once
+#include <vector>
+
+#include "Linear.h"
+#include "utils.h"
+
+class Encoder_base {
+  public:
+    static constexpr int buffer_num = 5; // encoder/encoder.h:9
+
+  protected:
+    int d_model;
+    int seq_len;
+    int nheads;
+    int batch;
+    half *buffer;              // caller-owned device workspace
+    half *buffers[buffer_num]; // units of batch*seq_len*d_model halves
+    Weight<half> ln_gamma[2];
+    Weight<half> ln_beta[2];
+    Weight<half> mask;  // [seq_len x seq_len] additive, shared by heads and batch
+    bool has_mask;
+    void *stream;       // hipStream_t; NULL = default stream
+    float log2_scale;   // 1 = base-2 softmax of the reference, log2(e) = textbook
+    // per-sequence lengths (optional)
+    std::vector<int> lens;
+    Weight<int> d_lens;
+    Weight<int> d_cu;
+    int total_rows; // sum of lengths when set, else batch*seq_len
+
+    int rows() const { return batch * seq_len; }
+
+  public:
+    // ln_* and mask_ are HOST pointers (d_model halves; seq_len*seq_len halves).
+    // mask_ == nullptr means no mask.
+    Encoder_base(int d_model_, int seq_len_, int nheads_, half *buffer_, half *ln_gamma_1,
+                 half *ln_beta_1, half *ln_gamma_2, half *ln_beta_2, half *mask_, int batch_ = 1)
+        : d_model(d_model_), seq_len(seq_len_), nheads(nheads_), batch(batch_), buffer(buffer_),
+          ln_gamma{Weight<half>(ln_gamma_1, d_model_), Weight<half>(ln_gamma_2, d_model_)},
+          ln_beta{Weight<half>(ln_beta_1, d_model_), Weight<half>(ln_beta_2, d_model_)},
+          has_mask(mask_ != nullptr), stream(nullptr), log2_scale(1.0f),
+          total_rows(batch_ * seq_len_) {
+        if (mask_)
+            mask = Weight<half>(mask_, seq_len_ * seq_len_);
+        for (int i = 0; i < buffer_num; i++)
+            buffers[i] = buffer + (size_t)i * batch * seq_len * d_model;
+    }
+    virtual ~Encoder_base() {}
+    virtual void run(half *out, half *in) = 0; // device pointers; out may alias in
+    static size_t buffer_size(int d_model_, int seq_len_, int /*nheads_*/, int batch_ = 1) {
+        return (size_t)buffer_num * d_model_ * seq_len_ * batch_ * sizeof(half);
+    }
+
+    void set_stream(void *s) { stream = s; }
+    void set_log2_scale(float v) { log2_scale = v; }
+    // HOST array of `batch` lengths in [0, seq_len]; nullptr clears them.
+    void set_seq_lens(const int *host_lens) {
+        lens.clear();
+        total_rows = batch * seq_len;
+        if (!host_lens)
+            return;
+        lens.assign(host_lens, host_lens + batch);
+        std::vector<int> cu(batch + 1, 0);
+        for (int b = 0; b < batch; b++)
+            cu[b + 1] = cu[b] + lens[b];
+        total_rows = cu[batch];
+        d_lens = Weight<int>(lens.data(), batch);
+        d_cu = Weight<int>(cu.data(), batch + 1);
+    }
+    int valid_rows() const { return total_rows; }
+    const int *device_cu_seqlens() const { return lens.empty() ? nullptr : d_cu.get(); }
+
+  protected:
+    half *mask_ptr() const { return has_mask ? mask.get() : nullptr; }
+    const int *lens_ptr() const { return lens.empty() ? nullptr : d_lens.get(); }
+
+    // steps 6-10 of encoder/encoder.cu:33-44, shared by every encoder kind:
+    // O projection, skip-LN with the layer input, FFN1+GELU, FFN2, skip-LN.
+    void tail(half *out, half *in, half *attn, const Linear_tile &O, const Linear_tile &M1,
+              const Linear_tile &M2, int nrows) {
+        O.run_rows(buffers[0], attn, nrows, stream);
+        etChk(et_skip_layernorm(buffers[0], in, ln_gamma[0].get(), ln_beta[0].get(), nrows, d_model, stream));
+        M1.run_rows(buffers[1], buffers[0], nrows, stream); // spans buffers[1..4]
+        M2.run_rows(out, buffers[1], nrows, stream);
+        etChk(et_skip_layernorm(out, buffers[0], ln_gamma[1].get(), ln_beta[1].get(), nrows, d_model, stream));
+    }
+};
+
+// On-the-fly attention + tensor-tile pruned linears (encoder/encoder.h:56-77,
+// encoder/encoder.cu:20-45).
+class Encoder_tile : public Encoder_base {
+  private:
+    Linear_tile Q_linear, K_linear, V_linear, O_linear, MLP1_linear, MLP2_linear;
+
+  public:
+    Encoder_tile(int d_model_, int seq_len_, int nheads_, half *buffer_, Linear_tile &&Q_linear_,
+                 Linear_tile &&K_linear_, Linear_tile &&V_linear_, Linear_tile &&O_linear_,
+                 Linear_tile &&MLP1_linear_, Linear_tile &&MLP2_linear_, half *ln_gamma_1,
+                 half *ln_beta_1, half *ln_gamma_2, half *ln_beta_2, half *mask_, int batch_ = 1)
+        : Encoder_base(d_model_, seq_len_, nheads_, buffer_, ln_gamma_1, ln_beta_1, ln_gamma_2,
+                       ln_beta_2, mask_, batch_),
+          Q_linear(std::move(Q_linear_)), K_linear(std::move(K_linear_)),
+          V_linear(std::move(V_linear_)), O_linear(std::move(O_linear_)),
+          MLP1_linear(std::move(MLP1_linear_)), MLP2_linear(std::move(MLP2_linear_)) {
+        // the reference asserts this (encoder/encoder.cu:17)
+        etRequire(MLP1_linear.is_gelu, "Encoder_tile: MLP1_linear must be the GELU variant");
+    }
+    void run(half *out, half *in) override {
+        const Linear_tile *qkv[3] = {&Q_linear, &K_linear, &V_linear};
+        half *outs[3] = {buffers[0], buffers[1], buffers[2]};
+        Linear_tile::run_multi(qkv, outs, 3, in, rows(), stream);
+        etChk(et_OTF_attention(buffers[3], buffers[0], buffers[1], buffers[2], mask_ptr(), seq_len,
+                               d_model, nheads, batch, lens_ptr(), log2_scale, stream));
+        tail(out, in, buffers[3], O_linear, MLP1_linear, MLP2_linear, rows());
+    }
+};
+
+// Attention-aware pruning: V projected by a row-pruned linear into a compact
+// [rows x nrow] matrix, attention over the surviving V columns
+// (encoder/encoder.h:79-100, encoder/encoder.cu:65-92).
+class Encoder_prune : public Encoder_base {
+  private:
+    Linear_tile Q_linear, K_linear;
+    Linear_row V_linear;
+    Linear_tile O_linear, MLP1_linear, MLP2_linear;
+
+  public:
+    Encoder_prune(int d_model_, int seq_len_, int nheads_, half *buffer_, Linear_tile &&Q_linear_,
+                  Linear_tile &&K_linear_, Linear_row &&V_linear_, Linear_tile &&O_linear_,
+                  Linear_tile &&MLP1_linear_, Linear_tile &&MLP2_linear_, half *ln_gamma_1,
+                  half *ln_beta_1, half *ln_gamma_2, half *ln_beta_2, half *mask_, int batch_ = 1)
+        : Encoder_base(d_model_, seq_len_, nheads_, buffer_, ln_gamma_1, ln_beta_1, ln_gamma_2,
+                       ln_beta_2, mask_, batch_),
+          Q_linear(std::move(Q_linear_)), K_linear(std::move(K_linear_)),
+          V_linear(std::move(V_linear_)), O_linear(std::move(O_linear_)),
+          MLP1_linear(std::move(MLP1_linear_)), MLP2_linear(std::move(MLP2_linear_)) {
+        etRequire(MLP1_linear.is_gelu, "Encoder_prune: MLP1_linear must be the GELU variant");
+    }
+    void run(half *out, half *in) override {
+        const Linear_tile *qk[2] = {&Q_linear, &K_linear};
+        half *outs[2] = {buffers[0], buffers[1]};
+        Linear_tile::run_multi(qk, outs, 2, in, rows(), stream);
+        V_linear.run_rows(buffers[2], in, rows(), stream);
+        // compact V has leading dimension nrow (what the GEMM wrote); the
+        // reference passes row_id_size here (encoder/encoder.cu:78) and reads
+        // the wrong rows whenever that is not a multiple of 16
+        etChk(et_Prune_attention(buffers[3], buffers[0], buffers[1], buffers[2], nullptr, 0,
+                                 V_linear.row_id.get(), V_linear.head_ptr.get(), V_linear.nrow,
+                                 mask_ptr(), seq_len, d_model, nheads, batch, lens_ptr(), log2_scale,
+                                 stream));
+        tail(out, in, buffers[3], O_linear, MLP1_linear, MLP2_linear, rows());
+    }
+};
+
+// Sequence-aware encoder (encoder/encoder.h:102-134, encoder/encoder.cu:116-149).
+// The reference's version writes scaled Q K^T for all heads to memory and runs
+// a second attention kernel on it; that path is kept behind use_shared_qk.
+// By default attention is the key-tiled on-the-fly kernel (no seq_len limit),
+// and when per-sequence lengths are set the layer runs on the PACKED valid
+// rows only: linears and LayerNorms see sum(len) rows, attention walks each
+// sequence's own rows, padding rows of `out` are written as zero.
+class Encoder_length : public Encoder_base {
+  private:
+    Linear_tile Q_linear, K_linear, V_linear, O_linear, MLP1_linear, MLP2_linear;
+    half *QK_buf;
+
+  public:
+    bool use_shared_qk;
+    Encoder_length(int d_model_, int seq_len_, int nheads_, half *buffer_, Linear_tile &&Q_linear_,
+                   Linear_tile &&K_linear_, Linear_tile &&V_linear_, Linear_tile &&O_linear_,
+                   Linear_tile &&MLP1_linear_, Linear_tile &&MLP2_linear_, half *ln_gamma_1,
+                   half *ln_beta_1, half *ln_gamma_2, half *ln_beta_2, half *mask_, int batch_ = 1)
+        : Encoder_base(d_model_, seq_len_, nheads_, buffer_, ln_gamma_1, ln_beta_1, ln_gamma_2,
+                       ln_beta_2, mask_, batch_),
+          Q_linear(std::move(Q_linear_)), K_linear(std::move(K_linear_)),
+          V_linear(std::move(V_linear_)), O_linear(std::move(O_linear_)),
+          MLP1_linear(std::move(MLP1_linear_)), MLP2_linear(std::move(MLP2_linear_)),
+          use_shared_qk(false) {
+        // after the five activation units (the reference offsets by
+        // d_model*nheads*buffer_num, which lands inside them)
+        QK_buf = buffer + (size_t)buffer_num * d_model * seq_len * batch;
+        etRequire(MLP1_linear.is_gelu, "Encoder_length: MLP1_linear must be the GELU variant");
+    }
+    static size_t buffer_size(int d_model_, int seq_len_, int nheads_, int batch_ = 1) {
+        return ((size_t)buffer_num * d_model_ * seq_len_ + (size_t)nheads_ * seq_len_ * seq_len_) *
+               batch_ * sizeof(half);
+    }
+
+    // One layer on packed rows: in_p/out_p are [valid_rows() x d_model] with
+    // sequence b at rows cu[b]..cu[b+1]-1; out_p may alias in_p.
+    void run_packed(half *out_p, half *in_p) {
+        const int n = total_rows;
+        const Linear_tile *qkv[3] = {&Q_linear, &K_linear, &V_linear};
+        half *outs[3] = {buffers[0], buffers[1], buffers[2]};
+        Linear_tile::run_multi(qkv, outs, 3, in_p, n, stream);
+        etChk(et_OTF_attention_varlen(buffers[3], buffers[0], buffers[1], buffers[2], mask_ptr(),
+                                      d_cu.get(), seq_len, d_model, nheads, batch, log2_scale, stream));
+        tail(out_p, in_p, buffers[3], O_linear, MLP1_linear, MLP2_linear, n);
+    }
+
+    void run(half *out, half *in) override {
+        if (!lens.empty()) {
+            // packed input parks in unit 4 (free until FFN1); FFN2 writes its
+            // packed result into the front of `out`, the second LayerNorm runs
+            // with the operands swapped (a+b == b+a) so its result lands in
+            // unit 0, from where it is expanded into `out`.
+            const int n = total_rows;
+            half *in_p = buffers[4];
+            etChk(et_pack_rows(in_p, in, d_cu.get(), batch, seq_len, d_model, stream));
+            const Linear_tile *qkv[3] = {&Q_linear, &K_linear, &V_linear};
+            half *outs[3] = {buffers[0], buffers[1], buffers[2]};
+            Linear_tile::run_multi(qkv, outs, 3, in_p, n, stream);
+            etChk(et_OTF_attention_varlen(buffers[3], buffers[0], buffers[1], buffers[2], mask_ptr(),
+                                          d_cu.get(), seq_len, d_model, nheads, batch, log2_scale, stream));
+            O_linear.run_rows(buffers[0], buffers[3], n, stream);
+            etChk(et_skip_layernorm(buffers[0], in_p, ln_gamma[0].get(), ln_beta[0].get(), n, d_model, stream));
+            MLP1_linear.run_rows(buffers[1], buffers[0], n, stream);
+            MLP2_linear.run_rows(out, buffers[1], n, stream);
+            etChk(et_skip_layernorm(buffers[0], out, ln_gamma[1].get(), ln_beta[1].get(), n, d_model, stream));
+            etChk(et_unpack_rows(out, buffers[0], d_cu.get(), batch, seq_len, d_model, stream));
+            return;
+        }
+        const Linear_tile *qkv[3] = {&Q_linear, &K_linear, &V_linear};
+        half *outs[3] = {buffers[0], buffers[1], buffers[2]};
+        Linear_tile::run_multi(qkv, outs, 3, in, rows(), stream);
+        if (use_shared_qk) {
+            etChk(et_qk_scores(QK_buf, buffers[0], buffers[1], seq_len, d_model, nheads, batch, stream));
+            etChk(et_sharedQK_attention(buffers[3], QK_buf, buffers[2], mask_ptr(), seq_len, d_model,
+                                        nheads, batch, nullptr, log2_scale, stream));
+        } else {
+            etChk(et_OTF_attention(buffers[3], buffers[0], buffers[1], buffers[2], mask_ptr(), seq_len,
+                                   d_model, nheads, batch, nullptr, log2_scale, stream));
+        }
+        tail(out, in, buffers[3], O_linear, MLP1_linear, MLP2_linear, rows());
+    }
+};
+
+// N Encoder_length layers over one workspace for variable-length batches: the
+// batch is packed once, every layer runs in place on the packed rows, the
+// result is expanded once.  No reference counterpart (it has no batch).
+class Encoder_stack {
+    std::vector<Encoder_length *> layers;
+    int d_model, seq_len, batch;
+
+  public:
+    Encoder_stack(std::vector<Encoder_length *> layers_, int d_model_, int seq_len_, int batch_)
+        : layers(std::move(layers_)), d_model(d_model_), seq_len(seq_len_), batch(batch_) {}
+    // act: device scratch of batch*seq_len*d_model halves (packed activations)
+    void run(half *out, half *in, half *act, void *stream) {
+        if (layers.empty())
+            return;
+        for (Encoder_length *l : layers)
+            l->set_stream(stream);
+        const int *cu = layers[0]->device_cu_seqlens();
+        if (!cu) { // full-length batch: layers chain through `act`
+            half *cur = in;
+            for (size_t i = 0; i < layers.size(); i++) {
+                half *dst = (i + 1 == layers.size()) ? out : act;
+                layers[i]->run(dst, cur);
+                cur = dst;
+            }
+            return;
+        }
+        etChk(et_pack_rows(act, in, cu, batch, seq_len, d_model, stream));
+        for (Encoder_length *l : layers)
+            l->run_packed(act, act);
+        etChk(et_unpack_rows(out, act, cu, batch, seq_len, d_model, stream));
+    }
+};

@@ -1,0 +1,127 @@
+"""The launchers of the reference's kernels/kernels.h over torch device tensors.
+
+Each function forwards raw device pointers to the C ABI (include/et_amd.h) on
+torch's current stream.  Names follow the reference launchers.
+"""
+from __future__ import annotations
+
+import torch
+
+from ._lib import check, lib
+
+LOG2E = 1.4426950408889634
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "device, contiguous tensors only"
+    return t.data_ptr()
+
+
+def _h(t):
+    assert t is None or t.dtype == torch.float16
+    return _p(t)
+
+
+def _i32(t):
+    assert t is None or t.dtype == torch.int32
+    return _p(t)
+
+
+def skip_layernorm(in_out, skip, gamma, beta):
+    """in place on in_out[num x size]; kernels/kernels.h:3-5"""
+    num, size = in_out.shape
+    check(lib().et_skip_layernorm(_h(in_out), _h(skip), _h(gamma), _h(beta), num, size, _stream()))
+    return in_out
+
+
+def tile_spmm_add_bias(X, row_ptr, row_offset, data, bias, N, gelu=False, out=None):
+    """Y = X W^T + bias with W as tile_mat; kernels/kernels.h:13-20"""
+    M, K = X.shape
+    Y = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=X.device)
+    fn = lib().et_tile_spmm_add_bias_gelu if gelu else lib().et_tile_spmm_add_bias
+    check(fn(_h(Y), _h(X), _i32(row_ptr), _i32(row_offset), _h(data), M, N, K, _h(bias), _stream()))
+    return Y
+
+
+def row_spmm_add_bias(X, weight, bias, out=None):
+    """out = X weight^T + bias, weight[N x K] row-major; kernels/kernels.h:7-11"""
+    M, K = X.shape
+    N = weight.shape[0]
+    Y = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=X.device)
+    check(lib().et_row_spmm_add_bias(_h(Y), _h(X), _h(weight), _h(bias), M, N, K, _stream()))
+    return Y
+
+
+def OTF_attention(Q, K, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2_scale=1.0, out=None):
+    """kernels/kernels.h:22-24 (+ batch, seq_lens, exponent base)"""
+    d_model = Q.shape[1]
+    Z = out if out is not None else torch.empty_like(Q)
+    check(lib().et_OTF_attention(_h(Z), _h(Q), _h(K), _h(V), _h(mask), seq_len, d_model, nhead, batch,
+                                 _i32(seq_lens), log2_scale, _stream()))
+    return Z
+
+
+def OTF_attention_varlen(Q, K, V, mask, cu_seqlens, max_seq_len, nhead, log2_scale=1.0, out=None):
+    d_model = Q.shape[1]
+    batch = cu_seqlens.numel() - 1
+    Z = out if out is not None else torch.empty_like(Q)
+    check(lib().et_OTF_attention_varlen(_h(Z), _h(Q), _h(K), _h(V), _h(mask), _i32(cu_seqlens), max_seq_len,
+                                        d_model, nhead, batch, log2_scale, _stream()))
+    return Z
+
+
+def Prune_attention(Q, K, V, qk_head_ptr, v_col_id, v_head_ptr, mask, seq_len, d_model, nhead, batch=1,
+                    seq_lens=None, log2_scale=1.0, out=None):
+    """kernels/kernels.h:26-30 (+ compact Q/K, batch, seq_lens, exponent base)"""
+    rows = Q.shape[0]
+    Z = out if out is not None else torch.empty((rows, d_model), dtype=torch.float16, device=Q.device)
+    check(lib().et_Prune_attention(_h(Z), _h(Q), _h(K), _h(V), _i32(qk_head_ptr), Q.shape[1], _i32(v_col_id),
+                                   _i32(v_head_ptr), V.shape[1], _h(mask), seq_len, d_model, nhead, batch,
+                                   _i32(seq_lens), log2_scale, _stream()))
+    return Z
+
+
+def qk_scores(Q, K, seq_len, nhead, batch=1):
+    """scaled Q K^T per head into [(b*nhead+h), S, S]; encoder/encoder.cu:126-130"""
+    d_model = Q.shape[1]
+    QK = torch.empty((batch * nhead, seq_len, seq_len), dtype=torch.float16, device=Q.device)
+    check(lib().et_qk_scores(_h(QK), _h(Q), _h(K), seq_len, d_model, nhead, batch, _stream()))
+    return QK
+
+
+def sharedQK_attention(QK, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2_scale=1.0, out=None):
+    """kernels/kernels.h:32-34"""
+    d_model = V.shape[1]
+    Z = out if out is not None else torch.empty_like(V)
+    check(lib().et_sharedQK_attention(_h(Z), _h(QK), _h(V), _h(mask), seq_len, d_model, nhead, batch,
+                                      _i32(seq_lens), log2_scale, _stream()))
+    return Z
+
+
+def pack_rows(padded, cu_seqlens, seq_len, total_rows):
+    width = padded.shape[1]
+    batch = cu_seqlens.numel() - 1
+    packed = torch.empty((total_rows, width), dtype=torch.float16, device=padded.device)
+    check(lib().et_pack_rows(_h(packed), _h(padded), _i32(cu_seqlens), batch, seq_len, width, _stream()))
+    return packed
+
+
+def unpack_rows(packed, cu_seqlens, seq_len):
+    width = packed.shape[1]
+    batch = cu_seqlens.numel() - 1
+    padded = torch.empty((batch * seq_len, width), dtype=torch.float16, device=packed.device)
+    check(lib().et_unpack_rows(_h(padded), _h(packed), _i32(cu_seqlens), batch, seq_len, width, _stream()))
+    return padded
+
+
+def scatter_cols(x, col_id, width):
+    rows, ld = x.shape
+    out = torch.empty((rows, width), dtype=torch.float16, device=x.device)
+    check(lib().et_scatter_cols(_h(out), _h(x), _i32(col_id), rows, col_id.numel(), ld, width, _stream()))
+    return out

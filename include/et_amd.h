@@ -1,0 +1,224 @@
+/*
+ * et_amd.h — C ABI of the MI355X (gfx950) implementation of the E.T. encoder
+ * hot path.  Plain pointers and sizes only; every entry point returns 0 on
+ * success or a negative ET_ERR_* code (never exits, never throws).  All
+ * activation / weight pointers are DEVICE pointers to IEEE binary16 unless a
+ * parameter is documented as host memory.  `stream` is a hipStream_t passed
+ * as void* (NULL = the default stream); launches are asynchronous on it.
+ *
+ * Each launcher names the reference interface it replaces
+ * (paths relative to the reference tree).
+ */
+#ifndef ET_AMD_H
+#define ET_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ET_OK 0
+#define ET_ERR_INVALID_ARG (-1) /* null pointer, non-positive or inconsistent size */
+#define ET_ERR_ALIGNMENT (-2)   /* pointer or leading dimension not 16-byte aligned */
+#define ET_ERR_UNSUPPORTED (-3) /* shape outside what the kernels cover */
+#define ET_ERR_HIP (-4)         /* a HIP runtime call failed; see et_last_error() */
+#define ET_ERR_FORMAT (-5)      /* malformed tile_mat / row_mat index arrays */
+
+/* Human-readable text for a code; message of the last failure on this thread. */
+const char *et_strerror(int code);
+const char *et_last_error(void);
+/* Version of this ABI (bumped on incompatible change). */
+int et_abi_version(void);
+
+/* ------------------------------------------------------------------------
+ * L0 launchers — one per prototype of kernels/kernels.h:3-34.
+ * ---------------------------------------------------------------------- */
+
+/* Replaces skip_layernorm_kernelLauncher (kernels/kernels.h:3-5,
+ * kernels/skip_layernorm.cu:101-112).  in_out[num x size] =
+ * LayerNorm(in_out + skip) * gamma + beta, eps 1e-6, biased variance, fp32
+ * statistics.  size must be even. */
+int et_skip_layernorm(void *in_out, const void *skip, const void *gamma,
+                      const void *beta, int num, int size, void *stream);
+
+/* Replaces tile_spmm_add_bias_kernelLauncher (kernels/kernels.h:13-15,
+ * kernels/linear.cu:152-158).  Y[M x N] = X[M x K] * W^T + bias with W[N x K]
+ * held as tile_mat: W_row_ptr[N/16+1], W_row_offset[ntile] (element column
+ * offsets, multiples of 16, any order inside a block-row),
+ * W_data[ntile*256] with W_data[i*256+n*16+k] = W[bn*16+n][W_row_offset[i]+k].
+ * K (= in_feat, the leading dimension of X) is an added argument: the
+ * reference launcher omits it and uses M in its place.  M is any positive
+ * row count; N and K are multiples of 16. */
+int et_tile_spmm_add_bias(void *Y, const void *X, const int *W_row_ptr,
+                          const int *W_row_offset, const void *W_data, int M,
+                          int N, int K, const void *bias, void *stream);
+
+/* Replaces tile_spmm_add_bias_gelu_kernelLauncher (kernels/kernels.h:17-20,
+ * kernels/linear.cu:160-167): as above followed by the tanh-form GELU of
+ * kernels/linear.cu:36-48 on the half-rounded sum. */
+int et_tile_spmm_add_bias_gelu(void *Y, const void *X, const int *W_row_ptr,
+                               const int *W_row_offset, const void *W_data,
+                               int M, int N, int K, const void *bias,
+                               void *stream);
+
+/* Replaces row_spmm_add_bias_kernelLauncher (kernels/kernels.h:7-11,
+ * kernels/linear.cu:18-34): out[M x N] = in[M x K] * weight^T + bias with
+ * weight[N x K] row-major (the compacted surviving rows, N padded to a
+ * multiple of 16).  The cuBLAS handle/algo pair becomes a stream. */
+int et_row_spmm_add_bias(void *out, const void *in, const void *weight,
+                         const void *bias, int M, int N, int K, void *stream);
+
+/* Replaces OTF_attention_kernelLauncher (kernels/kernels.h:22-24,
+ * kernels/attention.cu:122-134).  out, Q, K, V are [batch*seq_len x d_model];
+ * head h owns columns h*hd..(h+1)*hd-1, hd = d_model/nhead in {32,64,128}.
+ * Z = softmax((Q*scale) K^T + mask) V per head without writing the score
+ * matrix to memory; scale = half(sqrt(1/hd)) applied to Q in half; mask is
+ * one additive [seq_len x seq_len] half matrix shared by heads and batch, or
+ * NULL.  p = 2^(log2_scale*(s-max)): log2_scale 1.0f is the reference's
+ * base-2 softmax (kernels/attention.cu:33), 1.44269504f (log2 e) the textbook
+ * one.  Added: batch (>=1) and seq_lens (NULL, or batch ints in
+ * [0,seq_len]: keys at or beyond seq_lens[b] are ignored and query rows at or
+ * beyond it are written as zero). */
+int et_OTF_attention(void *out, const void *Q, const void *K, const void *V,
+                     const void *mask, int seq_len, int d_model, int nhead,
+                     int batch, const int *seq_lens, float log2_scale,
+                     void *stream);
+
+/* Variable-length (packed) form of et_OTF_attention for the
+ * sequence-length-aware path: rows of sequence b are
+ * cu_seqlens[b]..cu_seqlens[b+1]-1 of out/Q/K/V (no padding rows exist);
+ * mask, if given, is [max_seq_len x max_seq_len].  No reference counterpart
+ * (the reference has no batch dimension). */
+int et_OTF_attention_varlen(void *out, const void *Q, const void *K,
+                            const void *V, const void *mask,
+                            const int *cu_seqlens, int max_seq_len,
+                            int d_model, int nhead, int batch,
+                            float log2_scale, void *stream);
+
+/* Replaces Prune_attention_kernelLauncher (kernels/kernels.h:26-30,
+ * kernels/attention.cu:252-271).  V is compact [rows x ldv]; head h owns
+ * compact columns v_head_ptr[h]..v_head_ptr[h+1]-1 whose results are written
+ * to out[:, v_col_id[j]] (v_col_id sorted, inside the head's slice); every
+ * other column of out is written as zero.  The reference's nnz_col_v is ldv.
+ * Added: qk_head_ptr/ldqk — when non-NULL, Q and K are compact [rows x ldqk]
+ * and head h contracts over columns qk_head_ptr[h]..qk_head_ptr[h+1]-1 (at
+ * most hd of them); NULL keeps the reference's dense Q/K. batch, seq_lens,
+ * log2_scale as for et_OTF_attention. */
+int et_Prune_attention(void *out, const void *Q, const void *K, const void *V,
+                       const int *qk_head_ptr, int ldqk, const int *v_col_id,
+                       const int *v_head_ptr, int ldv, const void *mask,
+                       int seq_len, int d_model, int nhead, int batch,
+                       const int *seq_lens, float log2_scale, void *stream);
+
+/* Replaces sharedQK_attention_kernelLauncher (kernels/kernels.h:32-34,
+ * kernels/attention.cu:342-350): scores are read from
+ * QK[(b*nhead+h)][seq_len][seq_len] (halves, already scaled). */
+int et_sharedQK_attention(void *out, const void *QK, const void *V,
+                          const void *mask, int seq_len, int d_model,
+                          int nhead, int batch, const int *seq_lens,
+                          float log2_scale, void *stream);
+
+/* Replaces the cublasHgemmStridedBatched call of Encoder_length::run
+ * (encoder/encoder.cu:126-130): QK[(b*nhead+h)][q][k] =
+ * half(scale * sum_d Q[q][h*hd+d] K[k][h*hd+d]) from row-major
+ * [batch*seq_len x d_model] Q and K. */
+int et_qk_scores(void *QK, const void *Q, const void *K, int seq_len,
+                 int d_model, int nhead, int batch, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Planned tile linear — what Linear_tile (encoder/Linear.h:4-46) owns.
+ * The plan keeps device copies of the weight in a kernel-friendly order
+ * (tiles of a block-row sorted by column so K can be walked in LDS-sized
+ * chunks); results equal et_tile_spmm_add_bias on the same tile_mat up to
+ * fp32 summation order.
+ * ---------------------------------------------------------------------- */
+typedef struct et_tile_plan et_tile_plan;
+
+/* All pointers are HOST memory, as in the Linear_tile constructor
+ * (encoder/Linear.h:18-24). */
+int et_tile_plan_create(et_tile_plan **plan, int in_feat, int out_feat,
+                        int ntile, const void *data, const int *row_ptr,
+                        const int *row_offset, const void *bias);
+void et_tile_plan_destroy(et_tile_plan *plan);
+/* Linear_tile::run (encoder/Linear.h:36-45); gelu selects the GELU variant. */
+int et_tile_plan_run(const et_tile_plan *plan, void *Y, const void *X, int M,
+                     int gelu, void *stream);
+/* n (<= 4) planned linears with the same in_feat applied to the same X in ONE
+ * launch (the Q/K/V projections, encoder/encoder.cu:22-26, which the
+ * reference spreads over three streams). */
+int et_tile_plan_run_multi(const et_tile_plan *const *plans, void *const *Ys,
+                           int n, const void *X, int M, void *stream);
+/* device pointers of the plan's buffers, for tests (sorted order) */
+int et_tile_plan_query(const et_tile_plan *plan, int *in_feat, int *out_feat,
+                       int *ntile, int *nchunk, int *chunk_cols);
+
+/* ------------------------------------------------------------------------
+ * Pruned-weight formats (host side; all pointers HOST memory).
+ * ---------------------------------------------------------------------- */
+
+/* Seeded form of gen_sparse_tile_mat (test/tile_mat.cu:5-34): ntile =
+ * int(total*(1.0-sparsity)) tiles chosen by a splitmix64-driven Fisher-Yates
+ * shuffle of the row-major tile grid; block-rows list their tiles in shuffle
+ * order; row_offset = tile column * 16.  row_ptr: nrow/16+1 ints; row_offset:
+ * capacity (nrow/16)*(ncol/16) ints.  Returns ntile (>= 0) or an error. */
+int et_gen_sparse_tile_mat(int nrow, int ncol, float sparsity, uint64_t seed,
+                           int *row_ptr, int *row_offset);
+/* Seeded form of gen_sparse_row_mat (test/row_mat.cu:5-14): returns nn_row and
+ * fills row_id (capacity nrow) with the sorted surviving row ids. */
+int et_gen_sparse_row_mat(int nrow, float sparsity, uint64_t seed,
+                          int *row_id);
+/* keep `keep` of every head's head_dim rows (seeded, sorted); row_id capacity
+ * nhead*keep.  Balanced variant used for per-head Q/K pruning. */
+int et_gen_head_balanced_rows(int nhead, int head_dim, int keep, uint64_t seed,
+                              int *row_id);
+/* 0 if (row_ptr,row_offset) is a well-formed tile_mat of W[N x K]
+ * (the asserts of test/tile_mat.cu:31-33 plus range/alignment/duplicates). */
+int et_tile_mat_validate(int N, int K, int ntile, const int *row_ptr,
+                         const int *row_offset);
+/* data[i*256+n*16+k] = W[bn*16+n][row_offset[i]+k] from dense row-major W. */
+int et_tile_pack(const void *W, int N, int K, const int *row_ptr,
+                 const int *row_offset, void *data);
+/* CSR of a sorted row_id over heads: head_ptr[h] = #ids < h*head_dim,
+ * head_ptr[nhead] = n (intent of encoder/Linear.cu:74-88). */
+int et_head_ptr(const int *row_id, int n, int nhead, int head_dim,
+                int *head_ptr);
+
+/* ------------------------------------------------------------------------
+ * Sequence-length-aware path helpers (no reference counterpart).
+ * ---------------------------------------------------------------------- */
+/* packed[cu_seqlens[b]+t][:] = padded[b*seq_len+t][:] for t < len_b */
+int et_pack_rows(void *packed, const void *padded, const int *cu_seqlens,
+                 int batch, int seq_len, int width, void *stream);
+/* inverse; padding rows of `padded` are written as zero */
+int et_unpack_rows(void *padded, const void *packed, const int *cu_seqlens,
+                   int batch, int seq_len, int width, void *stream);
+/* out[r][col_id[j]] = in[r][j] for j < n, every other column of out[rows x
+ * width] zero: expands a row_mat linear's compact output
+ * (kernels/linear.cu:30-32) back to model width. */
+int et_scatter_cols(void *out, const void *in, const int *col_id, int rows,
+                    int n, int ld_in, int width, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Device memory / stream plumbing so that host code above this ABI needs no
+ * HIP headers (Weight<T>, encoder/utils.h:14-43; streams,
+ * encoder/encoder.h:36-39).
+ * ---------------------------------------------------------------------- */
+int et_malloc(void **ptr, size_t bytes);
+int et_free(void *ptr);
+int et_memcpy_h2d(void *dst, const void *src, size_t bytes);
+int et_memcpy_d2h(void *dst, const void *src, size_t bytes);
+int et_memcpy_d2d_async(void *dst, const void *src, size_t bytes, void *stream);
+int et_fill_zero(void *dst, size_t bytes, void *stream);
+int et_stream_create(void **stream);
+int et_stream_destroy(void *stream);
+int et_stream_synchronize(void *stream);
+int et_device_synchronize(void);
+/* number of compute units of the current device (0 if none) */
+int et_device_cu_count(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ET_AMD_H */

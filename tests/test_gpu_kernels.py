@@ -1,0 +1,282 @@
+"""Parity of the HIP kernels (through the C ABI) against the CPU oracle.
+
+Integer/index data must match bit for bit; fp16 activations within
+max-abs 2e-2 / mean-rel 1e-3 (helpers.MAX_ABS / MEAN_REL), usually far tighter.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle.et_oracle as orc
+from helpers import rng, randn_h, make_tile_linear, check_close
+
+pytestmark = pytest.mark.gpu
+
+LOG2E = math.log2(math.e)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+@pytest.fixture(scope="module")
+def K():
+    from et_amd import kernels
+    return kernels
+
+
+# ------------------------------------------------------------------ skip-LN
+@pytest.mark.parametrize("rows,size", [(128, 768), (1000, 768), (33, 1024), (5, 2048), (7, 4096), (9, 64), (6, 100), (3, 8200)])
+def test_skip_layernorm(K, rows, size):
+    r = rng(100 + rows)
+    a, s = randn_h(r, (rows, size)), randn_h(r, (rows, size))
+    g, b = randn_h(r, (size,), 0.3) + np.float16(1), randn_h(r, (size,), 0.3)
+    want = orc.skip_layernorm(a, s, g, b)
+    got = host(K.skip_layernorm(dev(a), dev(s), dev(g), dev(b)))
+    check_close(got, want, max_abs=4e-3, mean_rel=2e-4, what=f"skip_ln {rows}x{size}")
+    assert (got != want).mean() < 0.02   # fp32 reduction order only
+
+
+def test_skip_layernorm_constant_row_and_unit_stats(K):
+    d = 768
+    g, b = np.ones(d, np.float16), np.zeros(d, np.float16)
+    r = rng(7)
+    beta = randn_h(r, (d,))
+    const = np.full((4, d), 0.75, np.float16)
+    assert np.array_equal(host(K.skip_layernorm(dev(const), dev(const), dev(g), dev(beta))), np.repeat(beta[None], 4, 0))
+    a, s = randn_h(r, (64, d)), randn_h(r, (64, d))
+    y = host(K.skip_layernorm(dev(a), dev(s), dev(g), dev(b))).astype(np.float64)
+    assert np.abs(y.mean(1)).max() < 2e-3 and np.abs(y.var(1) - 1).max() < 5e-3
+
+
+# --------------------------------------------------------------- tile linear
+TILE_CASES = [
+    # M, N, K, sparsity, gelu
+    (128, 768, 768, 0.0, False),      # dense BERT projection (config 1 shape)
+    (100, 768, 768, 0.8, False),      # M not a multiple of the row panel
+    (64, 3072, 768, 0.5, True),       # FFN1 with GELU
+    (64, 768, 3072, 0.8, False),      # FFN2: K walked in chunks
+    (16, 16, 16, 0.0, False),         # one tile
+    (48, 64, 96, 0.95, False),        # mostly empty block-rows
+    (32, 32, 32, 1.0, True),          # no tile at all: Y = gelu(bias)
+    (1, 128, 1024, 0.3, False),       # single row, odd tile counts
+    (257, 1040, 1008, 0.6, True),     # ragged everything, largest single-panel K
+    (40, 48, 1024, 0.5, False),       # smallest K that needs two chunks
+]
+
+
+@pytest.mark.parametrize("M,N,Kd,sp,gelu", TILE_CASES)
+def test_tile_linear_raw_and_planned(K, M, N, Kd, sp, gelu):
+    from et_amd.encoder import Linear_tile
+    r = rng(200 + M + N)
+    lin = make_tile_linear(r, N, Kd, sp, seed=M + N + Kd, std=0.05, bias_std=0.2)
+    X = randn_h(r, (M, Kd))
+    want = orc.tile_linear(X, lin["row_ptr"], lin["row_offset"], lin["data"], lin["bias"], N, gelu=gelu)
+    want64 = orc.tile_linear(X, lin["row_ptr"], lin["row_offset"], lin["data"], lin["bias"], N, gelu=gelu, f64=True)
+    Xd = dev(X)
+    got = host(K.tile_spmm_add_bias(Xd, dev(lin["row_ptr"]), dev(lin["row_offset"]) if lin["row_offset"].size else None,
+                                    dev(lin["data"]) if lin["data"].size else None, dev(lin["bias"]), N, gelu=gelu))
+    tol = max(np.abs(want64.astype(np.float64)).max() * 2.0 ** -10, 1e-3)
+    check_close(got, want64, max_abs=tol, mean_rel=5e-4, what="tile raw vs f64")
+    check_close(got, want, max_abs=tol, mean_rel=5e-4, what="tile raw vs f32")
+    lt = Linear_tile(Kd, N, M, lin["row_offset"].size, lin["data"], lin["row_ptr"], lin["row_offset"], lin["bias"], gelu)
+    got2 = host(lt.run(Xd))
+    check_close(got2, want64, max_abs=tol, mean_rel=5e-4, what="tile planned vs f64")
+
+
+def test_tile_linear_closed_form_reference_smoke_inputs(K):
+    """weights = bias = 0.1 (test/gen_linear.cu:8,10): Y = 0.1*sum_{kept k} X + 0.1"""
+    r = rng(12)
+    M, N, Kd = 64, 768, 768
+    rp, ro = orc.gen_sparse_tile_mat(N, Kd, 0.8, seed=2)
+    data = np.full(ro.size * 256, 0.1, np.float16)
+    bias = np.full(N, 0.1, np.float16)
+    X = randn_h(r, (M, Kd))
+    got = host(K.tile_spmm_add_bias(dev(X), dev(rp), dev(ro), dev(data), dev(bias), N)).astype(np.float64)
+    c = float(np.float16(0.1))
+    for bn in range(N // 16):
+        cols = np.concatenate([np.arange(o, o + 16) for o in ro[rp[bn]:rp[bn + 1]]]) if rp[bn + 1] > rp[bn] else np.array([], int)
+        want = c * X[:, cols].astype(np.float64).sum(1) + c
+        assert np.abs(got[:, bn * 16:(bn + 1) * 16] - want[:, None]).max() <= np.abs(want).max() * 2.0 ** -10 + 1e-3
+
+
+def test_tile_linear_multi_qkv_one_launch(K):
+    from et_amd.encoder import Linear_tile, run_multi
+    r = rng(31)
+    M, d = 200, 768
+    lins = [make_tile_linear(r, d, d, 0.8, seed=50 + j, std=0.05, bias_std=0.1) for j in range(3)]
+    X = randn_h(r, (M, d))
+    lts = [Linear_tile(d, d, M, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"]) for l in lins]
+    outs = run_multi(lts, dev(X))
+    for l, o in zip(lins, outs):
+        want = orc.tile_linear(X, l["row_ptr"], l["row_offset"], l["data"], l["bias"], d, f64=True)
+        check_close(host(o), want, max_abs=2e-3, mean_rel=5e-4, what="qkv multi")
+
+
+def test_tile_linear_full_size_config2_rows_sample(K):
+    """config-2 shape (4096x768 -> 3072, 80 %): rows are independent, so a row sample pins the full-size launch"""
+    r = rng(32)
+    M, N, Kd = 4096, 3072, 768
+    lin = make_tile_linear(r, N, Kd, 0.8, seed=2024, std=0.02)
+    assert lin["row_offset"].size == 1843
+    X = randn_h(r, (M, Kd))
+    got = host(K.tile_spmm_add_bias(dev(X), dev(lin["row_ptr"]), dev(lin["row_offset"]), dev(lin["data"]), dev(lin["bias"]), N))
+    rows = np.sort(r.choice(M, 192, replace=False))
+    rows[:3] = [0, 31, 4095]
+    want = orc.tile_linear(X[rows], lin["row_ptr"], lin["row_offset"], lin["data"], lin["bias"], N, f64=True)
+    check_close(got[rows], want, max_abs=2e-3, mean_rel=5e-4, what="config-2 sample")
+    # linearity in X where it is exact in fp16: doubling X doubles Y (bias is 0),
+    # except for results in the subnormal range, whose grid does not scale
+    got2 = host(K.tile_spmm_add_bias(dev(X * np.float16(2)), dev(lin["row_ptr"]), dev(lin["row_offset"]), dev(lin["data"]), dev(lin["bias"]), N))
+    normal = np.abs(got) >= 2.0 ** -13
+    assert np.array_equal(got2[normal], (got * np.float16(2))[normal])
+    assert np.abs(got2.astype(np.float64) - 2 * got.astype(np.float64))[~normal].max() <= 2.0 ** -23
+
+
+def test_tile_linear_argument_errors(K):
+    from et_amd import EtError
+    r = rng(33)
+    lin = make_tile_linear(r, 32, 32, 0.0, seed=1)
+    X = dev(randn_h(r, (16, 32)))
+    with pytest.raises(EtError):   # N not a multiple of 16
+        K.tile_spmm_add_bias(X, dev(lin["row_ptr"]), dev(lin["row_offset"]), dev(lin["data"]), dev(lin["bias"]), 24)
+    with pytest.raises(EtError):   # misaligned X
+        K.tile_spmm_add_bias(dev(randn_h(r, (17, 32))).view(-1)[1:1 + 16 * 32].view(16, 32), dev(lin["row_ptr"]),
+                             dev(lin["row_offset"]), dev(lin["data"]), dev(lin["bias"]), 32)
+
+
+# ---------------------------------------------------------------- row linear
+@pytest.mark.parametrize("M,N,Kd", [(64, 240, 768), (100, 928, 768), (33, 240, 928), (16, 16, 16), (70, 384, 2048)])
+def test_row_linear(K, M, N, Kd):
+    r = rng(300 + N)
+    X, W, b = randn_h(r, (M, Kd)), randn_h(r, (N, Kd), 0.05), randn_h(r, (N,), 0.2)
+    want = orc.row_linear(X, W, b, f64=True)
+    got = host(K.row_spmm_add_bias(dev(X), dev(W), dev(b)))
+    check_close(got, want, max_abs=max(np.abs(want.astype(np.float64)).max() * 2.0 ** -10, 1e-3), mean_rel=5e-4, what="row linear")
+
+
+# ------------------------------------------------------------------ attention
+ATT_CASES = [
+    # S, H, d_model, batch, lens, mask, log2_scale
+    (128, 12, 768, 1, None, True, 1.0),            # config-1 shape, reference exponent
+    (128, 12, 768, 1, None, False, LOG2E),         # no mask, textbook exponent
+    (512, 12, 768, 2, None, True, 1.0),            # config-3 shape (batch cut to 2)
+    (512, 12, 768, 3, [512, 77, 300], True, LOG2E),  # per-sequence lengths
+    (100, 4, 256, 2, [100, 37], True, 1.0),        # S not a multiple of any tile
+    (64, 2, 64, 1, None, True, 1.0),               # head_dim 32
+    (96, 2, 256, 2, [96, 50], True, LOG2E),        # head_dim 128
+    (16, 1, 64, 1, None, True, 1.0),               # the reference's minimum block
+    (200, 12, 768, 1, [0], False, 1.0),            # empty sequence -> zeros
+]
+
+
+@pytest.mark.parametrize("S,H,d,B,lens,use_mask,ls", ATT_CASES)
+def test_otf_attention(K, S, H, d, B, lens, use_mask, ls):
+    r = rng(400 + S + H)
+    Q, Kk, V = (randn_h(r, (B * S, d)) for _ in range(3))
+    mask = randn_h(r, (S, S)) if use_mask else None
+    lens_np = None if lens is None else np.array(lens, np.int32)
+    want = orc.otf_attention(Q, Kk, V, mask, S, H, B, lens_np, ls, f64=True)
+    got = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), None if mask is None else dev(mask), S, H, B,
+                               None if lens is None else dev(lens_np), ls))
+    check_close(got, want, max_abs=5e-3, mean_rel=1e-3, what="OTF attention")
+    if lens is not None:
+        for b, L in enumerate(lens):
+            assert (got[b * S + L:(b + 1) * S] == 0).all()
+
+
+def test_otf_attention_closed_forms(K):
+    r = rng(41)
+    S, H, d = 128, 12, 768
+    V, Kk = randn_h(r, (S, d)), randn_h(r, (S, d))
+    zeroQ = np.zeros((S, d), np.float16)
+    got = host(K.OTF_attention(dev(zeroQ), dev(Kk), dev(V), None, S, H)).astype(np.float64)
+    want = np.repeat(V.astype(np.float64).mean(0, keepdims=True), S, 0)
+    assert np.abs(got - want).max() < 2e-3            # uniform scores -> column mean of V (P rounded to half)
+    mask = np.full((S, S), -60000.0, np.float16)
+    tgt = (np.arange(S) * 7) % S
+    mask[np.arange(S), tgt] = 0
+    got = host(K.OTF_attention(dev(randn_h(r, (S, d))), dev(Kk), dev(V), dev(mask), S, H))
+    assert np.array_equal(got, V[tgt])                # one-hot mask -> that V row exactly
+    ones = np.ones((S, d), np.float16)
+    got = host(K.OTF_attention(dev(randn_h(r, (S, d))), dev(Kk), dev(ones), dev(randn_h(r, (S, S))), S, H))
+    assert np.abs(got.astype(np.float64) - 1).max() <= 2.0 ** -10   # rows of P sum to 1
+
+
+def test_otf_attention_varlen_equals_padded(K):
+    r = rng(42)
+    S, H, d, B = 256, 12, 768, 4
+    lens = np.array([256, 31, 130, 64], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    Q, Kk, V = (randn_h(r, (B * S, d)) for _ in range(3))
+    mask = randn_h(r, (S, S), 0.5)
+    padded = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), dev(mask), S, H, B, dev(lens), 1.0))
+    sel = np.concatenate([np.arange(b * S, b * S + lens[b]) for b in range(B)])
+    packed = host(K.OTF_attention_varlen(dev(Q[sel]), dev(Kk[sel]), dev(V[sel]), dev(mask), dev(cu), S, H, 1.0))
+    assert np.array_equal(packed, padded[sel])        # same kernel, same arithmetic order
+    want = orc.otf_attention(Q, Kk, V, mask, S, H, B, lens, 1.0, f64=True)
+    check_close(packed, want[sel], max_abs=5e-3, mean_rel=1e-3, what="varlen attention")
+
+
+def test_prune_attention(K):
+    r = rng(43)
+    S, H, d, B = 160, 12, 768, 2
+    hd = d // H
+    Q, Kk, V = (randn_h(r, (B * S, d)) for _ in range(3))
+    mask = randn_h(r, (S, S), 0.3)
+    lens = np.array([160, 99], np.int32)
+    qk_id = orc.gen_head_balanced_rows(H, hd, 32, seed=1)
+    v_id = orc.gen_sparse_row_mat(d, 0.7, seed=3)                 # 230 kept columns, ragged over heads
+    qk_hp, v_hp = orc.head_ptr(qk_id, H, hd), orc.head_ptr(v_id, H, hd)
+    Qc, Kc, Vc = (np.ascontiguousarray(t) for t in (Q[:, qk_id], Kk[:, qk_id], V[:, v_id]))
+    want = orc.prune_attention(Qc, Kc, Vc, qk_hp, v_id, v_hp, mask, S, d, H, B, lens, f64=True)
+    got = host(K.Prune_attention(dev(Qc), dev(Kc), dev(Vc), dev(qk_hp), dev(v_id), dev(v_hp), dev(mask), S, d, H, B, dev(lens)))
+    check_close(got, want, max_abs=5e-3, mean_rel=1e-3, what="pruned attention")
+    other = np.setdiff1d(np.arange(d), v_id)
+    assert (got[:, other] == 0).all()
+    # the reference's wiring: dense Q/K, compact V (encoder/encoder.cu:76-79)
+    want2 = orc.prune_attention(Q, Kk, Vc, None, v_id, v_hp, mask, S, d, H, B, lens, f64=True)
+    got2 = host(K.Prune_attention(dev(Q), dev(Kk), dev(Vc), None, dev(v_id), dev(v_hp), dev(mask), S, d, H, B, dev(lens)))
+    check_close(got2, want2, max_abs=5e-3, mean_rel=1e-3, what="pruned attention, dense QK")
+
+
+def test_sharedqk_attention_and_scores(K):
+    r = rng(44)
+    S, H, d, B = 200, 12, 768, 2
+    Q, Kk, V = (randn_h(r, (B * S, d), 0.7) for _ in range(3))
+    mask = randn_h(r, (S, S), 0.3)
+    QK = host(K.qk_scores(dev(Q), dev(Kk), S, H, B))
+    want_qk = orc.qk_scores(Q, Kk, S, H, B, f64=True)
+    check_close(QK, want_qk, max_abs=2e-2, mean_rel=5e-4, what="qk scores")
+    want = orc.sharedqk_attention(QK, V, mask, S, H, B, f64=True)
+    got = host(K.sharedQK_attention(dev(QK), dev(V), dev(mask), S, H, B))
+    check_close(got, want, max_abs=5e-3, mean_rel=1e-3, what="sharedQK attention")
+
+
+# -------------------------------------------------------------- data movement
+def test_pack_unpack_scatter(K):
+    r = rng(45)
+    S, B, d = 64, 5, 768
+    lens = np.array([64, 1, 17, 0, 40], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    x = randn_h(r, (B * S, d))
+    sel = np.concatenate([np.arange(b * S, b * S + lens[b]) for b in range(B)]).astype(np.int64)
+    packed = host(K.pack_rows(dev(x), dev(cu), S, int(cu[-1])))
+    assert np.array_equal(packed, x[sel])
+    back = host(K.unpack_rows(dev(packed), dev(cu), S))
+    want = np.zeros_like(x)
+    want[sel] = x[sel]
+    assert np.array_equal(back, want)
+    ids = np.sort(r.choice(d, 230, replace=False)).astype(np.int32)
+    comp = randn_h(r, (50, 240))
+    sc = host(K.scatter_cols(dev(comp), dev(ids), d))
+    want = np.zeros((50, d), np.float16)
+    want[:, ids] = comp[:, :230]
+    assert np.array_equal(sc, want)
