@@ -1,0 +1,247 @@
+#!/usr/bin/env python3
+"""Benchmark of the E.T. encoder hot path on one MI355X.
+
+Workload (config.workload): one BERT-base-shape encoder layer, six tile-pruned
+linears at 80 % tile sparsity (16x16 tiles, seeded), on-the-fly fused attention,
+batch 16 x seq 512, fp16 storage / fp32 accumulate, all sequences full length,
+additive mask supplied (all zeros), base-2 softmax as in the reference.  A
+"step" is one Encoder_tile::run over that batch with inputs resident in HBM.
+
+Prints ONE JSON line: throughput in sequences/s (batch / layer time), the
+roofline figures of the dominant kernel measured live with HIP events around
+every launch of the layer sequence, a per-kernel table, and the CPU oracle
+timed on this box's host cores as a reported baseline.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--extras]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+MFMA_F16_PEAK_TF = 2500.0   # MI355X dense fp16 MFMA, published
+
+D, H, DFF = 768, 12, 3072
+
+
+def tile_bytes(T, N, K, ntile):
+    return 2 * T * K + 512 * ntile + 4 * ntile + 4 * (N // 16 + 1) + 2 * N + 2 * T * N
+
+
+def tile_flops(T, ntile):
+    return 512 * ntile * T
+
+
+def build_layer(orc, r, sparsity, seed):
+    from helpers import make_tile_linear, randn_h
+    shapes = [(D, D)] * 4 + [(DFF, D), (D, DFF)]
+    lins = [make_tile_linear(r, n, k, sparsity, seed=seed + j, std=0.02) for j, (n, k) in enumerate(shapes)]
+    ln = [np.ones(D, np.float16), np.zeros(D, np.float16), np.ones(D, np.float16), np.zeros(D, np.float16)]
+    return lins, ln
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--seq", type=int, default=512)
+    ap.add_argument("--sparsity", type=float, default=0.8)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--extras", action="store_true", help="also time the other BASELINE configurations")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU (the path needs no collectives; it shards by "
+              "batch). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import oracle.et_oracle as orc          # checker / CPU baseline only
+    from et_amd import kernels as K
+    from et_amd.encoder import Encoder_tile, Linear_tile, run_multi
+    from helpers import randn_h, rng
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    B, S = args.batch, args.seq
+    T = B * S
+    r = rng(2025)
+    lins, ln = build_layer(orc, r, args.sparsity, seed=3000)
+    x_h = randn_h(r, (T, D))
+    mask_h = np.zeros((S, S), np.float16)
+    x = torch.from_numpy(x_h).to(dev)
+
+    def mk_linears():
+        return [Linear_tile(l["K"], l["N"], T, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"],
+                            l["bias"], j == 4) for j, l in enumerate(lins)]
+
+    ws = torch.empty(Encoder_tile.buffer_size(D, S, H, B) // 2, dtype=torch.float16, device=dev)
+    enc = Encoder_tile(D, S, H, ws, *mk_linears(), *ln, mask_h, B)
+    out = torch.empty_like(x)
+
+    # ---- whole layer: W warm-up steps, then exactly K timed steps
+    for _ in range(args.warmup):
+        enc.run(out, x)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        enc.run(out, x)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    seqs_per_s = B / (wall / args.steps)
+
+    # ---- same launch sequence with HIP events around every kernel
+    L = mk_linears()
+    mask = torch.from_numpy(mask_h).to(dev)
+    gam = [torch.from_numpy(t).to(dev) for t in ln]
+    b = [torch.empty((T, D), dtype=torch.float16, device=dev) for _ in range(4)]
+    ffn = torch.empty((T, DFF), dtype=torch.float16, device=dev)
+    y = torch.empty((T, D), dtype=torch.float16, device=dev)
+    nt = [l["row_offset"].size for l in lins]
+    steps_def = [
+        ("tile_linear qkv (3 x 768->768, one launch)", lambda: run_multi(L[:3], x, b[:3]),
+         3 * tile_flops(T, nt[0]), sum(tile_bytes(T, D, D, nt[j]) for j in range(3)) - 2 * 2 * T * D, "hbm"),
+        ("attention (on-the-fly)", lambda: K.OTF_attention(b[0], b[1], b[2], mask, S, H, B, None, 1.0, out=b[3]),
+         4 * B * S * S * D, 8 * B * S * D + 2 * S * S, "mfma"),
+        ("tile_linear o (768->768)", lambda: L[3].run(b[3], out=b[0]), tile_flops(T, nt[3]), tile_bytes(T, D, D, nt[3]), "hbm"),
+        ("skip_layernorm 1", lambda: K.skip_layernorm(b[0], x, gam[0], gam[1]), 0, 6 * T * D + 4 * D, "hbm"),
+        ("tile_linear ffn1+gelu (768->3072)", lambda: L[4].run(b[0], out=ffn), tile_flops(T, nt[4]), tile_bytes(T, DFF, D, nt[4]), "hbm"),
+        ("tile_linear ffn2 (3072->768)", lambda: L[5].run(ffn, out=y), tile_flops(T, nt[5]), tile_bytes(T, D, DFF, nt[5]), "hbm"),
+        ("skip_layernorm 2", lambda: K.skip_layernorm(y, b[0], gam[2], gam[3]), 0, 6 * T * D + 4 * D, "hbm"),
+    ]
+    nk = len(steps_def)
+    reps = max(20, min(args.steps, 100))
+    for _ in range(5):
+        for _, fn, *_ in steps_def:
+            fn()
+    ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nk)] for _ in range(reps)]
+    torch.cuda.synchronize()
+    for i in range(reps):
+        for j, (_, fn, *_r) in enumerate(steps_def):
+            ev[i][j][0].record()
+            fn()
+            ev[i][j][1].record()
+    torch.cuda.synchronize()
+    kern = []
+    for j, (name, _, flops, nbytes, bound) in enumerate(steps_def):
+        us = float(np.mean([ev[i][j][0].elapsed_time(ev[i][j][1]) for i in range(reps)])) * 1e3
+        kern.append({"kernel": name, "us": round(us, 2), "algo_MB": round(nbytes / 1e6, 2), "GFLOP": round(flops / 1e9, 3),
+                     "GBps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                     "TFLOPs": round(flops / us / 1e6, 1), "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TF, 4),
+                     "bound": bound})
+    dom = max(kern, key=lambda k: k["us"])
+    if dom["bound"] == "hbm":
+        roof = {"kernel": dom["kernel"], "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": dom["hbm_frac"], "traffic": None, "mfma_frac": dom["mfma_frac"]}
+    else:
+        roof = {"kernel": dom["kernel"], "bound": "mfma", "achieved": dom["TFLOPs"], "peak": MFMA_F16_PEAK_TF,
+                "unit": "TFLOP/s", "frac": dom["mfma_frac"], "traffic": None, "hbm_frac": dom["hbm_frac"]}
+    layer_flops = sum(k["GFLOP"] for k in kern)
+    total_us = sum(k["us"] for k in kern)
+
+    # ---- parity spot check of the timed configuration (rows of the first sequence)
+    got = out[:S].float().cpu().numpy()
+    want = orc.encoder_tile_layer(x_h[:S], lins, ln, mask_h, S, H, 1, None, 1.0).astype(np.float32)
+    max_abs = float(np.abs(got - want).max())
+    mean_rel = float(np.abs(got - want).mean() / np.abs(want).mean())
+
+    # ---- CPU baseline: the fp32 host-loop oracle on a bounded sample of the same workload
+    cpu = None
+    if not args.no_cpu:
+        cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        nseq = 2
+        orc.encoder_tile_layer(x_h[:S], lins, ln, mask_h, S, H, 1, None, 1.0)  # warm
+        t0 = time.perf_counter()
+        orc.encoder_tile_layer(x_h[:nseq * S], lins, ln, mask_h, S, H, nseq, None, 1.0)
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(nseq / dt, 3), "unit": "seqs/s", "cores": cores, "kind": "port",
+               "sample": f"{nseq} of the {B} sequences (seq {S}) through the fp32 host-loop oracle layer, {dt:.2f} s",
+               "ms_per_seq": round(dt / nseq * 1e3, 2)}
+
+    extras = {}
+    if args.extras:
+        extras = run_extras(torch, orc, K, dev)
+
+    res = {
+        "metric": "encoder_layer_seqs_per_s", "value": round(seqs_per_s, 1), "unit": "seqs/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "latency_us": round(ms_per_step * 1e3, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 storage, f32 accumulate", "data": "synthetic",
+        "config": {"workload": f"BERT-base encoder layer, {int(args.sparsity * 100)}% tile-pruned linears (16x16), "
+                               f"on-the-fly attention, batch {B} x seq {S}, all full length (BASELINE config 3)",
+                   "batch": B, "seq_len": S, "d_model": D, "heads": H, "d_ff": DFF, "sparsity": args.sparsity,
+                   "softmax_base": 2, "mask": "additive zeros"},
+        "layer_GFLOP_surviving": round(layer_flops, 2),
+        "layer_mfma_frac": round(layer_flops / (ms_per_step * 1e3) / 1e3 / MFMA_F16_PEAK_TF, 4),
+        "sum_kernel_us": round(total_us, 1),
+        "parity_vs_oracle": {"max_abs": round(max_abs, 5), "mean_rel": round(mean_rel, 6), "rows": S},
+        "roofline": roof, "kernels": kern, "cpu_baseline": cpu,
+    }
+    if extras:
+        res["extras"] = extras
+    print(json.dumps(res))
+
+
+def run_extras(torch, orc, K, dev):
+    """Other BASELINE configurations, timed with HIP events (reported, not the headline)."""
+    from et_amd.encoder import Encoder_tile, Linear_tile
+    from helpers import make_tile_linear, randn_h, rng
+    out = {}
+
+    def timeit(fn, reps=100, warm=10):
+        for _ in range(warm):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps * 1e3  # us
+
+    # config 2: tile linear 4096x768 -> 3072 at 0/50/80/90 %
+    r = rng(7)
+    M, N, Kd = 4096, 3072, 768
+    X = torch.from_numpy(randn_h(r, (M, Kd))).to(dev)
+    Y = torch.empty((M, N), dtype=torch.float16, device=dev)
+    sweep = []
+    for sp in (0.0, 0.5, 0.8, 0.9):
+        lin = make_tile_linear(r, N, Kd, sp, seed=11, std=0.02)
+        nt = lin["row_offset"].size
+        lt = Linear_tile(Kd, N, M, nt, lin["data"], lin["row_ptr"], lin["row_offset"], lin["bias"])
+        us = timeit(lambda: lt.run(X, out=Y))
+        fl, by = tile_flops(M, nt), tile_bytes(M, N, Kd, nt)
+        sweep.append({"sparsity": sp, "ntile": nt, "us": round(us, 2), "mfma_frac": round(fl / us / 1e6 / MFMA_F16_PEAK_TF, 4),
+                      "hbm_frac": round(by / us / 1e3 / HBM_PEAK_GBS, 4)})
+    out["config2_tile_linear_4096x768x3072"] = sweep
+
+    # config 1: dense layer, batch 1 x seq 128
+    r = rng(8)
+    S, B = 128, 1
+    lins, ln = build_layer(orc, r, 0.0, seed=50)
+    x = torch.from_numpy(randn_h(r, (S, D))).to(dev)
+    ws = torch.empty(Encoder_tile.buffer_size(D, S, H, B) // 2, dtype=torch.float16, device=dev)
+    L = [Linear_tile(l["K"], l["N"], S, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], j == 4)
+         for j, l in enumerate(lins)]
+    enc = Encoder_tile(D, S, H, ws, *L, *ln, np.zeros((S, S), np.float16), B)
+    o = torch.empty_like(x)
+    us = timeit(lambda: enc.run(o, x))
+    out["config1_dense_layer_b1_s128"] = {"us": round(us, 2), "seqs_per_s": round(1e6 / us, 1)}
+    return out
+
+
+if __name__ == "__main__":
+    main()

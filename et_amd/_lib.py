@@ -74,6 +74,7 @@ PROTOTYPES = {
     "et_stream_synchronize": (_i, [_vp]),
     "et_device_synchronize": (_i, []),
     "et_device_cu_count": (_i, []),
+    "et_tuning_set": (_i, [C.c_char_p, _i]),
 }
 
 _lib = None

@@ -36,28 +36,44 @@ namespace et {
 constexpr int TL_THREADS = 512;
 constexpr int TL_WAVES = 8;
 constexpr int TL_BM = 32;
-constexpr int TL_PAD = 8;        // halves; makes the LDS row stride an odd multiple of 16 B
-constexpr int TL_MAX_PANEL = 1008; // single-panel K limit: 32*(1008+8)*2 B < 64 KB
+constexpr int TL_PAD = 16;       // halves; LDS row stride == 32 (mod 64) bytes: measured conflict-free for ds_read_b128
+constexpr int TL_MAX_PANEL = 992;  // single-panel K limit: 32*(992+16)*2 B < 64 KB
 constexpr int TL_CHUNK = 768;
 constexpr int TL_MAX_LIN = 4;
 
-enum { TL_CSR = 0, TL_FILTER = 1, TL_DENSE = 2 };
+// TL_PLAN: plan layout (see et_tile_plan_create): tiles ordered (chunk,
+//          block-row, column), every (chunk, block-row) segment padded to an
+//          even tile count with an all-zero tile, cptr[c*nbr + bn] in tiles.
+// TL_RAW:  caller's tile_mat as is (any order inside a block-row, odd counts),
+//          K fits one LDS panel; cptr is row_ptr.
+// TL_FILTER: caller's tile_mat, K walked in chunks by filtering every list.
+// TL_DENSE: W row-major [N x K] (the row-pruned linear's compacted rows).
+enum { TL_PLAN = 0, TL_RAW = 1, TL_FILTER = 2, TL_DENSE = 3 };
 
 struct TlProblem {
     f16 *Y;
-    const int *cptr;       // TL_CSR: per-(block-row,chunk) CSR; TL_FILTER: row_ptr
+    const int *cptr;
     const int *row_offset; // element column offset per tile
-    const f16 *data;       // tile_mat data, or dense row-major W for TL_DENSE
+    const f16 *data;       // tile data, or dense row-major W for TL_DENSE
     const f16 *bias;
     int N;
     int nbr; // N / 16
 };
 
+// kernel arguments; per-linear fields as separate arrays that are only ever
+// indexed with constants (a dynamically indexed by-value struct would be
+// copied to scratch memory)
 struct TlArgs {
-    TlProblem p[TL_MAX_LIN];
+    f16 *Y[TL_MAX_LIN];
+    const int *cptr[TL_MAX_LIN];
+    const int *row_offset[TL_MAX_LIN];
+    const f16 *data[TL_MAX_LIN];
+    const f16 *bias[TL_MAX_LIN];
+    int N[TL_MAX_LIN];
     const f16 *X;
-    int nlin, M, K, KC, nchunk, ncg, total, per_xcd;
+    int nlin, M, K, KC, nchunk, ncg, total, per_xcd, dbg;
 };
+#define TL_SEL(f) (lin == 0 ? a.f[0] : lin == 1 ? a.f[1] : lin == 2 ? a.f[2] : a.f[3])
 
 // tanh-form GELU of kernels/linear.cu:36-48: x^3 in half, the tanh argument
 // and 0.5(1+tanh u) in fp32, rounded to half, times x in half.
@@ -72,37 +88,105 @@ __device__ __forceinline__ f16 gelu_h(f16 v) {
     return v * (f16)t;
 }
 
-template <int NB, bool GELU, int MODE>
-__global__ void __launch_bounds__(TL_THREADS) tile_linear_kernel(const TlArgs a) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
-    f16 *xs = reinterpret_cast<f16 *>(tl_smem);
+// what every variant shares: workgroup -> (row panel, linear, column group)
+struct TlCtx {
+    int lin, cg, m0, wave, lane, c16, g4, khalf8, hi, ldx, bn_wg, bn0, ld_r, ld_c;
+};
 
+__device__ __forceinline__ bool tl_context(const TlArgs &a, int nb, TlCtx &x) {
     // Workgroups that share a row panel of X get consecutive ids on ONE XCD
     // (hardware round-robins consecutive workgroup ids over the 8 XCDs), so
     // the panel is fetched into that XCD's L2 once.
-    const int pid = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3);
+    const int pid = (a.dbg & 64) ? (int)blockIdx.x : (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3);
     if (pid >= a.total)
-        return;
+        return false;
     const int per_rp = a.ncg * a.nlin;
     const int rp = pid / per_rp;
     const int rest = pid - rp * per_rp;
-    const int lin = rest / a.ncg;
-    const int cg = rest - lin * a.ncg;
-    TlProblem P = a.p[0];
-    if (lin == 1) P = a.p[1];
-    if (lin == 2) P = a.p[2];
-    if (lin == 3) P = a.p[3];
+    x.lin = rest / a.ncg;
+    x.cg = rest - x.lin * a.ncg;
+    x.m0 = rp * TL_BM;
+    x.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    x.lane = threadIdx.x & 63;
+    x.c16 = x.lane & 15;
+    x.g4 = x.lane >> 4;
+    x.khalf8 = (x.g4 & 1) * 8;
+    x.hi = x.lane >> 5;
+    x.ldx = a.KC + ((a.KC & 31) ? 0 : TL_PAD);
+    x.bn_wg = x.cg * (TL_WAVES * nb);
+    x.bn0 = x.bn_wg + x.wave * nb;
+    x.ld_r = threadIdx.x >> 4; // 0..31: panel row this thread stages
+    x.ld_c = threadIdx.x & 15;
+    return true;
+}
 
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
-    const int c16 = lane & 15;
-    const int g4 = lane >> 4;
-    const int khalf8 = (g4 & 1) * 8;
-    const int hi = lane >> 5;
-    const int m0 = rp * TL_BM;
-    const int ldx = a.KC + TL_PAD;
-    const int bn_wg = cg * (TL_WAVES * NB);
-    const int bn0 = bn_wg + wave * NB;
+// bias (+GELU), round to half, stage in LDS (the X panel's storage), then
+// 16-byte row-contiguous stores
+template <int NB, bool GELU>
+__device__ __forceinline__ void tl_epilogue(const TlArgs &a, const TlCtx &x, f16 *xs, f16 *Y, int N,
+                                            int nbr, const f32x4 (&acc)[NB][2], const f16x4 (&b4)[NB]) {
+    __syncthreads(); // every wave is done reading the X panel
+    constexpr int BNW = TL_WAVES * NB * 16; // output columns per workgroup
+    constexpr int ldy = BNW + TL_PAD;
+    f16 *ys = xs;
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        const int bn = x.bn0 + j;
+        if (bn >= nbr)
+            continue;
+        const int ncol = (bn - x.bn_wg) * 16 + x.g4 * 4;
+#pragma unroll
+        for (int ms = 0; ms < 2; ms++) {
+            f16x4 o;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const f16 v = (f16)(acc[j][ms][r] + (float)b4[j][r]);
+                o[r] = GELU ? gelu_h(v) : v;
+            }
+            *reinterpret_cast<f16x4 *>(ys + (ms * 16 + x.c16) * ldy + ncol) = o;
+        }
+    }
+    __syncthreads();
+    const int col0 = x.bn_wg * 16;
+    const int wcols = min(BNW, N - col0);
+    const int cpr = wcols >> 3;
+    if (x.m0 + x.ld_r < a.M && !(a.dbg & 2)) {
+        u32x4 *dst = reinterpret_cast<u32x4 *>(Y + (size_t)(x.m0 + x.ld_r) * N + col0);
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(ys + x.ld_r * ldy);
+        for (int cc = x.ld_c; cc < cpr; cc += 16)
+            dst[cc] = src[cc];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Plan kernel (the fast path).  Because a wave owns NB CONSECUTIVE block-rows
+// and the plan stores tiles in (chunk, block-row) order with even segments,
+// the wave's work for a chunk is ONE contiguous stream of tile pairs: 1 KB of
+// W per pair at an address that is linear in the pair index, plus one int per
+// half-wave giving the LDS byte offset of that tile's X columns.  The stream
+// is consumed through a fixed 4-stage register pipeline (stage = pair index
+// mod 4), every load unconditional with a clamped address, so four pairs are
+// always in flight per wave and the waits are counted, not drained.  Products
+// accumulate into one running 32x16 accumulator; when the stream crosses a
+// block-row boundary (a scalar compare per pair) it is added into that
+// block-row's static accumulator.
+// ---------------------------------------------------------------------------
+template <int NB, bool GELU>
+__global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
+    f16 *xs = reinterpret_cast<f16 *>(tl_smem);
+    TlCtx x;
+    if (!tl_context(a, NB, x))
+        return;
+    const int lin = x.lin;
+    f16 *const Yp = TL_SEL(Y);
+    const int *const cptr = TL_SEL(cptr);
+    const int *const poff = TL_SEL(row_offset); // LDS byte offset per tile (chunk-local column * 2)
+    const f16 *const data = TL_SEL(data);
+    const f16 *const bias = TL_SEL(bias);
+    const int N = TL_SEL(N);
+    const int nbr = N >> 4;
+    const int hi = x.hi, lane = x.lane;
 
     f32x4 acc[NB][2];
 #pragma unroll
@@ -110,158 +194,260 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_kernel(const TlArgs a)
         acc[j][0] = f32x4{0.f, 0.f, 0.f, 0.f};
         acc[j][1] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+    const char *xlane = reinterpret_cast<const char *>(xs + x.c16 * x.ldx + x.khalf8);
+    const int xrow16 = 16 * x.ldx * 2; // bytes between the two 16-row subtiles
+    const bool rowok = (x.m0 + x.ld_r) < a.M && !(a.dbg & 1);
+    const u32x4 *xsrc = reinterpret_cast<const u32x4 *>(a.X + (size_t)(x.m0 + x.ld_r) * a.K);
+    u32x4 *xdst = reinterpret_cast<u32x4 *>(xs + x.ld_r * x.ldx);
 
-    const f16 *xlane = xs + c16 * ldx + khalf8;
-    const int ld_r = threadIdx.x >> 4; // 0..31: panel row this thread stages
-    const int ld_c = threadIdx.x & 15;
+    // global -> register half of the panel staging: all of a thread's loads
+    // are in flight together
+    u32x4 pv[8];
+#define TL_PANEL_LOAD(c_)                                                                         \
+    {                                                                                             \
+        const int pk0 = (c_) * a.KC;                                                              \
+        const int pcpr = min(a.KC, a.K - pk0) >> 3;                                               \
+        _Pragma("unroll") for (int u = 0; u < 8; u++) {                                           \
+            const int cc = x.ld_c + 16 * u;                                                       \
+            pv[u] = u32x4{0u, 0u, 0u, 0u};                                                        \
+            if (rowok && cc < pcpr)                                                               \
+                pv[u] = xsrc[(pk0 >> 3) + cc];                                                    \
+        }                                                                                         \
+    }
+    TL_PANEL_LOAD(0)
+
+    f16x4 b4[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        b4[j] = f16x4{0, 0, 0, 0};
+        if (x.bn0 + j < nbr)
+            b4[j] = *reinterpret_cast<const f16x4 *>(bias + (x.bn0 + j) * 16 + x.g4 * 4);
+    }
+    const f16 *wbase = data + hi * 256 + x.c16 * 16 + x.khalf8; // + pair * 512
+    const int *obase = poff + hi;                               // + pair * 2
+    const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+
+    for (int c = 0; c < a.nchunk; c++) {
+        const int kc = min(a.KC, a.K - c * a.KC);
+        // pair-index boundaries of the wave's block-rows: lane j holds the end
+        // of block-row j (read back with v_readlane)
+        const int bidx = c * nbr + min(x.bn0 + min(lane, NB), nbr);
+        const int bvec = cptr[bidx] >> 1;
+
+        if (c > 0) {
+            __syncthreads(); // every wave is done with the previous panel
+            TL_PANEL_LOAD(c)
+        }
+        {
+            const int cpr = kc >> 3;
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int cc = x.ld_c + 16 * u;
+                if (cc < cpr)
+                    xdst[cc] = pv[u];
+            }
+        }
+        // the first four pairs of the stream: requested before the barrier so
+        // that their latency overlaps the wait for the other waves
+        const int q0 = __builtin_amdgcn_readfirstlane(bvec);
+        const int qend = (a.dbg & 4) ? q0 : __builtin_amdgcn_readlane(bvec, NB);
+        const int qlast = max(qend - 1, q0);
+        f16x8 w0 = zero8, w1 = zero8, w2 = zero8, w3 = zero8;
+        int o0 = 0, o1 = 0, o2 = 0, o3 = 0;
+        if (q0 < qend) {
+            const int qa = q0, qb = min(q0 + 1, qlast), qc = min(q0 + 2, qlast), qd = min(q0 + 3, qlast);
+            o0 = obase[qa * 2];
+            w0 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qa * 512);
+            o1 = obase[qb * 2];
+            w1 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qb * 512);
+            o2 = obase[qc * 2];
+            w2 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qc * 512);
+            o3 = obase[qd * 2];
+            w3 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qd * 512);
+        }
+        __syncthreads();
+
+        if (q0 < qend) {
+            f32x4 cur0 = f32x4{0.f, 0.f, 0.f, 0.f}, cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
+            int j = 0;
+            int bend = __builtin_amdgcn_readlane(bvec, 1);
+            while (bend == q0 && j + 1 < NB) { // leading empty block-rows
+                j++;
+                bend = __builtin_amdgcn_readlane(bvec, j + 1);
+            }
+            // drain once here so that inside the loop the waits can be counted
+            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+            // X operands are read one stage ahead (ping-pong xa0/xb0 <-> xa1/xb1)
+            f16x8 xa0 = *reinterpret_cast<const f16x8 *>(xlane + o0);
+            f16x8 xb0 = *reinterpret_cast<const f16x8 *>(xlane + o0 + xrow16);
+            f16x8 xa1 = zero8, xb1 = zero8;
+#define TL_STAGE(W_, O_, ONEXT_, XA_, XB_, XAN_, XBN_, I_)                                        \
+    {                                                                                             \
+        XAN_ = *reinterpret_cast<const f16x8 *>(xlane + ONEXT_);                                  \
+        XBN_ = *reinterpret_cast<const f16x8 *>(xlane + ONEXT_ + xrow16);                         \
+        cur0 = mfma16x16x32(W_, XA_, cur0);                                                       \
+        cur1 = mfma16x16x32(W_, XB_, cur1);                                                       \
+        {                                                                                         \
+            const int qn = min(q + (I_) + 4, qlast);                                              \
+            O_ = obase[qn * 2];                                                                   \
+            W_ = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qn * 512);                      \
+        }                                                                                         \
+        if (q + (I_) + 1 == bend) { /* block-row j is complete: acc[j] += cur, branch-free */     \
+            _Pragma("unroll") for (int k = 0; k < NB; k++) {                                      \
+                const float mk = (k == j) ? 1.0f : 0.0f;                                          \
+                _Pragma("unroll") for (int r = 0; r < 4; r++) {                                   \
+                    acc[k][0][r] = __builtin_fmaf(cur0[r], mk, acc[k][0][r]);                     \
+                    acc[k][1][r] = __builtin_fmaf(cur1[r], mk, acc[k][1][r]);                     \
+                }                                                                                 \
+            }                                                                                     \
+            cur0 = f32x4{0.f, 0.f, 0.f, 0.f};                                                     \
+            cur1 = f32x4{0.f, 0.f, 0.f, 0.f};                                                     \
+            do {                                                                                  \
+                j++;                                                                              \
+                bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));                           \
+            } while (bend == q + (I_) + 1 && j + 1 < NB);                                         \
+        }                                                                                         \
+    }
+            int q = q0;
+            for (; q + 4 <= qend; q += 4) { // straight-line body: counted waits
+                TL_STAGE(w0, o0, o1, xa0, xb0, xa1, xb1, 0)
+                TL_STAGE(w1, o1, o2, xa1, xb1, xa0, xb0, 1)
+                TL_STAGE(w2, o2, o3, xa0, xb0, xa1, xb1, 2)
+                TL_STAGE(w3, o3, o0, xa1, xb1, xa0, xb0, 3)
+            }
+            if (q < qend) {
+                TL_STAGE(w0, o0, o1, xa0, xb0, xa1, xb1, 0)
+                if (q + 1 < qend) {
+                    TL_STAGE(w1, o1, o2, xa1, xb1, xa0, xb0, 1)
+                    if (q + 2 < qend)
+                        TL_STAGE(w2, o2, o3, xa0, xb0, xa1, xb1, 2)
+                }
+            }
+#undef TL_STAGE
+        }
+    }
+#undef TL_PANEL_LOAD
+    tl_epilogue<NB, GELU>(a, x, xs, Yp, N, nbr, acc, b4);
+}
+
+// ---------------------------------------------------------------------------
+// Generic kernel: the caller's own tile_mat (TL_RAW / TL_FILTER) or a dense
+// row-major weight (TL_DENSE).  Same mapping, plain per-block-row loops with
+// per-lane predicates.
+// ---------------------------------------------------------------------------
+template <int NB, bool GELU, int MODE>
+__global__ void __launch_bounds__(TL_THREADS) tile_linear_generic_kernel(const TlArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
+    f16 *xs = reinterpret_cast<f16 *>(tl_smem);
+    TlCtx x;
+    if (!tl_context(a, NB, x))
+        return;
+    const int lin = x.lin;
+    f16 *const Yp = TL_SEL(Y);
+    const int *const cptr = TL_SEL(cptr);
+    const int *const roff = TL_SEL(row_offset);
+    const f16 *const data = TL_SEL(data);
+    const f16 *const bias = TL_SEL(bias);
+    const int N = TL_SEL(N);
+    const int nbr = N >> 4;
+    const int hi = x.hi;
+
+    f32x4 acc[NB][2];
+    f16x4 b4[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        acc[j][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+        acc[j][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+        b4[j] = f16x4{0, 0, 0, 0};
+        if (x.bn0 + j < nbr)
+            b4[j] = *reinterpret_cast<const f16x4 *>(bias + (x.bn0 + j) * 16 + x.g4 * 4);
+    }
+    const f16 *xlane = xs + x.c16 * x.ldx + x.khalf8;
+    const int xrow16 = 16 * x.ldx;
+    const bool rowok = (x.m0 + x.ld_r) < a.M;
+    const u32x4 *xsrc = reinterpret_cast<const u32x4 *>(a.X + (size_t)(x.m0 + x.ld_r) * a.K);
+    u32x4 *xdst = reinterpret_cast<u32x4 *>(xs + x.ld_r * x.ldx);
+    const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
 
     for (int c = 0; c < a.nchunk; c++) {
         const int k0 = c * a.KC;
         const int kc = min(a.KC, a.K - k0);
         if (c > 0)
             __syncthreads();
-        { // stage X[m0..m0+31][k0..k0+kc) into LDS, rows beyond M as zeros
+        {
             const int cpr = kc >> 3;
-            const bool rowok = (m0 + ld_r) < a.M;
-            const u32x4 *src = reinterpret_cast<const u32x4 *>(a.X + (size_t)(m0 + ld_r) * a.K + k0);
-            u32x4 *dst = reinterpret_cast<u32x4 *>(xs + ld_r * ldx);
-            for (int cc = ld_c; cc < cpr; cc += 16) {
-                u32x4 v = u32x4{0u, 0u, 0u, 0u};
-                if (rowok)
-                    v = src[cc];
-                dst[cc] = v;
+            u32x4 pv[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int cc = x.ld_c + 16 * u;
+                pv[u] = u32x4{0u, 0u, 0u, 0u};
+                if (rowok && cc < cpr)
+                    pv[u] = xsrc[(k0 >> 3) + cc];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int cc = x.ld_c + 16 * u;
+                if (cc < cpr)
+                    xdst[cc] = pv[u];
             }
         }
         __syncthreads();
-
 #pragma unroll
         for (int j = 0; j < NB; j++) {
-            const int bn = bn0 + j;
-            if (bn >= P.nbr)
+            const int bn = x.bn0 + j;
+            if (bn >= nbr)
                 continue;
-            if (MODE == TL_CSR) {
-                const int s = P.cptr[bn * a.nchunk + c];
-                const int e = P.cptr[bn * a.nchunk + c + 1];
-                const f16 *wlane = P.data + c16 * 16 + khalf8;
-                int i = s;
-                f16x8 w_n = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-                int off_n = 0;
-                if (i + 1 < e) {
-                    off_n = P.row_offset[i + hi];
-                    w_n = *reinterpret_cast<const f16x8 *>(wlane + (size_t)(i + hi) * 256);
-                }
-                for (; i + 1 < e; i += 2) {
-                    const f16x8 w = w_n;
-                    const int off = off_n - k0;
-                    if (i + 3 < e) {
-                        off_n = P.row_offset[i + 2 + hi];
-                        w_n = *reinterpret_cast<const f16x8 *>(wlane + (size_t)(i + 2 + hi) * 256);
-                    }
+            if (MODE == TL_DENSE) {
+                const f16 *wrow = data + (size_t)(bn * 16 + x.c16) * a.K + k0 + x.khalf8;
+                const int nt = kc >> 4;
+                for (int i = 0; i < nt; i += 2) {
+                    const bool ok = i + hi < nt;
+                    const int off = (ok ? i + hi : i) * 16;
+                    f16x8 w = zero8;
+                    if (ok)
+                        w = *reinterpret_cast<const f16x8 *>(wrow + off);
                     const f16x8 x0 = *reinterpret_cast<const f16x8 *>(xlane + off);
-                    const f16x8 x1 = *reinterpret_cast<const f16x8 *>(xlane + off + 16 * ldx);
+                    const f16x8 x1 = *reinterpret_cast<const f16x8 *>(xlane + off + xrow16);
                     acc[j][0] = mfma16x16x32(w, x0, acc[j][0]);
                     acc[j][1] = mfma16x16x32(w, x1, acc[j][1]);
                 }
-                if (i < e) { // odd tail: the upper half-wave multiplies by zero weights
-                    const int off = P.row_offset[i] - k0;
-                    f16x8 w = *reinterpret_cast<const f16x8 *>(wlane + (size_t)i * 256);
-                    if (hi)
-                        w = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-                    const f16x8 x0 = *reinterpret_cast<const f16x8 *>(xlane + off);
-                    const f16x8 x1 = *reinterpret_cast<const f16x8 *>(xlane + off + 16 * ldx);
-                    acc[j][0] = mfma16x16x32(w, x0, acc[j][0]);
-                    acc[j][1] = mfma16x16x32(w, x1, acc[j][1]);
-                }
-            } else if (MODE == TL_FILTER) {
-                const int s = P.cptr[bn];
-                const int e = P.cptr[bn + 1];
-                const f16 *wlane = P.data + c16 * 16 + khalf8;
-                for (int i = s; i < e; i += 2) {
-                    const int ti = min(i + hi, e - 1);
-                    const int off = P.row_offset[ti] - k0;
-                    const bool ok = (i + hi < e) && off >= 0 && off < kc;
-                    if (__builtin_amdgcn_ballot_w64(ok) == 0)
+            } else {
+                const int fs = cptr[bn];
+                const int fe = cptr[bn + 1];
+                const f16 *wlane = data + x.c16 * 16 + x.khalf8;
+                for (int i = fs; i < fe; i += 2) {
+                    const int ti = min(i + hi, fe - 1);
+                    const int off = roff[ti] - k0;
+                    const bool ok = (i + hi < fe) && off >= 0 && off < kc;
+                    if (MODE == TL_FILTER && __builtin_amdgcn_ballot_w64(ok) == 0)
                         continue;
-                    const f16x8 z = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-                    f16x8 w = z, x0 = z, x1 = z;
+                    f16x8 w = zero8, x0 = zero8, x1 = zero8;
                     if (ok) {
                         w = *reinterpret_cast<const f16x8 *>(wlane + (size_t)ti * 256);
                         x0 = *reinterpret_cast<const f16x8 *>(xlane + off);
-                        x1 = *reinterpret_cast<const f16x8 *>(xlane + off + 16 * ldx);
+                        x1 = *reinterpret_cast<const f16x8 *>(xlane + off + xrow16);
                     }
                     acc[j][0] = mfma16x16x32(w, x0, acc[j][0]);
                     acc[j][1] = mfma16x16x32(w, x1, acc[j][1]);
                 }
-            } else { // TL_DENSE: every k-tile of the chunk, W row-major [N x K]
-                const f16 *wlane = P.data + (size_t)(bn * 16 + c16) * a.K + k0 + khalf8;
-                const int nt = kc >> 4;
-                int i = 0;
-                for (; i + 1 < nt; i += 2) {
-                    const int off = (i + hi) * 16;
-                    const f16x8 w = *reinterpret_cast<const f16x8 *>(wlane + off);
-                    const f16x8 x0 = *reinterpret_cast<const f16x8 *>(xlane + off);
-                    const f16x8 x1 = *reinterpret_cast<const f16x8 *>(xlane + off + 16 * ldx);
-                    acc[j][0] = mfma16x16x32(w, x0, acc[j][0]);
-                    acc[j][1] = mfma16x16x32(w, x1, acc[j][1]);
-                }
-                if (i < nt) {
-                    const int off = i * 16;
-                    f16x8 w = *reinterpret_cast<const f16x8 *>(wlane + off);
-                    if (hi)
-                        w = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-                    const f16x8 x0 = *reinterpret_cast<const f16x8 *>(xlane + off);
-                    const f16x8 x1 = *reinterpret_cast<const f16x8 *>(xlane + off + 16 * ldx);
-                    acc[j][0] = mfma16x16x32(w, x0, acc[j][0]);
-                    acc[j][1] = mfma16x16x32(w, x1, acc[j][1]);
-                }
             }
         }
     }
-
-    // ---- epilogue: bias (+GELU), round to half, stage in LDS, coalesced store
-    __syncthreads(); // every wave is done reading the X panel
-    constexpr int BNW = TL_WAVES * NB * 16; // output columns per workgroup
-    constexpr int ldy = BNW + TL_PAD;
-    f16 *ys = xs;
-#pragma unroll
-    for (int j = 0; j < NB; j++) {
-        const int bn = bn0 + j;
-        if (bn >= P.nbr)
-            continue;
-        const f16x4 b4 = *reinterpret_cast<const f16x4 *>(P.bias + bn * 16 + g4 * 4);
-        const int ncol = (bn - bn_wg) * 16 + g4 * 4;
-#pragma unroll
-        for (int ms = 0; ms < 2; ms++) {
-            f16x4 o;
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const f16 v = (f16)(acc[j][ms][r] + (float)b4[r]);
-                o[r] = GELU ? gelu_h(v) : v;
-            }
-            *reinterpret_cast<f16x4 *>(ys + (ms * 16 + c16) * ldy + ncol) = o;
-        }
-    }
-    __syncthreads();
-    {
-        const int col0 = bn_wg * 16;
-        const int wcols = min(BNW, P.N - col0);
-        const int cpr = wcols >> 3;
-        if (m0 + ld_r < a.M) {
-            u32x4 *dst = reinterpret_cast<u32x4 *>(P.Y + (size_t)(m0 + ld_r) * P.N + col0);
-            const u32x4 *src = reinterpret_cast<const u32x4 *>(ys + ld_r * ldy);
-            for (int cc = ld_c; cc < cpr; cc += 16)
-                dst[cc] = src[cc];
-        }
-    }
+    tl_epilogue<NB, GELU>(a, x, xs, Yp, N, nbr, acc, b4);
 }
+#undef TL_SEL
 
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 template <int NB, bool GELU, int MODE>
 static void launch_inst(const TlArgs &a, size_t lds, hipStream_t st) {
-    hipLaunchKernelGGL((tile_linear_kernel<NB, GELU, MODE>), dim3(a.per_xcd * 8),
-                       dim3(TL_THREADS), lds, st, a);
+    if constexpr (MODE == TL_PLAN)
+        hipLaunchKernelGGL((tile_linear_plan_kernel<NB, GELU>), dim3(a.per_xcd * 8),
+                           dim3(TL_THREADS), lds, st, a);
+    else
+        hipLaunchKernelGGL((tile_linear_generic_kernel<NB, GELU, MODE>), dim3(a.per_xcd * 8),
+                           dim3(TL_THREADS), lds, st, a);
 }
 
 template <bool GELU, int MODE>
@@ -275,23 +461,25 @@ static void launch_nb(int nb, const TlArgs &a, size_t lds, hipStream_t st) {
     }
 }
 
-static int env_int(const char *name, int dflt) {
-    const char *v = getenv(name);
-    return (v && *v) ? atoi(v) : dflt;
-}
+// Tuning knobs (et_tuning_set): 0 = automatic.
+static int g_tile_nb = 0;
+static int g_tile_min_wgs = 512;
+static int g_tile_dbg = 0;
 
-// Block-rows per wave: the largest NB that still yields enough workgroups to
-// fill 256 CUs a few times over.  ET_TILE_NB overrides (tuning aid).
+// Block-rows per wave.  Measured on the BERT-base shapes (rows 4096..8192):
+// three block-rows per wave is the best trade between panel re-reads (fewer
+// with larger NB) and register pressure / workgroup count (better with
+// smaller NB); small problems fall back to smaller NB to get enough
+// workgroups for 256 CUs.
 static int choose_nb(int nrp, int nbr_max, int nlin) {
-    static const int forced = env_int("ET_TILE_NB", 0);
+    const int forced = g_tile_nb;
     if (forced == 1 || forced == 2 || forced == 3 || forced == 4 || forced == 6)
         return forced;
-    static const int want = env_int("ET_TILE_MIN_WGS", 1536);
-    const int cand[5] = {6, 4, 3, 2, 1};
-    for (int i = 0; i < 5; i++) {
+    const int cand[3] = {3, 2, 1};
+    for (int i = 0; i < 3; i++) {
         const int nb = cand[i];
         const int ncg = (nbr_max + TL_WAVES * nb - 1) / (TL_WAVES * nb);
-        if ((long)nrp * ncg * nlin >= want)
+        if ((long)nrp * ncg * nlin >= g_tile_min_wgs)
             return nb;
     }
     return 1;
@@ -302,29 +490,38 @@ static int tile_launch(const TlProblem *probs, int nlin, const f16 *X, int M, in
     TlArgs a;
     memset(&a, 0, sizeof(a));
     int nbr_max = 0;
-    for (int i = 0; i < nlin; i++) {
-        a.p[i] = probs[i];
-        nbr_max = std::max(nbr_max, probs[i].nbr);
+    for (int i = 0; i < TL_MAX_LIN; i++) {
+        const TlProblem &p = probs[i < nlin ? i : 0];
+        a.Y[i] = p.Y;
+        a.cptr[i] = p.cptr;
+        a.row_offset[i] = p.row_offset;
+        a.data[i] = p.data;
+        a.bias[i] = p.bias;
+        a.N[i] = p.N;
+        if (i < nlin)
+            nbr_max = std::max(nbr_max, p.nbr);
     }
-    for (int i = nlin; i < TL_MAX_LIN; i++)
-        a.p[i] = probs[0];
     a.X = X;
     a.nlin = nlin;
     a.M = M;
     a.K = K;
     a.KC = KC;
     a.nchunk = nchunk;
+    a.dbg = g_tile_dbg;
     const int nrp = (M + TL_BM - 1) / TL_BM;
     const int nb = choose_nb(nrp, nbr_max, nlin);
     a.ncg = (nbr_max + TL_WAVES * nb - 1) / (TL_WAVES * nb);
     a.total = nrp * a.ncg * nlin;
     a.per_xcd = (a.total + 7) / 8;
-    const size_t lds_x = (size_t)TL_BM * (KC + TL_PAD) * sizeof(f16);
+    const size_t lds_x = (size_t)TL_BM * (KC + ((KC & 31) ? 0 : TL_PAD)) * sizeof(f16);
     const size_t lds_y = (size_t)TL_BM * (TL_WAVES * nb * 16 + TL_PAD) * sizeof(f16);
     const size_t lds = std::max(lds_x, lds_y);
-    if (mode == TL_CSR) {
-        if (gelu) launch_nb<true, TL_CSR>(nb, a, lds, st);
-        else launch_nb<false, TL_CSR>(nb, a, lds, st);
+    if (mode == TL_PLAN) {
+        if (gelu) launch_nb<true, TL_PLAN>(nb, a, lds, st);
+        else launch_nb<false, TL_PLAN>(nb, a, lds, st);
+    } else if (mode == TL_RAW) {
+        if (gelu) launch_nb<true, TL_RAW>(nb, a, lds, st);
+        else launch_nb<false, TL_RAW>(nb, a, lds, st);
     } else if (mode == TL_FILTER) {
         if (gelu) launch_nb<true, TL_FILTER>(nb, a, lds, st);
         else launch_nb<false, TL_FILTER>(nb, a, lds, st);
@@ -367,10 +564,27 @@ static int raw_tile_linear(void *Y, const void *X, const int *row_ptr, const int
     int KC, nchunk;
     chunking(K, &KC, &nchunk);
     return tile_launch(&p, 1, static_cast<const f16 *>(X), M, K, KC, nchunk, gelu,
-                       nchunk == 1 ? TL_CSR : TL_FILTER, static_cast<hipStream_t>(stream));
+                       nchunk == 1 ? TL_RAW : TL_FILTER, static_cast<hipStream_t>(stream));
 }
 
 } // namespace et
+
+extern "C" int et_tuning_set(const char *key, int value) {
+    if (key && !strcmp(key, "tile_nb")) {
+        et::g_tile_nb = value;
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "tile_min_wgs")) {
+        et::g_tile_min_wgs = value;
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "tile_dbg")) {
+        et::g_tile_dbg = value;
+        return ET_OK;
+    }
+    et::set_error("et_tuning_set: unknown key");
+    return ET_ERR_INVALID_ARG;
+}
 
 extern "C" int et_tile_spmm_add_bias(void *Y, const void *X, const int *W_row_ptr,
                                      const int *W_row_offset, const void *W_data, int M,
@@ -436,28 +650,40 @@ extern "C" int et_tile_plan_create(et_tile_plan **plan, int in_feat, int out_fea
     const int nbr = out_feat / 16;
     int KC, nchunk;
     chunking(in_feat, &KC, &nchunk);
-    // order each block-row's tiles by column; build the per-chunk CSR
+    // Plan layout: tiles ordered by (chunk, block-row, column); every
+    // (chunk, block-row) segment padded to an even count with an all-zero
+    // tile that reuses the segment's last column (so a pair never straddles
+    // two block-rows and the kernel needs no odd-tail handling).
     std::vector<int> order(ntile);
     std::iota(order.begin(), order.end(), 0);
     for (int bn = 0; bn < nbr; bn++)
         std::stable_sort(order.begin() + row_ptr[bn], order.begin() + row_ptr[bn + 1],
                          [&](int x, int y) { return row_offset[x] < row_offset[y]; });
-    std::vector<int> off(ntile), cptr((size_t)nbr * nchunk + 1);
-    std::vector<uint16_t> packed((size_t)ntile * 256);
+    std::vector<int> off, cptr((size_t)nbr * nchunk + 1);
+    std::vector<uint16_t> packed;
+    off.reserve(ntile + (size_t)nbr * nchunk);
+    packed.reserve(((size_t)ntile + (size_t)nbr * nchunk) * 256);
     const uint16_t *src = static_cast<const uint16_t *>(data);
-    for (int i = 0; i < ntile; i++) {
-        off[i] = row_offset[order[i]];
-        memcpy(&packed[(size_t)i * 256], src + (size_t)order[i] * 256, 512);
-    }
-    for (int bn = 0; bn < nbr; bn++) {
-        int i = row_ptr[bn];
-        for (int c = 0; c < nchunk; c++) {
-            while (i < row_ptr[bn + 1] && off[i] < c * KC)
-                i++;
-            cptr[(size_t)bn * nchunk + c] = i;
+    for (int c = 0; c < nchunk; c++) {
+        for (int bn = 0; bn < nbr; bn++) {
+            cptr[(size_t)c * nbr + bn] = (int)off.size();
+            int cnt = 0, last = 0;
+            for (int i = row_ptr[bn]; i < row_ptr[bn + 1]; i++) {
+                const int o = row_offset[order[i]];
+                if (o / KC != c)
+                    continue;
+                off.push_back((o - c * KC) * 2);
+                packed.insert(packed.end(), src + (size_t)order[i] * 256, src + (size_t)order[i] * 256 + 256);
+                last = (o - c * KC) * 2;
+                cnt++;
+            }
+            if (cnt & 1) {
+                off.push_back(last);
+                packed.insert(packed.end(), 256, (uint16_t)0);
+            }
         }
     }
-    cptr[(size_t)nbr * nchunk] = ntile;
+    cptr[(size_t)nbr * nchunk] = (int)off.size();
 
     et_tile_plan *p = new et_tile_plan();
     memset(p, 0, sizeof(*p));
@@ -531,7 +757,7 @@ extern "C" int et_tile_plan_run_multi(const et_tile_plan *const *plans, void *co
     if (M == 0)
         return ET_OK;
     return tile_launch(pr, n, static_cast<const f16 *>(X), M, plans[0]->in_feat, plans[0]->KC,
-                       plans[0]->nchunk, false, TL_CSR, static_cast<hipStream_t>(stream));
+                       plans[0]->nchunk, false, TL_PLAN, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int et_tile_plan_run(const et_tile_plan *plan, void *Y, const void *X, int M, int gelu,
@@ -551,5 +777,5 @@ extern "C" int et_tile_plan_run(const et_tile_plan *plan, void *Y, const void *X
     pr.N = plan->out_feat;
     pr.nbr = plan->out_feat / 16;
     return tile_launch(&pr, 1, static_cast<const f16 *>(X), M, plan->in_feat, plan->KC,
-                       plan->nchunk, gelu != 0, TL_CSR, static_cast<hipStream_t>(stream));
+                       plan->nchunk, gelu != 0, TL_PLAN, static_cast<hipStream_t>(stream));
 }

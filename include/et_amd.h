@@ -215,6 +215,11 @@ int et_stream_create(void **stream);
 int et_stream_destroy(void *stream);
 int et_stream_synchronize(void *stream);
 int et_device_synchronize(void);
+/* Launch-heuristic overrides for benchmarking sweeps; value 0 restores the
+ * automatic choice.  Keys: "tile_nb" (block-rows of W per wave in the tile
+ * linear: 1,2,3,4,6), "tile_min_wgs" (workgroups the automatic choice aims
+ * for).  Not thread-safe; results never depend on these. */
+int et_tuning_set(const char *key, int value);
 /* number of compute units of the current device (0 if none) */
 int et_device_cu_count(void);
 
