@@ -15,7 +15,10 @@ SOURCES = ["runtime.hip", "formats.cpp", "skip_layernorm.hip", "tile_linear.hip"
 # packed fp32 ops stay off: some of their forms have produced wrong results on
 # this hardware pool
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
-             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             # keep MFMA accumulators in VGPRs: the softmax / epilogue VALU work
+             # reads them directly instead of copying from AGPRs
+             "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 
 
 def hipcc() -> str:

@@ -23,11 +23,10 @@
 #include "common.h"
 
 #include <cmath>
+#include <type_traits>
 
 namespace et {
 
-constexpr int AT_THREADS = 256;
-constexpr int AT_WAVES = 4;
 constexpr int AT_KT = 64; // keys per tile
 
 struct AttnArgs {
@@ -53,20 +52,26 @@ __device__ __forceinline__ float xor_max_16_32(float v) {
     return v;
 }
 
-template <int HD, int QS, bool PRUNED, bool SHAREDQK>
-__global__ void __launch_bounds__(AT_THREADS) attention_kernel(const AttnArgs a) {
-    constexpr int DK = HD / 32;   // k-steps of Q K^T
-    constexpr int DV = HD / 16;   // 16-wide column subtiles of the output
-    constexpr int LDK = HD + 8;   // halves per staged K row
-    constexpr int LDV = AT_KT + 8; // halves per staged V^T row
+template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK>
+__global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attention_kernel(const AttnArgs a) {
+    constexpr int AT_THREADS = NW * 64; // NW waves, each owning 16*QS query rows
+    constexpr int AT_WAVES = NW;
+    constexpr int DK = HD / 32;    // k-steps of Q K^T
+    constexpr int DV = HD / 16;    // 16-wide column subtiles of the output
+    // LDS row strides.  K rows are read with ds_read_b128 by 16 lanes at a
+    // time: a stride of 32 (mod 64) bytes is conflict-free (measured); V^T rows
+    // are read with ds_read_b64, for which an odd multiple of 16 bytes is.
+    constexpr int LDK = HD + 16;
+    constexpr int LDV = AT_KT + 8;
     constexpr int QB = AT_WAVES * 16 * QS; // queries per workgroup
     constexpr int LDO = HD + 8;
-    constexpr int SM_KV = AT_KT * LDK + HD * LDV;
+    constexpr int KBUF = AT_KT * LDK, VBUF = HD * LDV;
+    constexpr int SM_KV = 2 * (KBUF + VBUF); // double-buffered key/value tiles
     constexpr int SM_O = QB * LDO;
     constexpr int SM = SM_KV > SM_O ? SM_KV : SM_O;
-    __shared__ __attribute__((aligned(16))) f16 smem[SM];
-    f16 *ks = smem;
-    f16 *vt = smem + AT_KT * LDK;
+    extern __shared__ __attribute__((aligned(16))) unsigned char at_smem[];
+    f16 *smem = reinterpret_cast<f16 *>(at_smem);
+    static_assert(SM * 2 <= 160 * 1024, "LDS budget");
 
     const int pid = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3);
     if (pid >= a.total)
@@ -109,6 +114,7 @@ __global__ void __launch_bounds__(AT_THREADS) attention_kernel(const AttnArgs a)
     const int c16 = lane & 15;
     const int g4 = lane >> 4;
     f16 *obase = a.out + (size_t)row0 * a.ldo + h * HD;
+    const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
 
     if (q0 < len) {
         // ---- Q fragments (B operand of S^T), scaled in half like the reference
@@ -119,7 +125,7 @@ __global__ void __launch_bounds__(AT_THREADS) attention_kernel(const AttnArgs a)
             const int q = q0 + (wave * QS + qs) * 16 + c16;
 #pragma unroll
             for (int s = 0; s < DK; s++) {
-                f16x8 v = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                f16x8 v = zero8;
                 if (!SHAREDQK && q < len) {
                     const f16 *qrow = a.Q + (size_t)(row0 + q) * a.ldq + qc0;
                     if (PRUNED)
@@ -145,71 +151,164 @@ __global__ void __launch_bounds__(AT_THREADS) attention_kernel(const AttnArgs a)
                               ((reinterpret_cast<uintptr_t>(a.mask) & 7u) == 0);
         const bool qk_vec = SHAREDQK && ((a.seq_len & 3) == 0) &&
                             ((reinterpret_cast<uintptr_t>(a.QK) & 7u) == 0);
+        const float ls = a.log2_scale;
 
-        for (int kb = 0; kb < len; kb += AT_KT) {
-            __syncthreads(); // previous tile fully consumed
-            if (!SHAREDQK) { // stage K tile, row-major [key][d]
-                constexpr int CPR = HD / 8;
-                for (int idx = tid; idx < AT_KT * CPR; idx += AT_THREADS) {
+        // ---- key/value tile staging: global -> registers -> LDS.  The
+        // registers of tile t+1 are in flight while tile t is being consumed.
+        constexpr int CPR = HD / 8;                                        // 16-byte chunks per K row
+        constexpr int NKL = (AT_KT * CPR + AT_THREADS - 1) / AT_THREADS;   // K chunks per thread
+        constexpr int DQ = HD / 4;                                         // 4-wide column groups of V
+        constexpr int NVW = ((AT_KT / 4) * DQ + AT_THREADS - 1) / AT_THREADS; // V 4x4 blocks per thread
+        f16x8 kreg[NKL];
+        f16x4 vreg[NVW][4];
+        // FULL: every key of the tile is valid, so no per-lane bounds checks
+        auto load_tile = [&](int kb, auto full_c) {
+            constexpr bool FULL = decltype(full_c)::value;
+            if (!SHAREDQK) {
+#pragma unroll
+                for (int i = 0; i < NKL; i++) {
+                    const int idx = tid + i * AT_THREADS;
                     const int key = idx / CPR, dc = idx % CPR;
-                    f16x8 v = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-                    if (kb + key < len) {
+                    f16x8 v = zero8;
+                    if ((AT_KT * CPR % AT_THREADS == 0 || idx < AT_KT * CPR) && (FULL || kb + key < len)) {
                         const f16 *krow = a.K + (size_t)(row0 + kb + key) * a.ldq + qc0;
                         if (PRUNED)
                             v = load8_guard(krow, dc * 8, nqk);
                         else
                             v = *reinterpret_cast<const f16x8 *>(krow + dc * 8);
                     }
-                    *reinterpret_cast<f16x8 *>(ks + key * LDK + dc * 8) = v;
+                    kreg[i] = v;
                 }
             }
-            { // stage V tile transposed, [d][key]; rows at or beyond len as zeros
-                constexpr int DQ = HD / 4;
-                for (int w = tid; w < (AT_KT / 4) * DQ; w += AT_THREADS) {
-                    const int dq = w % DQ, kq = w / DQ;
-                    f16x4 r4[4];
 #pragma unroll
-                    for (int kk = 0; kk < 4; kk++) {
-                        const int key = kb + kq * 4 + kk;
-                        f16x4 v = f16x4{0, 0, 0, 0};
-                        if (key < len) {
-                            const f16 *vrow = a.V + (size_t)(row0 + key) * a.ldv + vc0;
-                            if (PRUNED) {
+            for (int i = 0; i < NVW; i++) {
+                const int w = tid + i * AT_THREADS;
+                const int dq = w % DQ, kq = w / DQ;
 #pragma unroll
-                                for (int e = 0; e < 4; e++)
-                                    v[e] = (dq * 4 + e < nv) ? vrow[dq * 4 + e] : (f16)0;
-                            } else {
-                                v = *reinterpret_cast<const f16x4 *>(vrow + dq * 4);
-                            }
+                for (int kk = 0; kk < 4; kk++) {
+                    const int key = kb + kq * 4 + kk;
+                    f16x4 v = f16x4{0, 0, 0, 0};
+                    if (((AT_KT / 4) * DQ % AT_THREADS == 0 || w < (AT_KT / 4) * DQ) &&
+                        (FULL || key < len)) { // rows at or beyond len read as zero
+                        const f16 *vrow = a.V + (size_t)(row0 + key) * a.ldv + vc0;
+                        if (PRUNED) {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                v[e] = (dq * 4 + e < nv) ? vrow[dq * 4 + e] : (f16)0;
+                        } else {
+                            v = *reinterpret_cast<const f16x4 *>(vrow + dq * 4);
                         }
-                        r4[kk] = v;
                     }
+                    vreg[i][kk] = v;
+                }
+            }
+        };
+        auto store_tile = [&](int buf) {
+            f16 *ks = smem + buf * (KBUF + VBUF);
+            f16 *vt = ks + KBUF;
+            if (!SHAREDQK) {
+#pragma unroll
+                for (int i = 0; i < NKL; i++) {
+                    const int idx = tid + i * AT_THREADS;
+                    const int key = idx / CPR, dc = idx % CPR;
+                    if (AT_KT * CPR % AT_THREADS == 0 || idx < AT_KT * CPR)
+                        *reinterpret_cast<f16x8 *>(ks + key * LDK + dc * 8) = kreg[i];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < NVW; i++) { // V goes in transposed: [d][key]
+                const int w = tid + i * AT_THREADS;
+                const int dq = w % DQ, kq = w / DQ;
+                if ((AT_KT / 4) * DQ % AT_THREADS == 0 || w < (AT_KT / 4) * DQ) {
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        const f16x4 t = f16x4{r4[0][e], r4[1][e], r4[2][e], r4[3][e]};
+                        const f16x4 t = f16x4{vreg[i][0][e], vreg[i][1][e], vreg[i][2][e], vreg[i][3][e]};
                         *reinterpret_cast<f16x4 *>(vt + (dq * 4 + e) * LDV + kq * 4) = t;
                     }
                 }
             }
-            __syncthreads();
+        };
+        typedef std::integral_constant<bool, true> yes_t;
+        typedef std::integral_constant<bool, false> no_t;
 
+        const int nt = (len + AT_KT - 1) / AT_KT;
+        // all of this wave's query rows valid?  (wave-uniform)
+        const bool wave_rows_ok = q0 + (wave + 1) * QS * 16 <= len;
+        if (AT_KT <= len)
+            load_tile(0, yes_t{});
+        else
+            load_tile(0, no_t{});
+        store_tile(0);
+        __syncthreads();
+
+        // Additive mask values of one tile, in the score layout.  They are
+        // requested one tile ahead (right after the previous tile consumed
+        // its own) so the L2 latency is covered by a whole tile of work.
+        f16x4 mk[QS][4];
+        auto load_mask = [&](int kb, auto fast_c) {
+            constexpr bool FAST = decltype(fast_c)::value;
+#pragma unroll
+            for (int qs = 0; qs < QS; qs++) {
+                const int q = q0 + (wave * QS + qs) * 16 + c16;
+#pragma unroll
+                for (int ksub = 0; ksub < 4; ksub++) {
+                    const int key = kb + ksub * 16 + g4 * 4;
+                    const f16 *mrow = a.mask + (size_t)q * a.seq_len + key;
+                    f16x4 v = f16x4{0, 0, 0, 0};
+                    if (FAST) {
+                        v = *reinterpret_cast<const f16x4 *>(mrow);
+                    } else if (q < len) {
+                        if (mask_vec && key + 3 < len) {
+                            v = *reinterpret_cast<const f16x4 *>(mrow);
+                        } else {
+#pragma unroll
+                            for (int r = 0; r < 4; r++)
+                                if (key + r < len)
+                                    v[r] = mrow[r];
+                        }
+                    }
+                    mk[qs][ksub] = v;
+                }
+            }
+        };
+        const bool vec_ok = (!a.mask || mask_vec) && (!SHAREDQK || qk_vec);
+        auto fast_tile = [&](int kb) { return kb + AT_KT <= len && wave_rows_ok && vec_ok; };
+        if (a.mask) {
+            if (fast_tile(0))
+                load_mask(0, yes_t{});
+            else
+                load_mask(0, no_t{});
+        }
+
+        // One key tile.  FAST: all 64 keys and all of the wave's query rows are
+        // valid and the vector paths apply, so the body has no per-lane
+        // predicates at all.
+        auto tile_body = [&](int kb, const f16 *ks, const f16 *vt, auto fast_c) {
+            constexpr bool FAST = decltype(fast_c)::value;
             // ---- scores, transposed: st[ksub][qs][r] = S[q = c16][key = 16 ksub + 4 g4 + r]
             f32x4 st[4][QS];
             if (!SHAREDQK) {
+                // all K fragments of the tile are requested from LDS first, then
+                // the MFMAs run with the dependent pair (s, s+1) eight issues apart
+                f16x8 kfr[4][DK];
 #pragma unroll
-                for (int ksub = 0; ksub < 4; ksub++) {
+                for (int ksub = 0; ksub < 4; ksub++)
+#pragma unroll
+                    for (int s = 0; s < DK; s++)
+                        kfr[ksub][s] = *reinterpret_cast<const f16x8 *>(
+                            ks + (ksub * 16 + c16) * LDK + s * 32 + g4 * 8);
+#pragma unroll
+                for (int ksub = 0; ksub < 4; ksub++)
 #pragma unroll
                     for (int qs = 0; qs < QS; qs++)
                         st[ksub][qs] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int s = 0; s < DK; s++) {
-                        const f16x8 kf = *reinterpret_cast<const f16x8 *>(
-                            ks + (ksub * 16 + c16) * LDK + s * 32 + g4 * 8);
+                for (int s = 0; s < DK; s++)
+#pragma unroll
+                    for (int ksub = 0; ksub < 4; ksub++)
 #pragma unroll
                         for (int qs = 0; qs < QS; qs++)
-                            st[ksub][qs] = mfma16x16x32(kf, qf[qs][s], st[ksub][qs]);
-                    }
-                }
+                            st[ksub][qs] = mfma16x16x32(kfr[ksub][s], qf[qs][s], st[ksub][qs]);
             } else {
 #pragma unroll
                 for (int qs = 0; qs < QS; qs++) {
@@ -218,105 +317,143 @@ __global__ void __launch_bounds__(AT_THREADS) attention_kernel(const AttnArgs a)
                     for (int ksub = 0; ksub < 4; ksub++) {
                         const int key = kb + ksub * 16 + g4 * 4;
                         f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
-                        if (q < len) {
-                            const f16 *src = a.QK + ((size_t)bh * a.seq_len + q) * a.seq_len + key;
-                            if (qk_vec && key + 3 < len) {
-                                const f16x4 t = *reinterpret_cast<const f16x4 *>(src);
+                        const f16 *src = a.QK + ((size_t)bh * a.seq_len + q) * a.seq_len + key;
+                        if (FAST || (q < len && qk_vec && key + 3 < len)) {
+                            const f16x4 t4 = *reinterpret_cast<const f16x4 *>(src);
 #pragma unroll
-                                for (int r = 0; r < 4; r++)
-                                    v[r] = (float)t[r];
-                            } else {
+                            for (int r = 0; r < 4; r++)
+                                v[r] = (float)t4[r];
+                        } else if (q < len) {
 #pragma unroll
-                                for (int r = 0; r < 4; r++)
-                                    if (key + r < len)
-                                        v[r] = (float)src[r];
-                            }
+                            for (int r = 0; r < 4; r++)
+                                if (key + r < len)
+                                    v[r] = (float)src[r];
                         }
                         st[ksub][qs] = v;
                     }
                 }
             }
 
-            // ---- mask, online softmax, pack P
+            // ---- mask, online softmax, pack P as the B operand.  The running
+            // maximum is only raised when a row's new maximum exceeds it by
+            // more than 8 binades (P then stays <= 256, exact enough in half),
+            // so after the first tiles the accumulator rescale is skipped.
             f16x8 pf[QS][2];
+            if (a.mask) {
+#pragma unroll
+                for (int qs = 0; qs < QS; qs++)
+#pragma unroll
+                    for (int ksub = 0; ksub < 4; ksub++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            st[ksub][qs][r] += (float)mk[qs][ksub][r];
+                if (kb + AT_KT < len) { // next tile's mask
+                    if (fast_tile(kb + AT_KT))
+                        load_mask(kb + AT_KT, yes_t{});
+                    else
+                        load_mask(kb + AT_KT, no_t{});
+                }
+            }
 #pragma unroll
             for (int qs = 0; qs < QS; qs++) {
-                const int q = q0 + (wave * QS + qs) * 16 + c16;
+                if (!FAST) {
+#pragma unroll
+                    for (int ksub = 0; ksub < 4; ksub++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            if (kb + ksub * 16 + g4 * 4 + r >= len)
+                                st[ksub][qs][r] = -INFINITY;
+                }
                 float mx = -INFINITY;
 #pragma unroll
                 for (int ksub = 0; ksub < 4; ksub++) {
-                    const int key = kb + ksub * 16 + g4 * 4;
-                    float mk[4] = {0.f, 0.f, 0.f, 0.f};
-                    if (a.mask && q < len) {
-                        const f16 *mrow = a.mask + (size_t)q * a.seq_len + key;
-                        if (mask_vec && key + 3 < len) {
-                            const f16x4 t = *reinterpret_cast<const f16x4 *>(mrow);
-#pragma unroll
-                            for (int r = 0; r < 4; r++)
-                                mk[r] = (float)t[r];
-                        } else {
-#pragma unroll
-                            for (int r = 0; r < 4; r++)
-                                if (key + r < len)
-                                    mk[r] = (float)mrow[r];
-                        }
-                    }
-#pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        float s = (st[ksub][qs][r] + mk[r]) * a.log2_scale;
-                        if (key + r >= len)
-                            s = -INFINITY;
-                        st[ksub][qs][r] = s;
-                        mx = fmaxf(mx, s);
-                    }
+                    mx = fmaxf(fmaxf(mx, st[ksub][qs][0]), st[ksub][qs][1]);
+                    mx = fmaxf(fmaxf(mx, st[ksub][qs][2]), st[ksub][qs][3]);
                 }
                 mx = xor_max_16_32(mx);
-                const float m_new = fmaxf(m_run[qs], mx);
-                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-                const float alpha = __builtin_amdgcn_exp2f(m_run[qs] - m_use);
-                m_run[qs] = m_new;
+                const bool up = (mx - m_run[qs]) * ls > 8.0f; // also true for the first valid tile (m_run = -inf)
+                if (__builtin_amdgcn_ballot_w64(up) != 0) {
+                    const float m_new = up ? mx : m_run[qs];
+                    const float m_fin = (m_new == -INFINITY) ? 0.f : m_new;
+                    const float alpha = __builtin_amdgcn_exp2f((m_run[qs] - m_fin) * ls); // 1 where unchanged
+                    m_run[qs] = m_new;
+                    l_run[qs] *= alpha;
+#pragma unroll
+                    for (int d = 0; d < DV; d++)
+                        ot[d][qs] *= alpha;
+                }
+                const float msc = ((m_run[qs] == -INFINITY) ? 0.f : m_run[qs]) * ls;
                 float psum = 0.f;
-                f16 ph[16];
+                f16x2 ph[8];
 #pragma unroll
                 for (int ksub = 0; ksub < 4; ksub++)
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        const float p = __builtin_amdgcn_exp2f(st[ksub][qs][r] - m_use);
-                        psum += p;
-                        ph[ksub * 4 + r] = (f16)p;
+                    for (int r2 = 0; r2 < 2; r2++) {
+                        float p0 = __builtin_fmaf(st[ksub][qs][2 * r2], ls, -msc);
+                        float p1 = __builtin_fmaf(st[ksub][qs][2 * r2 + 1], ls, -msc);
+                        p0 = __builtin_amdgcn_exp2f(p0);
+                        p1 = __builtin_amdgcn_exp2f(p1);
+                        psum += p0 + p1;
+                        typedef float f32x2 __attribute__((ext_vector_type(2)));
+                        ph[ksub * 2 + r2] = __builtin_convertvector(f32x2{p0, p1}, f16x2);
                     }
-                l_run[qs] = l_run[qs] * alpha + psum;
-#pragma unroll
-                for (int d = 0; d < DV; d++)
-                    ot[d][qs] *= alpha;
+                l_run[qs] += psum;
 #pragma unroll
                 for (int kk = 0; kk < 2; kk++)
-                    pf[qs][kk] = f16x8{ph[kk * 8 + 0], ph[kk * 8 + 1], ph[kk * 8 + 2], ph[kk * 8 + 3],
-                                       ph[kk * 8 + 4], ph[kk * 8 + 5], ph[kk * 8 + 6], ph[kk * 8 + 7]};
+                    pf[qs][kk] = f16x8{ph[kk * 4 + 0][0], ph[kk * 4 + 0][1], ph[kk * 4 + 1][0], ph[kk * 4 + 1][1],
+                                       ph[kk * 4 + 2][0], ph[kk * 4 + 2][1], ph[kk * 4 + 3][0], ph[kk * 4 + 3][1]};
             }
 
-            // ---- O^T += V^T P^T
+            // ---- O^T += V^T P^T, same ordering: all V^T fragments first
+            {
+                f16x8 vfr[DV][2];
 #pragma unroll
-            for (int d = 0; d < DV; d++) {
+                for (int d = 0; d < DV; d++)
 #pragma unroll
-                for (int kk = 0; kk < 2; kk++) {
-                    const f16 *vrow = vt + (d * 16 + c16) * LDV + kk * 32 + g4 * 4;
-                    const f16x4 v0 = *reinterpret_cast<const f16x4 *>(vrow);
-                    const f16x4 v1 = *reinterpret_cast<const f16x4 *>(vrow + 16);
-                    const f16x8 vf = f16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                    for (int kk = 0; kk < 2; kk++) {
+                        const f16 *vrow = vt + (d * 16 + c16) * LDV + kk * 32 + g4 * 4;
+                        const f16x4 v0 = *reinterpret_cast<const f16x4 *>(vrow);
+                        const f16x4 v1 = *reinterpret_cast<const f16x4 *>(vrow + 16);
+                        vfr[d][kk] = f16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                    }
 #pragma unroll
-                    for (int qs = 0; qs < QS; qs++)
-                        ot[d][qs] = mfma16x16x32(vf, pf[qs][kk], ot[d][qs]);
-                }
+                for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                    for (int d = 0; d < DV; d++)
+#pragma unroll
+                        for (int qs = 0; qs < QS; qs++)
+                            ot[d][qs] = mfma16x16x32(vfr[d][kk], pf[qs][kk], ot[d][qs]);
             }
+        };
+
+        for (int t = 0; t < nt; t++) {
+            const int kb = t * AT_KT;
+            const f16 *ks = smem + (t & 1) * (KBUF + VBUF);
+            const f16 *vt = ks + KBUF;
+            const bool more = t + 1 < nt;
+            if (more) { // tile t+1: global loads in flight while tile t is consumed
+                if (kb + 2 * AT_KT <= len)
+                    load_tile(kb + AT_KT, yes_t{});
+                else
+                    load_tile(kb + AT_KT, no_t{});
+            }
+            if (fast_tile(kb))
+                tile_body(kb, ks, vt, yes_t{});
+            else
+                tile_body(kb, ks, vt, no_t{});
+            // publish tile t+1 into the other buffer (last read in iteration
+            // t-1, which every wave left before the previous barrier)
+            if (more)
+                store_tile((t + 1) & 1);
+            __syncthreads();
         }
 
-        // ---- normalise and stage the output block in LDS
-        __syncthreads();
+        // ---- normalise and stage the output block in LDS (all waves are past
+        // the loop's final barrier, so the tile buffers are free)
         f16 *os = smem;
         if (PRUNED) { // columns that no kept V column maps to must read as zero
             for (int i = tid; i < SM_O / 8; i += AT_THREADS)
-                reinterpret_cast<f16x8 *>(os)[i] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                reinterpret_cast<f16x8 *>(os)[i] = zero8;
             __syncthreads();
         }
 #pragma unroll
@@ -348,12 +485,11 @@ __global__ void __launch_bounds__(AT_THREADS) attention_kernel(const AttnArgs a)
             }
         }
         __syncthreads();
-        constexpr int CPR = HD / 8;
         for (int idx = tid; idx < QB * CPR; idx += AT_THREADS) {
             const int ql = idx / CPR, dc = idx % CPR;
             const int q = q0 + ql;
             if (q < rows_alloc) {
-                f16x8 v = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                f16x8 v = zero8;
                 if (q < len)
                     v = *reinterpret_cast<const f16x8 *>(os + ql * LDO + dc * 8);
                 *reinterpret_cast<f16x8 *>(obase + (size_t)q * a.ldo + dc * 8) = v;
@@ -366,8 +502,7 @@ __global__ void __launch_bounds__(AT_THREADS) attention_kernel(const AttnArgs a)
             const int ql = idx / CPR, dc = idx % CPR;
             const int q = q0 + ql;
             if (q < rows_alloc)
-                *reinterpret_cast<f16x8 *>(obase + (size_t)q * a.ldo + dc * 8) =
-                    f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                *reinterpret_cast<f16x8 *>(obase + (size_t)q * a.ldo + dc * 8) = zero8;
         }
     }
 }
@@ -416,15 +551,40 @@ qk_scores_kernel(f16 *__restrict__ QK, const f16 *__restrict__ Q, const f16 *__r
     }
 }
 
-template <int HD, bool PRUNED, bool SHAREDQK>
-static void attn_launch_qs(int qs, const AttnArgs &a, hipStream_t st) {
-    if (qs == 2)
-        hipLaunchKernelGGL((attention_kernel<HD, 2, PRUNED, SHAREDQK>), dim3(a.per_xcd * 8),
-                           dim3(AT_THREADS), 0, st, a);
-    else
-        hipLaunchKernelGGL((attention_kernel<HD, 1, PRUNED, SHAREDQK>), dim3(a.per_xcd * 8),
-                           dim3(AT_THREADS), 0, st, a);
+// LDS bytes of one workgroup (mirrors the constants inside the kernel)
+template <int HD, int QS, int NW> constexpr size_t attn_lds_bytes() {
+    constexpr int KV = 2 * (AT_KT * (HD + 16) + HD * (AT_KT + 8));
+    constexpr int O = NW * 16 * QS * (HD + 8);
+    return sizeof(f16) * (size_t)(KV > O ? KV : O);
 }
+
+template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK>
+static void attn_launch_one(const AttnArgs &a, hipStream_t st) {
+    constexpr size_t lds = attn_lds_bytes<HD, QS, NW>();
+    auto kern = attention_kernel<HD, QS, NW, PRUNED, SHAREDQK>;
+    if (lds > 64 * 1024) { // above the default dynamic-LDS limit: opt in once per kernel
+        static bool done = false;
+        if (!done) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            done = true;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3(a.per_xcd * 8), dim3(NW * 64), lds, st, a);
+}
+
+// variant 0: 4 waves x 32 query rows; 1: 8 waves x 16 rows; 2: 4 waves x 16 rows
+template <int HD, bool PRUNED, bool SHAREDQK>
+static void attn_launch_variant(int variant, const AttnArgs &a, hipStream_t st) {
+    if (variant == 0)
+        attn_launch_one<HD, 2, 4, PRUNED, SHAREDQK>(a, st);
+    else if (variant == 1)
+        attn_launch_one<HD, 1, 8, PRUNED, SHAREDQK>(a, st);
+    else
+        attn_launch_one<HD, 1, 4, PRUNED, SHAREDQK>(a, st);
+}
+
+static int g_attn_variant = -1; // et_tuning_set("attn_variant"): -1 = automatic
 
 static float head_scale(int hd) {
     // half(sqrt(1/head_dim)), kernels/attention.cu:126
@@ -449,22 +609,26 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
     }
     a.ldo = d_model;
     a.scale = head_scale(hd);
-    // queries per workgroup: 128 when that still fills the chip, else 64
-    int qs = 2;
+    // 128 query rows per workgroup when that still fills the chip, else 64
+    int variant = 0;
     {
         const long wg128 = (long)((a.seq_len + 127) / 128) * a.nhead * a.batch;
-        if (wg128 < 512 || hd == 128)
-            qs = 1;
+        if (wg128 < 512)
+            variant = 2;
+        if (hd == 128)
+            variant = 2;
+        if (g_attn_variant >= 0 && g_attn_variant <= 2 && !(hd == 128 && g_attn_variant == 0))
+            variant = g_attn_variant;
     }
-    const int QB = AT_WAVES * 16 * qs;
+    const int QB = variant == 2 ? 64 : 128;
     a.nqb = (a.seq_len + QB - 1) / QB;
     a.total = a.nqb * a.nhead * a.batch;
     a.per_xcd = (a.total + 7) / 8;
 #define ET_ATTN_CASE(HDV)                                                                         \
     if (hd == HDV) {                                                                              \
-        if (sharedqk) attn_launch_qs<HDV, false, true>(qs, a, st);                                \
-        else if (pruned) attn_launch_qs<HDV, true, false>(qs, a, st);                             \
-        else attn_launch_qs<HDV, false, false>(qs, a, st);                                        \
+        if (sharedqk) attn_launch_variant<HDV, false, true>(variant, a, st);                                \
+        else if (pruned) attn_launch_variant<HDV, true, false>(variant, a, st);                             \
+        else attn_launch_variant<HDV, false, false>(variant, a, st);                                        \
     }
     ET_ATTN_CASE(32)
     ET_ATTN_CASE(64)
@@ -472,6 +636,8 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
 #undef ET_ATTN_CASE
     return launch_status(who);
 }
+
+void set_attn_variant(int v) { g_attn_variant = v; }
 
 } // namespace et
 

@@ -33,6 +33,8 @@
 
 namespace et {
 
+void set_attn_variant(int v);
+
 constexpr int TL_THREADS = 512;
 constexpr int TL_WAVES = 8;
 constexpr int TL_BM = 32;
@@ -71,7 +73,7 @@ struct TlArgs {
     const f16 *bias[TL_MAX_LIN];
     int N[TL_MAX_LIN];
     const f16 *X;
-    int nlin, M, K, KC, nchunk, ncg, total, per_xcd, dbg;
+    int nlin, M, K, KC, nchunk, ncg, total, per_xcd;
 };
 #define TL_SEL(f) (lin == 0 ? a.f[0] : lin == 1 ? a.f[1] : lin == 2 ? a.f[2] : a.f[3])
 
@@ -97,7 +99,7 @@ __device__ __forceinline__ bool tl_context(const TlArgs &a, int nb, TlCtx &x) {
     // Workgroups that share a row panel of X get consecutive ids on ONE XCD
     // (hardware round-robins consecutive workgroup ids over the 8 XCDs), so
     // the panel is fetched into that XCD's L2 once.
-    const int pid = (a.dbg & 64) ? (int)blockIdx.x : (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3);
+    const int pid = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3);
     if (pid >= a.total)
         return false;
     const int per_rp = a.ncg * a.nlin;
@@ -150,7 +152,7 @@ __device__ __forceinline__ void tl_epilogue(const TlArgs &a, const TlCtx &x, f16
     const int col0 = x.bn_wg * 16;
     const int wcols = min(BNW, N - col0);
     const int cpr = wcols >> 3;
-    if (x.m0 + x.ld_r < a.M && !(a.dbg & 2)) {
+    if (x.m0 + x.ld_r < a.M) {
         u32x4 *dst = reinterpret_cast<u32x4 *>(Y + (size_t)(x.m0 + x.ld_r) * N + col0);
         const u32x4 *src = reinterpret_cast<const u32x4 *>(ys + x.ld_r * ldy);
         for (int cc = x.ld_c; cc < cpr; cc += 16)
@@ -196,7 +198,7 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
     }
     const char *xlane = reinterpret_cast<const char *>(xs + x.c16 * x.ldx + x.khalf8);
     const int xrow16 = 16 * x.ldx * 2; // bytes between the two 16-row subtiles
-    const bool rowok = (x.m0 + x.ld_r) < a.M && !(a.dbg & 1);
+    const bool rowok = (x.m0 + x.ld_r) < a.M;
     const u32x4 *xsrc = reinterpret_cast<const u32x4 *>(a.X + (size_t)(x.m0 + x.ld_r) * a.K);
     u32x4 *xdst = reinterpret_cast<u32x4 *>(xs + x.ld_r * x.ldx);
 
@@ -250,7 +252,7 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
         // the first four pairs of the stream: requested before the barrier so
         // that their latency overlaps the wait for the other waves
         const int q0 = __builtin_amdgcn_readfirstlane(bvec);
-        const int qend = (a.dbg & 4) ? q0 : __builtin_amdgcn_readlane(bvec, NB);
+        const int qend = __builtin_amdgcn_readlane(bvec, NB);
         const int qlast = max(qend - 1, q0);
         f16x8 w0 = zero8, w1 = zero8, w2 = zero8, w3 = zero8;
         int o0 = 0, o1 = 0, o2 = 0, o3 = 0;
@@ -464,7 +466,6 @@ static void launch_nb(int nb, const TlArgs &a, size_t lds, hipStream_t st) {
 // Tuning knobs (et_tuning_set): 0 = automatic.
 static int g_tile_nb = 0;
 static int g_tile_min_wgs = 512;
-static int g_tile_dbg = 0;
 
 // Block-rows per wave.  Measured on the BERT-base shapes (rows 4096..8192):
 // three block-rows per wave is the best trade between panel re-reads (fewer
@@ -507,7 +508,6 @@ static int tile_launch(const TlProblem *probs, int nlin, const f16 *X, int M, in
     a.K = K;
     a.KC = KC;
     a.nchunk = nchunk;
-    a.dbg = g_tile_dbg;
     const int nrp = (M + TL_BM - 1) / TL_BM;
     const int nb = choose_nb(nrp, nbr_max, nlin);
     a.ncg = (nbr_max + TL_WAVES * nb - 1) / (TL_WAVES * nb);
@@ -578,8 +578,8 @@ extern "C" int et_tuning_set(const char *key, int value) {
         et::g_tile_min_wgs = value;
         return ET_OK;
     }
-    if (key && !strcmp(key, "tile_dbg")) {
-        et::g_tile_dbg = value;
+    if (key && !strcmp(key, "attn_variant")) {
+        et::set_attn_variant(value);
         return ET_OK;
     }
     et::set_error("et_tuning_set: unknown key");

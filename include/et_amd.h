@@ -218,7 +218,9 @@ int et_device_synchronize(void);
 /* Launch-heuristic overrides for benchmarking sweeps; value 0 restores the
  * automatic choice.  Keys: "tile_nb" (block-rows of W per wave in the tile
  * linear: 1,2,3,4,6), "tile_min_wgs" (workgroups the automatic choice aims
- * for).  Not thread-safe; results never depend on these. */
+ * for), "attn_variant" (0: 4 waves x 32 query rows, 1: 8 waves x 16 rows,
+ * 2: 4 waves x 16 rows; -1 automatic).  Not thread-safe; results never depend
+ * on these beyond fp32 summation order. */
 int et_tuning_set(const char *key, int value);
 /* number of compute units of the current device (0 if none) */
 int et_device_cu_count(void);
