@@ -33,6 +33,19 @@ MFMA_F16_PEAK_TF = 2500.0   # MI355X dense fp16 MFMA, published
 
 D, H, DFF = 768, 12, 3072
 
+# HBM bytes per launch (fetch + write, MiB) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the
+# default workload and scaled by the 64 MiB copy kernel launched below; commands and raw figures are in
+# profiles/encoder_layer_b16_s512_hbm_traffic.txt.  Only valid for batch 16 x seq 512 at 80 % sparsity.
+MEASURED_TRAFFIC_MIB = {
+    "tile_linear qkv (3 x 768->768, one launch)": 17.91 + 36.00,
+    "attention (on-the-fly)": 40.35 + 12.00,
+    "tile_linear o (768->768)": 14.04 + 12.00,
+    "skip_layernorm 1": 24.04 + 12.00,
+    "tile_linear ffn1+gelu (768->3072)": 19.84 + 48.00,
+    "tile_linear ffn2 (3072->768)": 55.78 + 12.00,
+    "skip_layernorm 2": 24.04 + 12.00,
+}
+
 
 def tile_bytes(T, N, K, ntile):
     return 2 * T * K + 512 * ntile + 4 * ntile + 4 * (N // 16 + 1) + 2 * N + 2 * T * N
@@ -90,6 +103,16 @@ def main():
     enc = Encoder_tile(D, S, H, ws, *mk_linears(), *ln, mask_h, B)
     out = torch.empty_like(x)
 
+    # ---- a plain copy kernel of known size (64 MiB read + 64 MiB written):
+    # the reference that rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled against
+    from et_amd._lib import check, lib
+    cal_src = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+    cal_dst = torch.empty_like(cal_src)
+    cal_src.zero_()
+    check(lib().et_copy(cal_dst.data_ptr(), cal_src.data_ptr(), cal_src.numel(), torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    del cal_src, cal_dst
+
     # ---- whole layer: W warm-up steps, then exactly K timed steps
     for _ in range(args.warmup):
         enc.run(out, x)
@@ -141,13 +164,19 @@ def main():
                      "GBps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                      "TFLOPs": round(flops / us / 1e6, 1), "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TF, 4),
                      "bound": bound})
+    default_cfg = (B, S, args.sparsity) == (16, 512, 0.8)
+    for k in kern:
+        mib = MEASURED_TRAFFIC_MIB.get(k["kernel"]) if default_cfg else None
+        k["traffic_MB"] = None if mib is None else round(mib * 1.048576, 2)
     dom = max(kern, key=lambda k: k["us"])
     if dom["bound"] == "hbm":
         roof = {"kernel": dom["kernel"], "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": dom["hbm_frac"], "traffic": None, "mfma_frac": dom["mfma_frac"]}
+                "frac": dom["hbm_frac"], "traffic": dom["traffic_MB"], "traffic_unit": "MB/launch",
+                "mfma_frac": dom["mfma_frac"]}
     else:
         roof = {"kernel": dom["kernel"], "bound": "mfma", "achieved": dom["TFLOPs"], "peak": MFMA_F16_PEAK_TF,
-                "unit": "TFLOP/s", "frac": dom["mfma_frac"], "traffic": None, "hbm_frac": dom["hbm_frac"]}
+                "unit": "TFLOP/s", "frac": dom["mfma_frac"], "traffic": dom["traffic_MB"],
+                "traffic_unit": "MB/launch", "hbm_frac": dom["hbm_frac"]}
     layer_flops = sum(k["GFLOP"] for k in kern)
     total_us = sum(k["us"] for k in kern)
 

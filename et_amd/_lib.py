@@ -69,6 +69,7 @@ PROTOTYPES = {
     "et_memcpy_d2h": (_i, [_vp, _vp, _sz]),
     "et_memcpy_d2d_async": (_i, [_vp, _vp, _sz, _vp]),
     "et_fill_zero": (_i, [_vp, _sz, _vp]),
+    "et_copy": (_i, [_vp, _vp, _sz, _vp]),
     "et_stream_create": (_i, [C.POINTER(_vp)]),
     "et_stream_destroy": (_i, [_vp]),
     "et_stream_synchronize": (_i, [_vp]),

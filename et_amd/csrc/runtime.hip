@@ -68,6 +68,14 @@ scatter_cols_kernel(f16 *__restrict__ out, const f16 *__restrict__ in,
     }
 }
 
+// plain streaming copy, 16 bytes per lane; also the known-size reference that
+// hardware traffic counters are scaled against
+__global__ void __launch_bounds__(256) copy_kernel(u32x4 *__restrict__ dst, const u32x4 *__restrict__ src, size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16;
+         i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+
 __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t nwords) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nwords;
          i += (size_t)gridDim.x * blockDim.x)
@@ -131,6 +139,19 @@ int et_fill_zero(void *dst, size_t bytes, void *stream) {
     hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<uint32_t *>(dst), nw);
     return launch_status("et_fill_zero");
+}
+int et_copy(void *dst, const void *src, size_t bytes, void *stream) {
+    using namespace et;
+    ET_REQUIRE((dst && src) || bytes == 0, ET_ERR_INVALID_ARG, "et_copy: null pointer");
+    ET_REQUIRE(bytes % 16 == 0 && aligned16(dst) && aligned16(src), ET_ERR_ALIGNMENT,
+               "et_copy: needs 16-byte granularity");
+    if (!bytes)
+        return ET_OK;
+    const size_t n16 = bytes / 16;
+    const int grid = (int)std::min<size_t>((n16 + 255) / 256, 16384);
+    hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<u32x4 *>(dst), static_cast<const u32x4 *>(src), n16);
+    return launch_status("et_copy");
 }
 int et_stream_create(void **stream) {
     ET_REQUIRE(stream, ET_ERR_INVALID_ARG, "et_stream_create: null out pointer");

@@ -211,6 +211,10 @@ int et_memcpy_h2d(void *dst, const void *src, size_t bytes);
 int et_memcpy_d2h(void *dst, const void *src, size_t bytes);
 int et_memcpy_d2d_async(void *dst, const void *src, size_t bytes, void *stream);
 int et_fill_zero(void *dst, size_t bytes, void *stream);
+/* plain device-to-device copy KERNEL (16-byte granularity); unlike a runtime
+ * memcpy it always shows up as a kernel dispatch, which makes it the
+ * known-size reference for scaling hardware traffic counters */
+int et_copy(void *dst, const void *src, size_t bytes, void *stream);
 int et_stream_create(void **stream);
 int et_stream_destroy(void *stream);
 int et_stream_synchronize(void *stream);

@@ -1,0 +1,99 @@
+"""CPU-only checks of the shipped library: the C ABI loads and exports every
+symbol the headers declare, the host-side format code is bit-identical to the
+oracle's independent restatement, and argument validation fails cleanly
+(negative codes, no exit) before anything touches a device."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import oracle.et_oracle as orc
+from et_amd import _lib, formats
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    names = []
+    for hdr in ("et_amd.h", "et_encoder.h"):
+        text = open(os.path.join(ROOT, "include", hdr)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names += re.findall(r"\b(et_[A-Za-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = C.CDLL(_lib.LIB_PATH)
+    syms = declared_symbols()
+    assert len(syms) >= 50
+    missing = [s for s in syms if not hasattr(lib, s)]
+    assert not missing, missing
+    # and the Python binding covers the same set
+    assert set(_lib.PROTOTYPES) == set(syms)
+    assert _lib.lib().et_abi_version() == 1
+
+
+@pytest.mark.parametrize("N,K,sp", [(768, 768, 0.8), (3072, 768, 0.5), (768, 3072, 0.9), (64, 96, 0.33), (16, 16, 0.0), (32, 32, 1.0)])
+def test_tile_mat_generator_bit_exact_vs_oracle(N, K, sp):
+    for seed in (0, 1, 12345678901234567):
+        a = formats.gen_sparse_tile_mat(N, K, sp, seed)
+        b = orc.gen_sparse_tile_mat(N, K, sp, seed)
+        assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+        assert formats.tile_mat_validate(N, K, a[0], a[1]) == 0
+
+
+def test_row_mat_and_head_ptr_bit_exact_vs_oracle():
+    for nrow, sp in ((768, 0.7), (3072, 0.5), (768, 0.0), (100, 0.99)):
+        assert np.array_equal(formats.gen_sparse_row_mat(nrow, sp, 9), orc.gen_sparse_row_mat(nrow, sp, 9))
+    ids = formats.gen_sparse_row_mat(768, 0.7, 3)
+    assert np.array_equal(formats.head_ptr(ids, 12, 64), orc.head_ptr(ids, 12, 64))
+    assert np.array_equal(formats.gen_head_balanced_rows(12, 64, 32, 5), orc.gen_head_balanced_rows(12, 64, 32, 5))
+
+
+def test_tile_pack_byte_identical_vs_oracle():
+    r = np.random.default_rng(4)
+    W = r.standard_normal((96, 160)).astype(np.float16)
+    rp, ro = formats.gen_sparse_tile_mat(96, 160, 0.6, 8)
+    assert np.array_equal(formats.tile_pack(W, rp, ro).view(np.uint16), orc.tile_pack(W, rp, ro).view(np.uint16))
+
+
+def test_validate_codes_match_oracle():
+    rp, ro = formats.gen_sparse_tile_mat(64, 64, 0.5, 1)
+    cases = []
+    bad = ro.copy(); bad[0] += 8; cases.append((64, 64, rp, bad))
+    bad = ro.copy(); bad[0] = 64; cases.append((64, 64, rp, bad))
+    bad = rp.copy(); bad[-1] += 1; cases.append((64, 64, bad, ro))
+    bad = rp.copy(); bad[0] = 1; cases.append((64, 64, bad, ro))
+    cases.append((60, 64, rp, ro))
+    for N, K, p, o in cases:
+        got, want = formats.tile_mat_validate(N, K, p, o), orc.tile_mat_validate(N, K, p, o)
+        assert got == want and got < 0
+
+
+def test_argument_errors_return_codes_without_a_device():
+    l = _lib.lib()
+    # null pointers / bad sizes are rejected before any HIP call
+    assert l.et_skip_layernorm(None, None, None, None, 4, 768, None) == -1
+    assert l.et_tile_spmm_add_bias(None, None, None, None, None, 16, 16, 16, None, None) == -1
+    assert l.et_OTF_attention(None, None, None, None, None, 128, 768, 12, 1, None, 1.0, None) == -1
+    assert l.et_row_spmm_add_bias(None, None, None, None, 16, 16, 16, None) == -1
+    buf = (C.c_uint16 * 64)()
+    p = C.addressof(buf)
+    assert l.et_tile_spmm_add_bias(p, p, p, p, p, 16, 24, 16, p, None) == -3          # N not a multiple of 16
+    assert l.et_OTF_attention(p, p, p, p, None, 128, 768, 7, 1, None, 1.0, None) == -1  # d_model % nhead
+    assert l.et_OTF_attention(p, p, p, p, None, 128, 96, 2, 1, None, 1.0, None) == -3   # head_dim 48 unsupported
+    assert b"head_dim" in l.et_last_error()
+    assert l.et_strerror(-3) == b"unsupported shape"
+    with pytest.raises(_lib.EtError):
+        formats.gen_sparse_tile_mat(100, 64, 0.5, 1)     # nrow not a multiple of 16
+    with pytest.raises(_lib.EtError):
+        formats.gen_sparse_row_mat(64, 1.5, 1)
+    # malformed tile_mat is refused at plan construction (ET_ERR_FORMAT), no device needed
+    rp, ro = formats.gen_sparse_tile_mat(32, 32, 0.0, 1)
+    bad = ro.copy(); bad[0] = 5
+    data = np.zeros(ro.size * 256, np.float16); bias = np.zeros(32, np.float16)
+    h = C.c_void_p()
+    rc = l.et_tile_plan_create(C.byref(h), 32, 32, int(ro.size), data.ctypes.data, rp.ctypes.data, bad.ctypes.data, bias.ctypes.data)
+    assert rc == -5 and not h.value
