@@ -60,6 +60,16 @@ __device__ __forceinline__ f32x4 mfma16x16x32(f16x8 a, f16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 
+// 16 bytes per lane straight from global memory into LDS
+// (global_load_lds_dwordx4): lane L of the wave writes at lds_base + 16*L;
+// lds_base must be wave-uniform, the source address is free per lane.
+// Completion is tracked by vmcnt.
+__device__ __forceinline__ void load_lds16(const void *gsrc, void *lds_base) {
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void *)gsrc,
+        (__attribute__((address_space(3))) void *)lds_base, 16, 0, 0);
+}
+
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
 
 // ---- wave64 reductions (all lanes receive the result) -----------------------

@@ -198,22 +198,26 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
     }
     const char *xlane = reinterpret_cast<const char *>(xs + x.c16 * x.ldx + x.khalf8);
     const int xrow16 = 16 * x.ldx * 2; // bytes between the two 16-row subtiles
-    const bool rowok = (x.m0 + x.ld_r) < a.M;
-    const u32x4 *xsrc = reinterpret_cast<const u32x4 *>(a.X + (size_t)(x.m0 + x.ld_r) * a.K);
-    u32x4 *xdst = reinterpret_cast<u32x4 *>(xs + x.ld_r * x.ldx);
-
-    // global -> register half of the panel staging: all of a thread's loads
-    // are in flight together
-    u32x4 pv[8];
+    // X panel staging: global -> LDS directly (global_load_lds_dwordx4: lane L
+    // of the issuing wave writes 16 bytes at  base + 16*L, the source address is
+    // free per lane).  Wave w fills panel rows 4w..4w+3, each row as one 64-lane
+    // and one partial instruction; no VGPRs are held and nothing waits until the
+    // barrier.  Rows at or beyond M are left unwritten: a panel row only feeds
+    // the output row of the same index, which is never stored.
 #define TL_PANEL_LOAD(c_)                                                                         \
     {                                                                                             \
         const int pk0 = (c_) * a.KC;                                                              \
-        const int pcpr = min(a.KC, a.K - pk0) >> 3;                                               \
-        _Pragma("unroll") for (int u = 0; u < 8; u++) {                                           \
-            const int cc = x.ld_c + 16 * u;                                                       \
-            pv[u] = u32x4{0u, 0u, 0u, 0u};                                                        \
-            if (rowok && cc < pcpr)                                                               \
-                pv[u] = xsrc[(pk0 >> 3) + cc];                                                    \
+        const int pcpr = min(a.KC, a.K - pk0) >> 3; /* 16-byte chunks per row, <= 124 */          \
+        _Pragma("unroll") for (int rr = 0; rr < 4; rr++) {                                        \
+            const int row = x.wave * 4 + rr;                                                      \
+            if (x.m0 + row < a.M) {                                                               \
+                const f16 *src = a.X + (size_t)(x.m0 + row) * a.K + pk0;                          \
+                f16 *dstrow = xs + row * x.ldx;                                                   \
+                if (lane < pcpr)                                                                  \
+                    load_lds16(src + lane * 8, dstrow);                                           \
+                if (64 + lane < pcpr)                                                             \
+                    load_lds16(src + (64 + lane) * 8, dstrow + 512);                              \
+            }                                                                                     \
         }                                                                                         \
     }
     TL_PANEL_LOAD(0)
@@ -230,7 +234,6 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
     const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
 
     for (int c = 0; c < a.nchunk; c++) {
-        const int kc = min(a.KC, a.K - c * a.KC);
         // pair-index boundaries of the wave's block-rows: lane j holds the end
         // of block-row j (read back with v_readlane)
         const int bidx = c * nbr + min(x.bn0 + min(lane, NB), nbr);
@@ -239,15 +242,6 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
         if (c > 0) {
             __syncthreads(); // every wave is done with the previous panel
             TL_PANEL_LOAD(c)
-        }
-        {
-            const int cpr = kc >> 3;
-#pragma unroll
-            for (int u = 0; u < 8; u++) {
-                const int cc = x.ld_c + 16 * u;
-                if (cc < cpr)
-                    xdst[cc] = pv[u];
-            }
         }
         // the first four pairs of the stream: requested before the barrier so
         // that their latency overlaps the wait for the other waves
@@ -267,6 +261,9 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
             o3 = obase[qd * 2];
             w3 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qd * 512);
         }
+        // the panel (and, with it, the first pairs) must have landed before
+        // any wave reads LDS
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
         __syncthreads();
 
         if (q0 < qend) {
@@ -277,8 +274,6 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
                 j++;
                 bend = __builtin_amdgcn_readlane(bvec, j + 1);
             }
-            // drain once here so that inside the loop the waits can be counted
-            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
             // X operands are read one stage ahead (ping-pong xa0/xb0 <-> xa1/xb1)
             f16x8 xa0 = *reinterpret_cast<const f16x8 *>(xlane + o0);
             f16x8 xb0 = *reinterpret_cast<const f16x8 *>(xlane + o0 + xrow16);
