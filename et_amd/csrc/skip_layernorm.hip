@@ -10,59 +10,87 @@
 
 namespace et {
 
-// One wave per row; the row is held as NCH chunks of 8 halves per lane.
-template <int NCH>
+// One wave handles ROWS consecutive rows, one after the other; a row is held
+// as NCH chunks of 8 halves per lane.  The next row's loads are issued before
+// the current row is reduced, so every wave keeps reads in flight while it
+// computes and stores (with one row per wave the whole grid is resident at
+// once and all waves read, then all waves write).
+template <int NCH, int ROWS>
 __global__ void __launch_bounds__(256)
 skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip,
                           const f16 *__restrict__ gamma,
                           const f16 *__restrict__ beta, int num, int size) {
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
-    const long row = (long)blockIdx.x * 4 + wave;
-    if (row >= num)
+    const long row0 = ((long)blockIdx.x * 4 + wave) * ROWS;
+    if (row0 >= num)
         return;
     const int nchunk = size >> 3;
-    f16x8 *a = reinterpret_cast<f16x8 *>(in_out + row * size);
-    const f16x8 *s = reinterpret_cast<const f16x8 *>(skip + row * size);
     const f16x8 *g = reinterpret_cast<const f16x8 *>(gamma);
     const f16x8 *b = reinterpret_cast<const f16x8 *>(beta);
+    const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
 
-    f16x8 x[NCH];
-    float sum = 0.f;
+    f16x8 an[NCH], sn[NCH]; // next row, raw
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
         const int c = lane + i * 64;
+        an[i] = zero8;
+        sn[i] = zero8;
         if (c < nchunk) {
-            x[i] = a[c] + __builtin_nontemporal_load(&s[c]); // half add, one rounding
-#pragma unroll
-            for (int j = 0; j < 8; j++)
-                sum += (float)x[i][j];
+            an[i] = reinterpret_cast<const f16x8 *>(in_out + row0 * size)[c];
+            sn[i] = reinterpret_cast<const f16x8 *>(skip + row0 * size)[c];
         }
     }
-    const float mean = wave_sum(sum) / (float)size;
-    float var = 0.f;
 #pragma unroll
-    for (int i = 0; i < NCH; i++) {
-        const int c = lane + i * 64;
-        if (c < nchunk) {
+    for (int r = 0; r < ROWS; r++) {
+        const long row = row0 + r;
+        if (row >= num)
+            break;
+        f16x8 x[NCH];
+        float sum = 0.f;
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const float d = (float)x[i][j] - mean;
-                var += d * d;
+        for (int i = 0; i < NCH; i++) {
+            x[i] = an[i] + sn[i]; // half add, one rounding (kernels/skip_layernorm.cu:20)
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                sum += (float)x[i][j]; // chunks beyond the row are zero
+        }
+        if (r + 1 < ROWS && row + 1 < num) {
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                const int c = lane + i * 64;
+                if (c < nchunk) {
+                    an[i] = reinterpret_cast<const f16x8 *>(in_out + (row + 1) * size)[c];
+                    sn[i] = reinterpret_cast<const f16x8 *>(skip + (row + 1) * size)[c];
+                }
             }
         }
-    }
-    const float rstd = rsqrtf(wave_sum(var) / (float)size + 1e-6f);
+        const float mean = wave_sum(sum) / (float)size;
+        float var = 0.f;
 #pragma unroll
-    for (int i = 0; i < NCH; i++) {
-        const int c = lane + i * 64;
-        if (c < nchunk) {
-            const f16x8 gg = g[c], bb = b[c];
-            f16x8 y;
+        for (int i = 0; i < NCH; i++) {
+            const int c = lane + i * 64;
+            if (c < nchunk) {
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-                y[j] = (f16)(((float)x[i][j] - mean) * rstd * (float)gg[j] + (float)bb[j]);
-            a[c] = y;
+                for (int j = 0; j < 8; j++) {
+                    const float d = (float)x[i][j] - mean;
+                    var += d * d;
+                }
+            }
+        }
+        const float rstd = rsqrtf(wave_sum(var) / (float)size + 1e-6f);
+        f16x8 *a = reinterpret_cast<f16x8 *>(in_out + row * size);
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int c = lane + i * 64;
+            if (c < nchunk) {
+                const f16x8 gg = g[c], bb = b[c];
+                f16x8 y;
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    y[j] = (f16)(((float)x[i][j] - mean) * rstd * (float)gg[j] + (float)bb[j]);
+                a[c] = y;
+            }
         }
     }
 }
@@ -96,6 +124,9 @@ skip_layernorm_generic_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ 
         a[c] = (f16)(((float)a[c] - mean) * rstd * (float)gamma[c] + (float)beta[c]);
 }
 
+int g_ln_rows = 0; // et_tuning_set("ln_rows"): 0 = automatic
+void set_ln_rows(int v) { g_ln_rows = v; }
+
 } // namespace et
 
 extern "C" int et_skip_layernorm(void *in_out, const void *skip, const void *gamma,
@@ -112,21 +143,28 @@ extern "C" int et_skip_layernorm(void *in_out, const void *skip, const void *gam
     const f16 *s = static_cast<const f16 *>(skip);
     const f16 *g = static_cast<const f16 *>(gamma);
     const f16 *b = static_cast<const f16 *>(beta);
-    const dim3 grid((num + 3) / 4), block(256);
+    const dim3 block(256);
     const bool vec = (size % 8 == 0) && size <= 4096 && aligned16(in_out) &&
                      aligned16(skip) && aligned16(gamma) && aligned16(beta);
     if (!vec) {
-        hipLaunchKernelGGL(skip_layernorm_generic_kernel, grid, block, 0, st, a, s, g, b, num, size);
+        hipLaunchKernelGGL(skip_layernorm_generic_kernel, dim3((num + 3) / 4), block, 0, st, a, s, g, b, num, size);
     } else {
         const int nch = (size / 8 + 63) / 64;
-        if (nch <= 1)
-            hipLaunchKernelGGL(skip_layernorm_vec_kernel<1>, grid, block, 0, st, a, s, g, b, num, size);
-        else if (nch <= 2)
-            hipLaunchKernelGGL(skip_layernorm_vec_kernel<2>, grid, block, 0, st, a, s, g, b, num, size);
-        else if (nch <= 4)
-            hipLaunchKernelGGL(skip_layernorm_vec_kernel<4>, grid, block, 0, st, a, s, g, b, num, size);
-        else
-            hipLaunchKernelGGL(skip_layernorm_vec_kernel<8>, grid, block, 0, st, a, s, g, b, num, size);
+        // rows per wave: enough waves to fill the chip first (256 CUs x 32 waves)
+        const int rows = g_ln_rows > 0 ? g_ln_rows : (num >= 4 * 8192 ? 4 : num >= 2 * 8192 ? 2 : 1);
+        const dim3 grid((num + 4 * rows - 1) / (4 * rows));
+#define ET_LN_CASE(NCH_)                                                                          \
+    if (rows >= 4)                                                                                \
+        hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 4>), grid, block, 0, st, a, s, g, b, num, size); \
+    else if (rows >= 2)                                                                           \
+        hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 2>), grid, block, 0, st, a, s, g, b, num, size); \
+    else                                                                                          \
+        hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 1>), grid, block, 0, st, a, s, g, b, num, size);
+        if (nch <= 1) { ET_LN_CASE(1) }
+        else if (nch <= 2) { ET_LN_CASE(2) }
+        else if (nch <= 4) { ET_LN_CASE(4) }
+        else { ET_LN_CASE(8) }
+#undef ET_LN_CASE
     }
     return launch_status("et_skip_layernorm launch");
 }

@@ -34,6 +34,7 @@
 namespace et {
 
 void set_attn_variant(int v);
+void set_ln_rows(int v);
 
 constexpr int TL_THREADS = 512;
 constexpr int TL_WAVES = 8;
@@ -157,6 +158,48 @@ __device__ __forceinline__ void tl_epilogue(const TlArgs &a, const TlCtx &x, f16
         const u32x4 *src = reinterpret_cast<const u32x4 *>(ys + x.ld_r * ldy);
         for (int cc = x.ld_c; cc < cpr; cc += 16)
             dst[cc] = src[cc];
+    }
+}
+
+// Per-wave epilogue: bias (+GELU), round to half, transpose through a
+// wave-private LDS tile (32 rows x 16*NB columns, no barrier: a wave's LDS
+// operations execute in order), then 16-byte stores of 32*NB contiguous bytes
+// per row.  Waves never wait for each other here, so one wave's stores overlap
+// the other waves' MFMAs.
+template <int NB> constexpr int tl_wave_stage_halves() { return TL_BM * (16 * NB + 8); }
+
+template <int NB, bool GELU>
+__device__ __forceinline__ void tl_epilogue_wave(const TlArgs &a, const TlCtx &x, f16 *stage, f16 *Y,
+                                                 int N, int nbr, const f32x4 (&acc)[NB][2],
+                                                 const f16x4 (&b4)[NB]) {
+    constexpr int lds = 16 * NB + 8; // halves per staged row
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+#pragma unroll
+        for (int ms = 0; ms < 2; ms++) {
+            f16x4 o;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const f16 v = (f16)(acc[j][ms][r] + (float)b4[j][r]);
+                o[r] = GELU ? gelu_h(v) : v;
+            }
+            *reinterpret_cast<f16x4 *>(stage + (ms * 16 + x.c16) * lds + j * 16 + x.g4 * 4) = o;
+        }
+    }
+    // valid block-rows of this wave (the last column group may be partial)
+    const int nvalid = min(NB, nbr - x.bn0);
+    if (nvalid <= 0)
+        return;
+    const int cpr = 2 * nvalid; // 16-byte chunks per row
+    f16 *ybase = Y + (size_t)x.m0 * N + x.bn0 * 16;
+#pragma unroll
+    for (int t = 0; t < NB; t++) {
+        const int i = x.lane + 64 * t;
+        const int r = i / (2 * NB), c = i - r * (2 * NB);
+        if (c < cpr && x.m0 + r < a.M) {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + r * lds + c * 8);
+            *reinterpret_cast<u32x4 *>(ybase + (size_t)r * N + c * 8) = v;
+        }
     }
 }
 
@@ -324,7 +367,8 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
         }
     }
 #undef TL_PANEL_LOAD
-    tl_epilogue<NB, GELU>(a, x, xs, Yp, N, nbr, acc, b4);
+    f16 *stage = xs + TL_BM * x.ldx + x.wave * tl_wave_stage_halves<NB>();
+    tl_epilogue_wave<NB, GELU>(a, x, stage, Yp, N, nbr, acc, b4);
 }
 
 // ---------------------------------------------------------------------------
@@ -510,7 +554,11 @@ static int tile_launch(const TlProblem *probs, int nlin, const f16 *X, int M, in
     a.per_xcd = (a.total + 7) / 8;
     const size_t lds_x = (size_t)TL_BM * (KC + ((KC & 31) ? 0 : TL_PAD)) * sizeof(f16);
     const size_t lds_y = (size_t)TL_BM * (TL_WAVES * nb * 16 + TL_PAD) * sizeof(f16);
-    const size_t lds = std::max(lds_x, lds_y);
+    // plan kernel: panel + one private staging tile per wave; generic kernel:
+    // the output tile reuses the panel's storage
+    const size_t lds = mode == TL_PLAN
+                           ? lds_x + (size_t)TL_WAVES * TL_BM * (16 * nb + 8) * sizeof(f16)
+                           : std::max(lds_x, lds_y);
     if (mode == TL_PLAN) {
         if (gelu) launch_nb<true, TL_PLAN>(nb, a, lds, st);
         else launch_nb<false, TL_PLAN>(nb, a, lds, st);
@@ -571,6 +619,10 @@ extern "C" int et_tuning_set(const char *key, int value) {
     }
     if (key && !strcmp(key, "tile_min_wgs")) {
         et::g_tile_min_wgs = value;
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "ln_rows")) {
+        et::set_ln_rows(value);
         return ET_OK;
     }
     if (key && !strcmp(key, "attn_variant")) {
