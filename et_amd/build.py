@@ -37,7 +37,7 @@ def build(verbose: bool = False) -> str:
             continue
         obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
         cmd = [hipcc(), "-x", "hip", "-c", path, "-o", obj, "-I", os.path.join(HERE, "..", "include"),
-               "-I", HERE] + HIP_FLAGS
+               "-I", HERE] + HIP_FLAGS + os.environ.get("ET_AMD_EXTRA_HIPFLAGS", "").split()
         if verbose:
             print(" ".join(cmd))
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

@@ -75,6 +75,7 @@ struct TlArgs {
     int N[TL_MAX_LIN];
     const f16 *X;
     int nlin, M, K, KC, nchunk, ncg, total, per_xcd;
+    int ipw; // plan kernel: consecutive work items per (persistent) workgroup
 };
 #define TL_SEL(f) (lin == 0 ? a.f[0] : lin == 1 ? a.f[1] : lin == 2 ? a.f[2] : a.f[3])
 
@@ -204,43 +205,64 @@ __device__ __forceinline__ void tl_epilogue_wave(const TlArgs &a, const TlCtx &x
 }
 
 // ---------------------------------------------------------------------------
-// Plan kernel (the fast path).  Because a wave owns NB CONSECUTIVE block-rows
-// and the plan stores tiles in (chunk, block-row) order with even segments,
-// the wave's work for a chunk is ONE contiguous stream of tile pairs: 1 KB of
-// W per pair at an address that is linear in the pair index, plus one int per
-// half-wave giving the LDS byte offset of that tile's X columns.  The stream
-// is consumed through a fixed 4-stage register pipeline (stage = pair index
-// mod 4), every load unconditional with a clamped address, so four pairs are
-// always in flight per wave and the waits are counted, not drained.  Products
-// accumulate into one running 32x16 accumulator; when the stream crosses a
-// block-row boundary (a scalar compare per pair) it is added into that
-// block-row's static accumulator.
+// Plan kernel (the fast path).
+//
+// Work items are (row panel, linear, column group) triples, numbered with the
+// row panel slowest.  A workgroup is persistent over `ipw` consecutive items:
+// as long as the row panel does not change (and K fits one chunk) the X panel
+// stays in LDS, so it is fetched once for several column groups, and because
+// every wave stages its output through a private LDS tile the waves never
+// meet at a barrier between items - one wave's stores overlap the others'
+// MFMAs and the next item's weight loads.
+//
+// Within an item a wave owns NB CONSECUTIVE block-rows, and the plan stores
+// tiles in (chunk, block-row) order with even segments, so the wave's work for
+// a chunk is ONE contiguous stream of tile pairs: 1 KB of W per pair at an
+// address that is linear in the pair index, plus one int per half-wave giving
+// the LDS byte offset of that tile's X columns.  The stream is consumed
+// through a fixed 4-stage register pipeline (stage = pair index mod 4), every
+// load unconditional with a clamped address, so four pairs are always in
+// flight per wave and the waits are counted, not drained.  Products accumulate
+// into one running 32x16 accumulator; when the stream crosses a block-row
+// boundary (a scalar compare per pair) it is added into that block-row's
+// static accumulator.
 // ---------------------------------------------------------------------------
+#ifdef TL_TRACE
+__device__ unsigned long long *g_trace = nullptr; // per wave: start, panel, compute, epilogue ticks, HW ids
+#define TL_TICK() __builtin_readcyclecounter()
+#endif
+
 template <int NB, bool GELU>
 __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
     f16 *xs = reinterpret_cast<f16 *>(tl_smem);
-    TlCtx x;
-    if (!tl_context(a, NB, x))
+    // Workgroups with consecutive virtual ids run on ONE XCD (hardware
+    // round-robins consecutive workgroup ids over the 8 XCDs), so the column
+    // groups of a row panel that do not fit one workgroup share that XCD's L2.
+    const int vid = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3);
+    const int it0 = vid * a.ipw;
+    const int it1 = min(it0 + a.ipw, a.total);
+    if (it0 >= it1)
         return;
-    const int lin = x.lin;
-    f16 *const Yp = TL_SEL(Y);
-    const int *const cptr = TL_SEL(cptr);
-    const int *const poff = TL_SEL(row_offset); // LDS byte offset per tile (chunk-local column * 2)
-    const f16 *const data = TL_SEL(data);
-    const f16 *const bias = TL_SEL(bias);
-    const int N = TL_SEL(N);
-    const int nbr = N >> 4;
+    TlCtx x;
+    x.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    x.lane = threadIdx.x & 63;
+    x.c16 = x.lane & 15;
+    x.g4 = x.lane >> 4;
+    x.khalf8 = (x.g4 & 1) * 8;
+    x.hi = x.lane >> 5;
+    x.ldx = a.KC + ((a.KC & 31) ? 0 : TL_PAD);
     const int hi = x.hi, lane = x.lane;
-
-    f32x4 acc[NB][2];
-#pragma unroll
-    for (int j = 0; j < NB; j++) {
-        acc[j][0] = f32x4{0.f, 0.f, 0.f, 0.f};
-        acc[j][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
     const char *xlane = reinterpret_cast<const char *>(xs + x.c16 * x.ldx + x.khalf8);
     const int xrow16 = 16 * x.ldx * 2; // bytes between the two 16-row subtiles
+    f16 *const stage = xs + TL_BM * x.ldx + x.wave * tl_wave_stage_halves<NB>();
+    const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    const int per_rp = a.ncg * a.nlin;
+#ifdef TL_TRACE
+    const unsigned long long tt0 = TL_TICK();
+    unsigned long long tpanel = 0, tcomp = 0, tepi = 0, tlast = tt0, tgap = 0;
+#endif
+
     // X panel staging: global -> LDS directly (global_load_lds_dwordx4: lane L
     // of the issuing wave writes 16 bytes at  base + 16*L, the source address is
     // free per lane).  Wave w fills panel rows 4w..4w+3, each row as one 64-lane
@@ -263,64 +285,99 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
             }                                                                                     \
         }                                                                                         \
     }
-    TL_PANEL_LOAD(0)
 
-    f16x4 b4[NB];
+    int panel_rp = -1; // row panel currently in LDS (single-chunk problems only)
+    bool lds_used = false;
+    for (int it = it0; it < it1; it++) {
+        const int rp = it / per_rp;
+        const int rest = it - rp * per_rp;
+        const int lin = rest / a.ncg;
+        x.lin = lin;
+        x.cg = rest - lin * a.ncg;
+        x.m0 = rp * TL_BM;
+        x.bn_wg = x.cg * (TL_WAVES * NB);
+        x.bn0 = x.bn_wg + x.wave * NB;
+        f16 *const Yp = TL_SEL(Y);
+        const int *const cptr = TL_SEL(cptr);
+        const int *const poff = TL_SEL(row_offset); // LDS byte offset per tile (chunk-local column * 2)
+        const f16 *const data = TL_SEL(data);
+        const f16 *const bias = TL_SEL(bias);
+        const int N = TL_SEL(N);
+        const int nbr = N >> 4;
+
+        f32x4 acc[NB][2];
+        f16x4 b4[NB];
 #pragma unroll
-    for (int j = 0; j < NB; j++) {
-        b4[j] = f16x4{0, 0, 0, 0};
-        if (x.bn0 + j < nbr)
-            b4[j] = *reinterpret_cast<const f16x4 *>(bias + (x.bn0 + j) * 16 + x.g4 * 4);
-    }
-    const f16 *wbase = data + hi * 256 + x.c16 * 16 + x.khalf8; // + pair * 512
-    const int *obase = poff + hi;                               // + pair * 2
-    const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-
-    for (int c = 0; c < a.nchunk; c++) {
-        // pair-index boundaries of the wave's block-rows: lane j holds the end
-        // of block-row j (read back with v_readlane)
-        const int bidx = c * nbr + min(x.bn0 + min(lane, NB), nbr);
-        const int bvec = cptr[bidx] >> 1;
-
-        if (c > 0) {
-            __syncthreads(); // every wave is done with the previous panel
-            TL_PANEL_LOAD(c)
+        for (int j = 0; j < NB; j++) {
+            acc[j][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+            acc[j][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+            b4[j] = f16x4{0, 0, 0, 0};
+            if (x.bn0 + j < nbr)
+                b4[j] = *reinterpret_cast<const f16x4 *>(bias + (x.bn0 + j) * 16 + x.g4 * 4);
         }
-        // the first four pairs of the stream: requested before the barrier so
-        // that their latency overlaps the wait for the other waves
-        const int q0 = __builtin_amdgcn_readfirstlane(bvec);
-        const int qend = __builtin_amdgcn_readlane(bvec, NB);
-        const int qlast = max(qend - 1, q0);
-        f16x8 w0 = zero8, w1 = zero8, w2 = zero8, w3 = zero8;
-        int o0 = 0, o1 = 0, o2 = 0, o3 = 0;
-        if (q0 < qend) {
-            const int qa = q0, qb = min(q0 + 1, qlast), qc = min(q0 + 2, qlast), qd = min(q0 + 3, qlast);
-            o0 = obase[qa * 2];
-            w0 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qa * 512);
-            o1 = obase[qb * 2];
-            w1 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qb * 512);
-            o2 = obase[qc * 2];
-            w2 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qc * 512);
-            o3 = obase[qd * 2];
-            w3 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qd * 512);
-        }
-        // the panel (and, with it, the first pairs) must have landed before
-        // any wave reads LDS
-        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
-        __syncthreads();
+        const f16 *wbase = data + hi * 256 + x.c16 * 16 + x.khalf8; // + pair * 512
+        const int *obase = poff + hi;                               // + pair * 2
 
-        if (q0 < qend) {
-            f32x4 cur0 = f32x4{0.f, 0.f, 0.f, 0.f}, cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
-            int j = 0;
-            int bend = __builtin_amdgcn_readlane(bvec, 1);
-            while (bend == q0 && j + 1 < NB) { // leading empty block-rows
-                j++;
-                bend = __builtin_amdgcn_readlane(bvec, j + 1);
+        for (int c = 0; c < a.nchunk; c++) {
+#ifdef TL_TRACE
+            const unsigned long long ta = TL_TICK();
+            tgap += ta - tlast;
+#endif
+            // pair-index boundaries of the wave's block-rows: lane j holds the end
+            // of block-row j (read back with v_readlane)
+            const int bidx = c * nbr + min(x.bn0 + min(lane, NB), nbr);
+            const int bvec = cptr[bidx] >> 1;
+
+            const bool reload = a.nchunk > 1 || rp != panel_rp; // workgroup-uniform
+            if (reload) {
+                // (The load, its wait and both barriers stay in this one block:
+                // with the wait further down, behind the first weight loads,
+                // the compiler loses track of the DMA and drains every load in
+                // the pipelined loop below instead of counting.)
+                if (lds_used)
+                    __syncthreads(); // every wave is done with the previous panel
+                TL_PANEL_LOAD(c)
+                lds_used = true;
+                __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's part has landed
+                __syncthreads();                    // ... and everyone else's
             }
-            // X operands are read one stage ahead (ping-pong xa0/xb0 <-> xa1/xb1)
-            f16x8 xa0 = *reinterpret_cast<const f16x8 *>(xlane + o0);
-            f16x8 xb0 = *reinterpret_cast<const f16x8 *>(xlane + o0 + xrow16);
-            f16x8 xa1 = zero8, xb1 = zero8;
+            // the first four pairs of the stream
+            const int q0 = __builtin_amdgcn_readfirstlane(bvec);
+            const int qend = __builtin_amdgcn_readlane(bvec, NB);
+            const int qlast = max(qend - 1, q0);
+            f16x8 w0 = zero8, w1 = zero8, w2 = zero8, w3 = zero8;
+            int o0 = 0, o1 = 0, o2 = 0, o3 = 0;
+            if (q0 < qend) {
+                const int qa = q0, qb = min(q0 + 1, qlast), qc = min(q0 + 2, qlast), qd = min(q0 + 3, qlast);
+                o0 = obase[qa * 2];
+                w0 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qa * 512);
+                o1 = obase[qb * 2];
+                w1 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qb * 512);
+                o2 = obase[qc * 2];
+                w2 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qc * 512);
+                o3 = obase[qd * 2];
+                w3 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qd * 512);
+            }
+#ifdef TL_TRACE
+            const unsigned long long tb = TL_TICK();
+            tpanel += tb - ta;
+#endif
+
+            if (q0 < qend) {
+                f32x4 cur0 = f32x4{0.f, 0.f, 0.f, 0.f}, cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
+                int j = 0;
+                int bend = __builtin_amdgcn_readlane(bvec, 1);
+                // leading empty block-rows (straight-line scalar code: loops
+                // in here would defeat the counted waits of the pipeline)
+#pragma unroll
+                for (int t = 0; t < NB - 1; t++) {
+                    j += (bend == q0 && j + 1 < NB) ? 1 : 0;
+                    bend = __builtin_amdgcn_readlane(bvec, j + 1);
+                }
+                // X operands are read one stage ahead (ping-pong xa0/xb0 <-> xa1/xb1)
+                f16x8 xa0 = *reinterpret_cast<const f16x8 *>(xlane + o0);
+                f16x8 xb0 = *reinterpret_cast<const f16x8 *>(xlane + o0 + xrow16);
+                f16x8 xa1 = zero8, xb1 = zero8;
 #define TL_STAGE(W_, O_, ONEXT_, XA_, XB_, XAN_, XBN_, I_)                                        \
     {                                                                                             \
         XAN_ = *reinterpret_cast<const f16x8 *>(xlane + ONEXT_);                                  \
@@ -342,33 +399,56 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
             }                                                                                     \
             cur0 = f32x4{0.f, 0.f, 0.f, 0.f};                                                     \
             cur1 = f32x4{0.f, 0.f, 0.f, 0.f};                                                     \
-            do {                                                                                  \
-                j++;                                                                              \
+            j++;                                                                                  \
+            bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));                               \
+            _Pragma("unroll") for (int t = 0; t < NB - 2; t++) { /* skip empty block-rows */      \
+                j += (bend == q + (I_) + 1 && j + 1 < NB) ? 1 : 0;                                \
                 bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));                           \
-            } while (bend == q + (I_) + 1 && j + 1 < NB);                                         \
+            }                                                                                     \
         }                                                                                         \
     }
-            int q = q0;
-            for (; q + 4 <= qend; q += 4) { // straight-line body: counted waits
-                TL_STAGE(w0, o0, o1, xa0, xb0, xa1, xb1, 0)
-                TL_STAGE(w1, o1, o2, xa1, xb1, xa0, xb0, 1)
-                TL_STAGE(w2, o2, o3, xa0, xb0, xa1, xb1, 2)
-                TL_STAGE(w3, o3, o0, xa1, xb1, xa0, xb0, 3)
-            }
-            if (q < qend) {
-                TL_STAGE(w0, o0, o1, xa0, xb0, xa1, xb1, 0)
-                if (q + 1 < qend) {
+                int q = q0;
+                for (; q + 4 <= qend; q += 4) { // straight-line body: counted waits
+                    TL_STAGE(w0, o0, o1, xa0, xb0, xa1, xb1, 0)
                     TL_STAGE(w1, o1, o2, xa1, xb1, xa0, xb0, 1)
-                    if (q + 2 < qend)
-                        TL_STAGE(w2, o2, o3, xa0, xb0, xa1, xb1, 2)
+                    TL_STAGE(w2, o2, o3, xa0, xb0, xa1, xb1, 2)
+                    TL_STAGE(w3, o3, o0, xa1, xb1, xa0, xb0, 3)
                 }
-            }
+                if (q < qend) {
+                    TL_STAGE(w0, o0, o1, xa0, xb0, xa1, xb1, 0)
+                    if (q + 1 < qend) {
+                        TL_STAGE(w1, o1, o2, xa1, xb1, xa0, xb0, 1)
+                        if (q + 2 < qend)
+                            TL_STAGE(w2, o2, o3, xa0, xb0, xa1, xb1, 2)
+                    }
+                }
 #undef TL_STAGE
+            }
+#ifdef TL_TRACE
+            tlast = TL_TICK();
+            tcomp += tlast - tb;
+#endif
         }
+        panel_rp = a.nchunk > 1 ? -1 : rp;
+#ifdef TL_TRACE
+        const unsigned long long te = TL_TICK();
+#endif
+        tl_epilogue_wave<NB, GELU>(a, x, stage, Yp, N, nbr, acc, b4);
+#ifdef TL_TRACE
+        tlast = TL_TICK();
+        tepi += tlast - te;
+#endif
     }
 #undef TL_PANEL_LOAD
-    f16 *stage = xs + TL_BM * x.ldx + x.wave * tl_wave_stage_halves<NB>();
-    tl_epilogue_wave<NB, GELU>(a, x, stage, Yp, N, nbr, acc, b4);
+#ifdef TL_TRACE
+    if (g_trace && lane == 0) {
+        unsigned hwid, xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        unsigned long long *t = g_trace + ((size_t)blockIdx.x * TL_WAVES + x.wave) * 8;
+        t[0] = tt0; t[1] = tpanel; t[2] = tcomp; t[3] = tepi; t[4] = TL_TICK(); t[5] = hwid; t[6] = xcc; t[7] = tgap;
+    }
+#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -505,6 +585,7 @@ static void launch_nb(int nb, const TlArgs &a, size_t lds, hipStream_t st) {
 // Tuning knobs (et_tuning_set): 0 = automatic.
 static int g_tile_nb = 0;
 static int g_tile_min_wgs = 512;
+static int g_tile_ipw = 0;
 
 // Block-rows per wave.  Measured on the BERT-base shapes (rows 4096..8192):
 // three block-rows per wave is the best trade between panel re-reads (fewer
@@ -551,7 +632,20 @@ static int tile_launch(const TlProblem *probs, int nlin, const f16 *X, int M, in
     const int nb = choose_nb(nrp, nbr_max, nlin);
     a.ncg = (nbr_max + TL_WAVES * nb - 1) / (TL_WAVES * nb);
     a.total = nrp * a.ncg * nlin;
-    a.per_xcd = (a.total + 7) / 8;
+    a.ipw = 1;
+    if (mode == TL_PLAN && nchunk == 1) {
+        // persistent workgroups: as many items of one row panel per workgroup
+        // as still leaves every CU its share of workgroups
+        const int per_rp = a.ncg * nlin;
+        for (int d = per_rp; d > 1; d--)
+            if (per_rp % d == 0 && a.total / d >= g_tile_min_wgs) {
+                a.ipw = d;
+                break;
+            }
+        if (g_tile_ipw > 0)
+            a.ipw = g_tile_ipw;
+    }
+    a.per_xcd = ((a.total + a.ipw - 1) / a.ipw + 7) / 8;
     const size_t lds_x = (size_t)TL_BM * (KC + ((KC & 31) ? 0 : TL_PAD)) * sizeof(f16);
     const size_t lds_y = (size_t)TL_BM * (TL_WAVES * nb * 16 + TL_PAD) * sizeof(f16);
     // plan kernel: panel + one private staging tile per wave; generic kernel:
@@ -615,6 +709,10 @@ static int raw_tile_linear(void *Y, const void *X, const int *row_ptr, const int
 extern "C" int et_tuning_set(const char *key, int value) {
     if (key && !strcmp(key, "tile_nb")) {
         et::g_tile_nb = value;
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "tile_ipw")) {
+        et::g_tile_ipw = value;
         return ET_OK;
     }
     if (key && !strcmp(key, "tile_min_wgs")) {
@@ -826,3 +924,11 @@ extern "C" int et_tile_plan_run(const et_tile_plan *plan, void *Y, const void *X
     return tile_launch(&pr, 1, static_cast<const f16 *>(X), M, plan->in_feat, plan->KC,
                        plan->nchunk, gelu != 0, TL_PLAN, static_cast<hipStream_t>(stream));
 }
+
+#ifdef TL_TRACE
+// profiling builds only: per-wave phase tick counters are written to `buf`
+// (8 x u64 per wave, indexed by hardware workgroup id)
+extern "C" int et_debug_trace(void *buf) {
+    return hipMemcpyToSymbol(HIP_SYMBOL(et::g_trace), &buf, sizeof(buf)) == hipSuccess ? 0 : -1;
+}
+#endif
