@@ -452,6 +452,315 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
 }
 
 // ---------------------------------------------------------------------------
+// Resident-panel kernel: the plan kernel for K that fits one LDS panel (every
+// BERT-base linear except FFN2).  Same tile stream and 4-stage pipeline as
+// above, with three differences that take work off the critical path of a
+// wave:
+//  * a finished block-row is converted (bias, GELU, half) and written to the
+//    wave's staging tile right where the stream crosses its boundary, so there
+//    are no per-block-row accumulators to fold into and the conversion work
+//    overlaps the weight loads already in flight;
+//  * the next item's block-row boundaries and bias are requested before the
+//    current item's stream starts, and its first four weight pairs before the
+//    current item's output tile is stored - a wave sees one memory latency per
+//    item instead of three;
+//  * items that share the row panel reuse it without any barrier.
+// ---------------------------------------------------------------------------
+struct TlItem {
+    int rp, lin, cg, bn0, nbr, N;
+    f16 *Y;
+    const int *cptr;
+    const int *poff;
+    const f16 *data;
+    const f16 *bias;
+};
+
+// GELU of four halves: x^3 in (packed) half, the sigmoid form of
+// 0.5(1+tanh u) = 1/(1+exp(-2u)) in fp32, rounded to half, times x in half
+// (kernels/linear.cu:36-48).
+__device__ __forceinline__ f16x4 gelu4(f16x4 v) {
+    const f16x4 x2 = v * v;
+    const f16x4 x3 = v * x2;
+    f32x4 t;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const float s = __builtin_fmaf(0.044715f, (float)x3[r], (float)v[r]);
+        const float e = __builtin_amdgcn_exp2f(s * (-1.5957691216057308f * 1.4426950408889634f));
+        t[r] = __builtin_amdgcn_rcpf(1.0f + e);
+    }
+    return v * __builtin_convertvector(t, f16x4);
+}
+
+// one finished 32x16 block-row tile -> wave-private staging tile
+template <bool GELU>
+__device__ __forceinline__ void tl_stage_tile(f16 *dst, int lds, f32x4 c0, f32x4 c1, f16x4 bj) {
+    const f32x4 bf = __builtin_convertvector(bj, f32x4);
+    f16x4 o0 = __builtin_convertvector(c0 + bf, f16x4);
+    f16x4 o1 = __builtin_convertvector(c1 + bf, f16x4);
+    if (GELU) {
+        o0 = gelu4(o0);
+        o1 = gelu4(o1);
+    }
+    *reinterpret_cast<f16x4 *>(dst) = o0;
+    *reinterpret_cast<f16x4 *>(dst + 16 * lds) = o1;
+}
+
+template <int NB, bool GELU>
+__global__ void __launch_bounds__(TL_THREADS) tile_linear_resident_kernel(const TlArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
+    f16 *xs = reinterpret_cast<f16 *>(tl_smem);
+    const int vid = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3); // see tile_linear_plan_kernel
+    const int it0 = vid * a.ipw;
+    const int it1 = min(it0 + a.ipw, a.total);
+    if (it0 >= it1)
+        return;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int c16 = lane & 15, g4 = lane >> 4, khalf8 = (g4 & 1) * 8, hi = lane >> 5;
+    const int ldx = a.KC + ((a.KC & 31) ? 0 : TL_PAD);
+    const char *xlane = reinterpret_cast<const char *>(xs + c16 * ldx + khalf8);
+    const int xrow16 = 16 * ldx * 2; // bytes between the two 16-row subtiles
+    constexpr int lds = 16 * NB + 8; // halves per staged row
+    f16 *const stage = xs + TL_BM * ldx + wave * tl_wave_stage_halves<NB>();
+    f16 *const stage_lane = stage + c16 * lds + g4 * 4;
+    const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    const int lane_w = hi * 256 + c16 * 16 + khalf8; // lane's halves inside a 1 KB tile pair
+
+    // pair-index boundaries of a wave's block-rows: lane j holds the start of
+    // block-row j, lane NB the end of the last one (read back with v_readlane)
+#define TL_BVEC(t_) ((t_).cptr[min((t_).bn0 + min(lane, NB), (t_).nbr)] >> 1)
+    // (block-rows beyond the matrix read the last block-row's bias; their
+    // output is never stored)
+#define TL_BIAS(dst_, t_)                                                                         \
+    _Pragma("unroll") for (int k = 0; k < NB; k++)                                                \
+        dst_[k] = *reinterpret_cast<const f16x4 *>(                                               \
+            (t_).bias + min((t_).bn0 + k, (t_).nbr - 1) * 16 + g4 * 4);
+    // wave w fills panel rows 4w..4w+3 (see tile_linear_plan_kernel)
+#define TL_PANEL(rp_)                                                                             \
+    {                                                                                             \
+        const int pcpr = a.K >> 3;                                                                \
+        _Pragma("unroll") for (int rr = 0; rr < 4; rr++) {                                        \
+            const int row = (rp_) * TL_BM + wave * 4 + rr;                                        \
+            if (row < a.M) {                                                                      \
+                const f16 *src = a.X + (size_t)row * a.K;                                         \
+                f16 *dstrow = xs + (wave * 4 + rr) * ldx;                                         \
+                if (lane < pcpr)                                                                  \
+                    load_lds16(src + lane * 8, dstrow);                                           \
+                if (64 + lane < pcpr)                                                             \
+                    load_lds16(src + (64 + lane) * 8, dstrow + 512);                              \
+            }                                                                                     \
+        }                                                                                         \
+        __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): this wave's part has landed */           \
+        __syncthreads();                    /* ... and everyone else's */                         \
+    }
+    // the first four pairs of an item's stream
+#define TL_PRELOAD(t_, bvec_)                                                                     \
+    {                                                                                             \
+        q0 = __builtin_amdgcn_readfirstlane(bvec_);                                               \
+        qend = __builtin_amdgcn_readlane(bvec_, NB);                                              \
+        qlast = max(qend - 1, q0);                                                                \
+        wbase = (t_).data + lane_w;                                                               \
+        obase = (t_).poff + hi;                                                                   \
+        const int qb = min(q0 + 1, qlast), qc = min(q0 + 2, qlast), qd = min(q0 + 3, qlast);      \
+        o0 = obase[q0 * 2];                                                                       \
+        w0 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)q0 * 512);                          \
+        o1 = obase[qb * 2];                                                                       \
+        w1 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qb * 512);                          \
+        o2 = obase[qc * 2];                                                                       \
+        w2 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qc * 512);                          \
+        o3 = obase[qd * 2];                                                                       \
+        w3 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qd * 512);                          \
+    }
+
+    // Per-linear arguments are read from the kernel-argument segment with a
+    // run-time index (scalar loads).  Indexing the by-value struct itself would
+    // make the compiler copy it to scratch memory, and chains of selects over
+    // its constant-indexed elements compile to long branch ladders.
+    typedef const __attribute__((address_space(4))) char *KArg;
+    const KArg ka = (KArg)__builtin_amdgcn_kernarg_segment_ptr(); // TlArgs is the only argument
+#define TL_KARG(type_, field_, lin_)                                                              \
+    (*(const __attribute__((address_space(4))) type_ *)(ka + offsetof(TlArgs, field_) +           \
+                                                         (lin_) * sizeof(type_)))
+    auto tl_item = [&](int rp, int lin, int cg) {
+        TlItem t;
+        t.rp = rp;
+        t.lin = lin;
+        t.cg = cg;
+        t.bn0 = (cg * TL_WAVES + wave) * NB;
+        typedef f16 *YPtr;
+        typedef const int *IPtr;
+        typedef const f16 *HPtr;
+        t.Y = TL_KARG(YPtr, Y, lin);
+        t.cptr = TL_KARG(IPtr, cptr, lin);
+        t.poff = TL_KARG(IPtr, row_offset, lin);
+        t.data = TL_KARG(HPtr, data, lin);
+        t.bias = TL_KARG(HPtr, bias, lin);
+        t.N = TL_KARG(int, N, lin);
+        t.nbr = t.N >> 4;
+        return t;
+    };
+    // the item after t in (row panel, linear, column group) order
+    auto tl_next = [&](const TlItem &t) {
+        const bool cw = t.cg + 1 == a.ncg;
+        const bool lw = cw && t.lin + 1 == a.nlin;
+        return tl_item(t.rp + (lw ? 1 : 0), lw ? 0 : t.lin + (cw ? 1 : 0), cw ? 0 : t.cg + 1);
+    };
+#ifdef TL_TRACE
+    const unsigned long long tt0 = TL_TICK();
+    unsigned long long tpanel = 0, tcomp = 0, tepi = 0, tgap = 0, tlast = tt0;
+#endif
+    const int per_rp = a.ncg * a.nlin;
+    const int rp0 = it0 / per_rp, rest0 = it0 - rp0 * per_rp;
+    TlItem cur = tl_item(rp0, rest0 / a.ncg, rest0 % a.ncg);
+    int bvec = TL_BVEC(cur);
+    f16x4 b4[NB];
+    TL_BIAS(b4, cur)
+    TL_PANEL(cur.rp)
+    int q0, qend, qlast;
+    const f16 *wbase;
+    const int *obase;
+    f16x8 w0, w1, w2, w3;
+    int o0, o1, o2, o3;
+    // (an empty stream still loads pair q0: cptr's last entry is the padded
+    // tile count, and the plan's arrays hold one spare pair behind it)
+    TL_PRELOAD(cur, bvec)
+#ifdef TL_TRACE
+    tlast = TL_TICK();
+    tpanel = tlast - tt0;
+#endif
+
+    for (int it = it0;; it++) {
+        const bool has_next = it + 1 < it1;
+        const TlItem nxt = tl_next(cur); // (past the last item: a valid linear, never run)
+        const int bvec_n = TL_BVEC(nxt);
+        f16x4 b4n[NB];
+        TL_BIAS(b4n, nxt)
+
+#ifdef TL_TRACE
+        const unsigned long long ta = TL_TICK();
+        tgap += ta - tlast;
+#endif
+        if (q0 < qend) {
+            f32x4 cur0 = f32x4{0.f, 0.f, 0.f, 0.f}, cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
+            int j = 0;
+            int bend = __builtin_amdgcn_readlane(bvec, 1);
+            // leading empty block-rows (straight-line scalar code: loops in
+            // here would defeat the counted waits of the pipeline)
+#pragma unroll
+            for (int t = 0; t < NB - 1; t++) {
+                j += (bend == q0 && j + 1 < NB) ? 1 : 0;
+                bend = __builtin_amdgcn_readlane(bvec, j + 1);
+            }
+            f16x8 xa0 = *reinterpret_cast<const f16x8 *>(xlane + o0);
+            f16x8 xb0 = *reinterpret_cast<const f16x8 *>(xlane + o0 + xrow16);
+            f16x8 xa1 = zero8, xb1 = zero8;
+#define TL_STAGE(W_, O_, ONEXT_, XA_, XB_, XAN_, XBN_, I_)                                        \
+    {                                                                                             \
+        XAN_ = *reinterpret_cast<const f16x8 *>(xlane + ONEXT_);                                  \
+        XBN_ = *reinterpret_cast<const f16x8 *>(xlane + ONEXT_ + xrow16);                         \
+        cur0 = mfma16x16x32(W_, XA_, cur0);                                                       \
+        cur1 = mfma16x16x32(W_, XB_, cur1);                                                       \
+        {                                                                                         \
+            const int qn = min(q + (I_) + 4, qlast);                                              \
+            O_ = obase[qn * 2];                                                                   \
+            W_ = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qn * 512);                      \
+        }                                                                                         \
+        if (q + (I_) + 1 == bend) { /* block-row j is complete */                                 \
+            f16x4 bj = b4[0];                                                                     \
+            _Pragma("unroll") for (int k = 1; k < NB; k++) bj = (j == k) ? b4[k] : bj;            \
+            tl_stage_tile<GELU>(stage_lane + j * 16, lds, cur0, cur1, bj);                        \
+            cur0 = f32x4{0.f, 0.f, 0.f, 0.f};                                                     \
+            cur1 = f32x4{0.f, 0.f, 0.f, 0.f};                                                     \
+            j++;                                                                                  \
+            bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));                               \
+            _Pragma("unroll") for (int t = 0; t < NB - 2; t++) { /* skip empty block-rows */      \
+                j += (bend == q + (I_) + 1 && j + 1 < NB) ? 1 : 0;                                \
+                bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));                           \
+            }                                                                                     \
+        }                                                                                         \
+    }
+            int q = q0;
+            for (; q + 4 <= qend; q += 4) { // straight-line body: counted waits
+                TL_STAGE(w0, o0, o1, xa0, xb0, xa1, xb1, 0)
+                TL_STAGE(w1, o1, o2, xa1, xb1, xa0, xb0, 1)
+                TL_STAGE(w2, o2, o3, xa0, xb0, xa1, xb1, 2)
+                TL_STAGE(w3, o3, o0, xa1, xb1, xa0, xb0, 3)
+            }
+            if (q < qend) {
+                TL_STAGE(w0, o0, o1, xa0, xb0, xa1, xb1, 0)
+                if (q + 1 < qend) {
+                    TL_STAGE(w1, o1, o2, xa1, xb1, xa0, xb0, 1)
+                    if (q + 2 < qend)
+                        TL_STAGE(w2, o2, o3, xa0, xb0, xa1, xb1, 2)
+                }
+            }
+#undef TL_STAGE
+        }
+#ifdef TL_TRACE
+        const unsigned long long tb = TL_TICK();
+        tcomp += tb - ta;
+#endif
+        // block-rows without any tile: bias only
+#pragma unroll
+        for (int k = 0; k < NB; k++)
+            if (__builtin_amdgcn_readlane(bvec, k) == __builtin_amdgcn_readlane(bvec, k + 1))
+                tl_stage_tile<GELU>(stage_lane + k * 16, lds, f32x4{0.f, 0.f, 0.f, 0.f},
+                                    f32x4{0.f, 0.f, 0.f, 0.f}, b4[k]);
+
+        const bool same_panel = has_next && nxt.rp == cur.rp;
+        if (same_panel)
+            TL_PRELOAD(nxt, bvec_n)
+
+        // staging tile -> Y: 16-byte stores of 32*NB contiguous bytes per row
+        {
+            const int nvalid = min(NB, cur.nbr - cur.bn0); // the last column group may be partial
+            const int cpr = 2 * nvalid;                    // 16-byte chunks per row
+            const int m0 = cur.rp * TL_BM;
+            f16 *ybase = cur.Y + (size_t)m0 * cur.N + cur.bn0 * 16;
+#pragma unroll
+            for (int t = 0; t < NB; t++) {
+                const int i = lane + 64 * t;
+                const int r = i / (2 * NB), c = i - r * (2 * NB);
+                if (c < cpr && m0 + r < a.M) {
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + r * lds + c * 8);
+                    *reinterpret_cast<u32x4 *>(ybase + (size_t)r * cur.N + c * 8) = v;
+                }
+            }
+        }
+#ifdef TL_TRACE
+        tlast = TL_TICK();
+        tepi += tlast - tb;
+#endif
+        if (!has_next)
+            break;
+        if (!same_panel) {
+            __syncthreads(); // every wave is done with the previous panel
+            TL_PANEL(nxt.rp)
+            TL_PRELOAD(nxt, bvec_n)
+        }
+        cur = nxt;
+        bvec = bvec_n;
+#pragma unroll
+        for (int k = 0; k < NB; k++)
+            b4[k] = b4n[k];
+    }
+#undef TL_PRELOAD
+#undef TL_PANEL
+#undef TL_BIAS
+#ifdef TL_TRACE
+    if (g_trace && lane == 0) {
+        unsigned hwid, xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        unsigned long long *t = g_trace + ((size_t)blockIdx.x * TL_WAVES + wave) * 8;
+        t[0] = tt0; t[1] = tpanel; t[2] = tcomp; t[3] = tepi; t[4] = TL_TICK(); t[5] = hwid; t[6] = xcc; t[7] = tgap;
+    }
+#endif
+#undef TL_BVEC
+#undef TL_KARG
+}
+
+// ---------------------------------------------------------------------------
 // Generic kernel: the caller's own tile_mat (TL_RAW / TL_FILTER) or a dense
 // row-major weight (TL_DENSE).  Same mapping, plain per-block-row loops with
 // per-lane predicates.
@@ -563,10 +872,14 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_generic_kernel(const T
 // ---------------------------------------------------------------------------
 template <int NB, bool GELU, int MODE>
 static void launch_inst(const TlArgs &a, size_t lds, hipStream_t st) {
-    if constexpr (MODE == TL_PLAN)
-        hipLaunchKernelGGL((tile_linear_plan_kernel<NB, GELU>), dim3(a.per_xcd * 8),
-                           dim3(TL_THREADS), lds, st, a);
-    else
+    if constexpr (MODE == TL_PLAN) {
+        if (a.nchunk == 1)
+            hipLaunchKernelGGL((tile_linear_resident_kernel<NB, GELU>), dim3(a.per_xcd * 8),
+                               dim3(TL_THREADS), lds, st, a);
+        else
+            hipLaunchKernelGGL((tile_linear_plan_kernel<NB, GELU>), dim3(a.per_xcd * 8),
+                               dim3(TL_THREADS), lds, st, a);
+    } else
         hipLaunchKernelGGL((tile_linear_generic_kernel<NB, GELU, MODE>), dim3(a.per_xcd * 8),
                            dim3(TL_THREADS), lds, st, a);
 }
@@ -829,6 +1142,11 @@ extern "C" int et_tile_plan_create(et_tile_plan **plan, int in_feat, int out_fea
         }
     }
     cptr[(size_t)nbr * nchunk] = (int)off.size();
+    // one spare all-zero pair behind the last one: the kernels request the
+    // first pairs of a wave's stream before they know whether it is empty
+    off.push_back(0);
+    off.push_back(0);
+    packed.insert(packed.end(), 512, (uint16_t)0);
 
     et_tile_plan *p = new et_tile_plan();
     memset(p, 0, sizeof(*p));
