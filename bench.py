@@ -39,11 +39,7 @@ D, H, DFF = 768, 12, 3072
 MEASURED_TRAFFIC_MIB = {
     "tile_linear qkv (3 x 768->768, one launch)": 17.91 + 36.00,
     "attention (on-the-fly)": 40.35 + 12.00,
-    "tile_linear o (768->768)": 14.04 + 12.00,
-    "skip_layernorm 1": 24.04 + 12.00,
     "tile_linear ffn1+gelu (768->3072)": 19.84 + 48.00,
-    "tile_linear ffn2 (3072->768)": 55.78 + 12.00,
-    "skip_layernorm 2": 24.04 + 12.00,
 }
 
 
@@ -138,11 +134,11 @@ def main():
          3 * tile_flops(T, nt[0]), sum(tile_bytes(T, D, D, nt[j]) for j in range(3)) - 2 * 2 * T * D, "hbm"),
         ("attention (on-the-fly)", lambda: K.OTF_attention(b[0], b[1], b[2], mask, S, H, B, None, 1.0, out=b[3]),
          4 * B * S * S * D, 8 * B * S * D + 2 * S * S, "mfma"),
-        ("tile_linear o (768->768)", lambda: L[3].run(b[3], out=b[0]), tile_flops(T, nt[3]), tile_bytes(T, D, D, nt[3]), "hbm"),
-        ("skip_layernorm 1", lambda: K.skip_layernorm(b[0], x, gam[0], gam[1]), 0, 6 * T * D + 4 * D, "hbm"),
+        ("tile_linear o (768->768) + skip + LayerNorm", lambda: L[3].run_ln(b[3], x, gam[0], gam[1], out=b[0]),
+         tile_flops(T, nt[3]), tile_bytes(T, D, D, nt[3]) + 2 * T * D + 4 * D, "hbm"),
         ("tile_linear ffn1+gelu (768->3072)", lambda: L[4].run(b[0], out=ffn), tile_flops(T, nt[4]), tile_bytes(T, DFF, D, nt[4]), "hbm"),
-        ("tile_linear ffn2 (3072->768)", lambda: L[5].run(ffn, out=y), tile_flops(T, nt[5]), tile_bytes(T, D, DFF, nt[5]), "hbm"),
-        ("skip_layernorm 2", lambda: K.skip_layernorm(y, b[0], gam[2], gam[3]), 0, 6 * T * D + 4 * D, "hbm"),
+        ("tile_linear ffn2 (3072->768) + skip + LayerNorm", lambda: L[5].run_ln(ffn, b[0], gam[2], gam[3], out=y),
+         tile_flops(T, nt[5]), tile_bytes(T, D, DFF, nt[5]) + 2 * T * D + 4 * D, "hbm"),
     ]
     nk = len(steps_def)
     reps = max(20, min(args.steps, 100))

@@ -30,6 +30,8 @@ PROTOTYPES = {
     "et_tile_plan_create": (_i, [C.POINTER(_vp), _i, _i, _i, _vp, _ip, _ip, _vp]),
     "et_tile_plan_destroy": (None, [_vp]),
     "et_tile_plan_run": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "et_tile_plan_run_ln": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
+    "et_tile_plan_ln_fusable": (_i, [_vp]),
     "et_tile_plan_run_multi": (_i, [C.POINTER(_vp), C.POINTER(_vp), _i, _vp, _i, _vp]),
     "et_tile_plan_query": (_i, [_vp, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
     "et_gen_sparse_tile_mat": (_i, [_i, _i, _f, _u64, _ip, _ip]),
@@ -46,6 +48,7 @@ PROTOTYPES = {
     "et_linear_tile_destroy": (None, [_vp]),
     "et_linear_tile_run": (_i, [_vp, _vp, _vp, _vp]),
     "et_linear_tile_run_rows": (_i, [_vp, _vp, _vp, _i, _vp]),
+    "et_linear_tile_run_rows_ln": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
     "et_linear_tile_run_multi": (_i, [C.POINTER(_vp), C.POINTER(_vp), _i, _vp, _i, _vp]),
     "et_linear_row_create": (_i, [C.POINTER(_vp), _i, _i, _i, _vp, _ip, _i, _vp, _i]),
     "et_linear_row_destroy": (None, [_vp]),

@@ -80,6 +80,17 @@ int et_linear_tile_run_rows(const et_linear_tile *h, void *out, const void *in, 
     }
     return guarded([&] { h->impl.run_rows(H(out), H(in), rows, stream); });
 }
+int et_linear_tile_run_rows_ln(const et_linear_tile *h, void *out, const void *in, const void *skip,
+                               const void *gamma, const void *beta, int rows, void *stream) {
+    if (!h) {
+        et::set_error("et_linear_tile_run_rows_ln: null handle");
+        return ET_ERR_INVALID_ARG;
+    }
+    return guarded([&] {
+        h->impl.run_rows_ln(H(out), H(in), static_cast<const half *>(skip), static_cast<const half *>(gamma),
+                            static_cast<const half *>(beta), rows, stream);
+    });
+}
 int et_linear_tile_run_multi(const et_linear_tile *const *hs, void *const *outs, int n, const void *in,
                              int rows, void *stream) {
     if (!hs || !outs || n < 1 || n > 4) {

@@ -76,6 +76,8 @@ struct TlArgs {
     const f16 *X;
     int nlin, M, K, KC, nchunk, ncg, total, per_xcd;
     int ipw; // plan kernel: consecutive work items per (persistent) workgroup
+    // fused skip + LayerNorm epilogue (plan kernels with LN = true)
+    const f16 *skip, *gamma, *beta;
 };
 #define TL_SEL(f) (lin == 0 ? a.f[0] : lin == 1 ? a.f[1] : lin == 2 ? a.f[2] : a.f[3])
 
@@ -169,7 +171,7 @@ __device__ __forceinline__ void tl_epilogue(const TlArgs &a, const TlCtx &x, f16
 // the other waves' MFMAs.
 template <int NB> constexpr int tl_wave_stage_halves() { return TL_BM * (16 * NB + 8); }
 
-template <int NB, bool GELU>
+template <int NB, bool GELU, bool STORE = true>
 __device__ __forceinline__ void tl_epilogue_wave(const TlArgs &a, const TlCtx &x, f16 *stage, f16 *Y,
                                                  int N, int nbr, const f32x4 (&acc)[NB][2],
                                                  const f16x4 (&b4)[NB]) {
@@ -187,6 +189,8 @@ __device__ __forceinline__ void tl_epilogue_wave(const TlArgs &a, const TlCtx &x
             *reinterpret_cast<f16x4 *>(stage + (ms * 16 + x.c16) * lds + j * 16 + x.g4 * 4) = o;
         }
     }
+    if (!STORE)
+        return;
     // valid block-rows of this wave (the last column group may be partial)
     const int nvalid = min(NB, nbr - x.bn0);
     if (nvalid <= 0)
@@ -200,6 +204,71 @@ __device__ __forceinline__ void tl_epilogue_wave(const TlArgs &a, const TlCtx &x
         if (c < cpr && x.m0 + r < a.M) {
             const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + r * lds + c * 8);
             *reinterpret_cast<u32x4 *>(ybase + (size_t)r * N + c * 8) = v;
+        }
+    }
+}
+
+// Fused skip connection + LayerNorm over a workgroup's 32 finished rows (the
+// math of skip_layernorm.hip: x = half(y + skip), fp32 mean and biased
+// two-pass variance, eps 1e-6).  The workgroup covers the whole row: wave k's
+// staging tile holds columns [k*16*NB, (k+1)*16*NB).  Wave w normalises rows
+// w*32/NW .. one after the other, a row spread over its 64 lanes in 16-byte
+// pieces; the caller has put a barrier between the staging writes and this.
+template <int NB, int NW>
+__device__ __forceinline__ void tl_ln_rows(const TlArgs &a, const f16 *stage0, int wave, int lane,
+                                           int m0, f16 *Y, int N) {
+    constexpr int lds = 16 * NB + 8;
+    constexpr int RPW = TL_BM / NW;
+    constexpr int NCH = (NW * NB * 2 + 63) / 64; // 16-byte pieces per lane and row
+    const int npiece = N >> 3;
+    const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int rr = 0; rr < RPW; rr++) {
+        const int r = wave * RPW + rr;
+        const long row = (long)m0 + r;
+        if (row >= a.M)
+            break;
+        f16x8 xv[NCH];
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int ch = lane + 64 * i;
+            xv[i] = zero8;
+            if (ch < npiece) {
+                const int tile = ch / (2 * NB), c = ch - tile * (2 * NB);
+                const f16x8 y = *reinterpret_cast<const f16x8 *>(
+                    stage0 + tile * tl_wave_stage_halves<NB>() + r * lds + c * 8);
+                const f16x8 sk = *reinterpret_cast<const f16x8 *>(a.skip + row * N + ch * 8);
+                xv[i] = y + sk; // half add, one rounding (kernels/skip_layernorm.cu:20)
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                sum += (float)xv[i][j];
+        }
+        const float mean = wave_sum(sum) / (float)N;
+        float var = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; i++)
+            if (lane + 64 * i < npiece) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const float d = (float)xv[i][j] - mean;
+                    var += d * d;
+                }
+            }
+        const float rstd = rsqrtf(wave_sum(var) / (float)N + 1e-6f);
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int ch = lane + 64 * i;
+            if (ch < npiece) {
+                const f16x8 gg = *reinterpret_cast<const f16x8 *>(a.gamma + ch * 8);
+                const f16x8 bb = *reinterpret_cast<const f16x8 *>(a.beta + ch * 8);
+                f16x8 o;
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    o[j] = (f16)(((float)xv[i][j] - mean) * rstd * (float)gg[j] + (float)bb[j]);
+                *reinterpret_cast<f16x8 *>(Y + row * N + ch * 8) = o;
+            }
         }
     }
 }
@@ -232,8 +301,8 @@ __device__ unsigned long long *g_trace = nullptr; // per wave: start, panel, com
 #define TL_TICK() __builtin_readcyclecounter()
 #endif
 
-template <int NB, bool GELU>
-__global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlArgs a) {
+template <int NB, bool GELU, int NW, bool LN>
+__global__ void __launch_bounds__(NW * 64) tile_linear_plan_kernel(const TlArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
     f16 *xs = reinterpret_cast<f16 *>(tl_smem);
     // Workgroups with consecutive virtual ids run on ONE XCD (hardware
@@ -255,7 +324,8 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
     const int hi = x.hi, lane = x.lane;
     const char *xlane = reinterpret_cast<const char *>(xs + x.c16 * x.ldx + x.khalf8);
     const int xrow16 = 16 * x.ldx * 2; // bytes between the two 16-row subtiles
-    f16 *const stage = xs + TL_BM * x.ldx + x.wave * tl_wave_stage_halves<NB>();
+    f16 *const stage0 = xs + TL_BM * x.ldx;
+    f16 *const stage = stage0 + x.wave * tl_wave_stage_halves<NB>();
     const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     const int per_rp = a.ncg * a.nlin;
 #ifdef TL_TRACE
@@ -273,8 +343,8 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
     {                                                                                             \
         const int pk0 = (c_) * a.KC;                                                              \
         const int pcpr = min(a.KC, a.K - pk0) >> 3; /* 16-byte chunks per row, <= 124 */          \
-        _Pragma("unroll") for (int rr = 0; rr < 4; rr++) {                                        \
-            const int row = x.wave * 4 + rr;                                                      \
+        _Pragma("unroll") for (int rr = 0; rr < TL_BM / NW; rr++) {                               \
+            const int row = x.wave * (TL_BM / NW) + rr;                                           \
             if (x.m0 + row < a.M) {                                                               \
                 const f16 *src = a.X + (size_t)(x.m0 + row) * a.K + pk0;                          \
                 f16 *dstrow = xs + row * x.ldx;                                                   \
@@ -295,7 +365,7 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
         x.lin = lin;
         x.cg = rest - lin * a.ncg;
         x.m0 = rp * TL_BM;
-        x.bn_wg = x.cg * (TL_WAVES * NB);
+        x.bn_wg = x.cg * (NW * NB);
         x.bn0 = x.bn_wg + x.wave * NB;
         f16 *const Yp = TL_SEL(Y);
         const int *const cptr = TL_SEL(cptr);
@@ -433,7 +503,12 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
 #ifdef TL_TRACE
         const unsigned long long te = TL_TICK();
 #endif
-        tl_epilogue_wave<NB, GELU>(a, x, stage, Yp, N, nbr, acc, b4);
+        tl_epilogue_wave<NB, GELU, !LN>(a, x, stage, Yp, N, nbr, acc, b4);
+        if (LN) {
+            __syncthreads(); // every wave's part of the rows is staged
+            tl_ln_rows<NB, NW>(a, stage0, x.wave, lane, x.m0, Yp, N);
+            lds_used = true; // (the next item's panel load starts with a barrier)
+        }
 #ifdef TL_TRACE
         tlast = TL_TICK();
         tepi += tlast - te;
@@ -445,7 +520,7 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_plan_kernel(const TlAr
         unsigned hwid, xcc;
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        unsigned long long *t = g_trace + ((size_t)blockIdx.x * TL_WAVES + x.wave) * 8;
+        unsigned long long *t = g_trace + ((size_t)blockIdx.x * NW + x.wave) * 8;
         t[0] = tt0; t[1] = tpanel; t[2] = tcomp; t[3] = tepi; t[4] = TL_TICK(); t[5] = hwid; t[6] = xcc; t[7] = tgap;
     }
 #endif
@@ -505,8 +580,8 @@ __device__ __forceinline__ void tl_stage_tile(f16 *dst, int lds, f32x4 c0, f32x4
     *reinterpret_cast<f16x4 *>(dst + 16 * lds) = o1;
 }
 
-template <int NB, bool GELU>
-__global__ void __launch_bounds__(TL_THREADS) tile_linear_resident_kernel(const TlArgs a) {
+template <int NB, bool GELU, int NW, bool LN>
+__global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
     f16 *xs = reinterpret_cast<f16 *>(tl_smem);
     const int vid = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3); // see tile_linear_plan_kernel
@@ -521,7 +596,8 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_resident_kernel(const 
     const char *xlane = reinterpret_cast<const char *>(xs + c16 * ldx + khalf8);
     const int xrow16 = 16 * ldx * 2; // bytes between the two 16-row subtiles
     constexpr int lds = 16 * NB + 8; // halves per staged row
-    f16 *const stage = xs + TL_BM * ldx + wave * tl_wave_stage_halves<NB>();
+    f16 *const stage0 = xs + TL_BM * ldx;
+    f16 *const stage = stage0 + wave * tl_wave_stage_halves<NB>();
     f16 *const stage_lane = stage + c16 * lds + g4 * 4;
     const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     const int lane_w = hi * 256 + c16 * 16 + khalf8; // lane's halves inside a 1 KB tile pair
@@ -539,11 +615,11 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_resident_kernel(const 
 #define TL_PANEL(rp_)                                                                             \
     {                                                                                             \
         const int pcpr = a.K >> 3;                                                                \
-        _Pragma("unroll") for (int rr = 0; rr < 4; rr++) {                                        \
-            const int row = (rp_) * TL_BM + wave * 4 + rr;                                        \
+        _Pragma("unroll") for (int rr = 0; rr < TL_BM / NW; rr++) {                               \
+            const int row = (rp_) * TL_BM + wave * (TL_BM / NW) + rr;                             \
             if (row < a.M) {                                                                      \
                 const f16 *src = a.X + (size_t)row * a.K;                                         \
-                f16 *dstrow = xs + (wave * 4 + rr) * ldx;                                         \
+                f16 *dstrow = xs + (wave * (TL_BM / NW) + rr) * ldx;                                       \
                 if (lane < pcpr)                                                                  \
                     load_lds16(src + lane * 8, dstrow);                                           \
                 if (64 + lane < pcpr)                                                             \
@@ -586,7 +662,7 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_resident_kernel(const 
         t.rp = rp;
         t.lin = lin;
         t.cg = cg;
-        t.bn0 = (cg * TL_WAVES + wave) * NB;
+        t.bn0 = (cg * NW + wave) * NB;
         typedef f16 *YPtr;
         typedef const int *IPtr;
         typedef const f16 *HPtr;
@@ -711,8 +787,14 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_resident_kernel(const 
         if (same_panel)
             TL_PRELOAD(nxt, bvec_n)
 
-        // staging tile -> Y: 16-byte stores of 32*NB contiguous bytes per row
-        {
+        if (LN) {
+            // the workgroup holds whole rows: skip connection + LayerNorm here
+            __syncthreads(); // every wave's part of the rows is staged
+            tl_ln_rows<NB, NW>(a, stage0, wave, lane, cur.rp * TL_BM, cur.Y, cur.N);
+            if (has_next && same_panel)
+                __syncthreads(); // the staging tiles are free again
+        } else {
+            // staging tile -> Y: 16-byte stores of 32*NB contiguous bytes per row
             const int nvalid = min(NB, cur.nbr - cur.bn0); // the last column group may be partial
             const int cpr = 2 * nvalid;                    // 16-byte chunks per row
             const int m0 = cur.rp * TL_BM;
@@ -752,7 +834,7 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_resident_kernel(const 
         unsigned hwid, xcc;
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        unsigned long long *t = g_trace + ((size_t)blockIdx.x * TL_WAVES + wave) * 8;
+        unsigned long long *t = g_trace + ((size_t)blockIdx.x * NW + wave) * 8;
         t[0] = tt0; t[1] = tpanel; t[2] = tcomp; t[3] = tepi; t[4] = TL_TICK(); t[5] = hwid; t[6] = xcc; t[7] = tgap;
     }
 #endif
@@ -872,16 +954,17 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_generic_kernel(const T
 // ---------------------------------------------------------------------------
 template <int NB, bool GELU, int MODE>
 static void launch_inst(const TlArgs &a, size_t lds, hipStream_t st) {
+    const dim3 grid(a.per_xcd * 8), block(TL_THREADS);
     if constexpr (MODE == TL_PLAN) {
+        // (block-rows per wave beyond 3 never paid off for the plan kernels)
+        constexpr int PNB = NB > 3 ? 3 : NB;
         if (a.nchunk == 1)
-            hipLaunchKernelGGL((tile_linear_resident_kernel<NB, GELU>), dim3(a.per_xcd * 8),
-                               dim3(TL_THREADS), lds, st, a);
+            hipLaunchKernelGGL((tile_linear_resident_kernel<PNB, GELU, TL_WAVES, false>), grid, block, lds, st, a);
         else
-            hipLaunchKernelGGL((tile_linear_plan_kernel<NB, GELU>), dim3(a.per_xcd * 8),
-                               dim3(TL_THREADS), lds, st, a);
-    } else
-        hipLaunchKernelGGL((tile_linear_generic_kernel<NB, GELU, MODE>), dim3(a.per_xcd * 8),
-                           dim3(TL_THREADS), lds, st, a);
+            hipLaunchKernelGGL((tile_linear_plan_kernel<PNB, GELU, TL_WAVES, false>), grid, block, lds, st, a);
+    } else {
+        hipLaunchKernelGGL((tile_linear_generic_kernel<NB, GELU, MODE>), grid, block, lds, st, a);
+    }
 }
 
 template <bool GELU, int MODE>
@@ -895,10 +978,75 @@ static void launch_nb(int nb, const TlArgs &a, size_t lds, hipStream_t st) {
     }
 }
 
+// Fused linear + skip + LayerNorm: one workgroup of 16 waves covers whole rows.
+constexpr int TL_LN_WAVES = 16;
+
+template <int NB>
+static int launch_ln_inst(const TlArgs &a, size_t lds, hipStream_t st) {
+    const dim3 grid(a.per_xcd * 8), block(TL_LN_WAVES * 64);
+    if (a.nchunk == 1) {
+        auto k = tile_linear_resident_kernel<NB, false, TL_LN_WAVES, true>;
+        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(k, grid, block, lds, st, a);
+    } else {
+        auto k = tile_linear_plan_kernel<NB, false, TL_LN_WAVES, true>;
+        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(k, grid, block, lds, st, a);
+    }
+    return launch_status("tile_linear+LayerNorm launch");
+}
+
+// block-rows per wave of the fused kernel for a matrix of nbr block-rows; 0 if
+// the rows do not fit one workgroup (then the caller runs the two kernels)
+static int ln_block_rows(int nbr) {
+    const int need = (nbr + TL_LN_WAVES - 1) / TL_LN_WAVES;
+    return need <= 3 ? need : need == 4 ? 4 : need <= 6 ? 6 : 0;
+}
+
+static int tile_launch_ln(const TlProblem &p, const f16 *X, int M, int K, int KC, int nchunk,
+                          const f16 *skip, const f16 *gamma, const f16 *beta, hipStream_t st) {
+    TlArgs a;
+    memset(&a, 0, sizeof(a));
+    for (int i = 0; i < TL_MAX_LIN; i++) {
+        a.Y[i] = p.Y;
+        a.cptr[i] = p.cptr;
+        a.row_offset[i] = p.row_offset;
+        a.data[i] = p.data;
+        a.bias[i] = p.bias;
+        a.N[i] = p.N;
+    }
+    a.X = X;
+    a.nlin = 1;
+    a.M = M;
+    a.K = K;
+    a.KC = KC;
+    a.nchunk = nchunk;
+    a.ncg = 1;
+    a.total = (M + TL_BM - 1) / TL_BM;
+    a.ipw = 1;
+    a.per_xcd = (a.total + 7) / 8;
+    a.skip = skip;
+    a.gamma = gamma;
+    a.beta = beta;
+    const int nb = ln_block_rows(p.nbr);
+    const size_t lds = (size_t)TL_BM * (KC + ((KC & 31) ? 0 : TL_PAD)) * sizeof(f16) +
+                       (size_t)TL_LN_WAVES * TL_BM * (16 * nb + 8) * sizeof(f16);
+    switch (nb) {
+    case 1: return launch_ln_inst<1>(a, lds, st);
+    case 2: return launch_ln_inst<2>(a, lds, st);
+    case 3: return launch_ln_inst<3>(a, lds, st);
+    case 4: return launch_ln_inst<4>(a, lds, st);
+    default: return launch_ln_inst<6>(a, lds, st);
+    }
+}
+
 // Tuning knobs (et_tuning_set): 0 = automatic.
 static int g_tile_nb = 0;
 static int g_tile_min_wgs = 512;
 static int g_tile_ipw = 0;
+static int g_tile_fuse_ln = 1;
 
 // Block-rows per wave.  Measured on the BERT-base shapes (rows 4096..8192):
 // three block-rows per wave is the best trade between panel re-reads (fewer
@@ -1026,6 +1174,10 @@ extern "C" int et_tuning_set(const char *key, int value) {
     }
     if (key && !strcmp(key, "tile_ipw")) {
         et::g_tile_ipw = value;
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "tile_fuse_ln")) {
+        et::g_tile_fuse_ln = value;
         return ET_OK;
     }
     if (key && !strcmp(key, "tile_min_wgs")) {
@@ -1221,6 +1373,47 @@ extern "C" int et_tile_plan_run_multi(const et_tile_plan *const *plans, void *co
         return ET_OK;
     return tile_launch(pr, n, static_cast<const f16 *>(X), M, plans[0]->in_feat, plans[0]->KC,
                        plans[0]->nchunk, false, TL_PLAN, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int et_tile_plan_ln_fusable(const et_tile_plan *plan) {
+    return plan && et::ln_block_rows(plan->out_feat / 16) != 0 && plan->out_feat % 8 == 0 &&
+                   et::g_tile_fuse_ln != 0
+               ? 1
+               : 0;
+}
+
+extern "C" int et_tile_plan_run_ln(const et_tile_plan *plan, void *Y, const void *X,
+                                   const void *skip, const void *gamma, const void *beta, int M,
+                                   void *stream) {
+    using namespace et;
+    ET_REQUIRE(plan && Y && X && skip && gamma && beta, ET_ERR_INVALID_ARG,
+               "et_tile_plan_run_ln: null pointer");
+    ET_REQUIRE(M >= 0, ET_ERR_INVALID_ARG, "et_tile_plan_run_ln: M=%d", M);
+    ET_REQUIRE(aligned16(Y) && aligned16(X) && aligned16(skip) && aligned16(gamma) && aligned16(beta),
+               ET_ERR_ALIGNMENT, "et_tile_plan_run_ln: pointers must be 16-byte aligned");
+    if (M == 0)
+        return ET_OK;
+    const int nbr = plan->out_feat / 16;
+    if (!et_tile_plan_ln_fusable(plan)) {
+        // rows too wide for one workgroup: the two kernels, one after the other
+        ET_REQUIRE(Y != skip, ET_ERR_INVALID_ARG,
+                   "et_tile_plan_run_ln: Y must not alias skip for out_feat=%d", plan->out_feat);
+        const int rc = et_tile_plan_run(plan, Y, X, M, 0, stream);
+        if (rc != ET_OK)
+            return rc;
+        return et_skip_layernorm(Y, skip, gamma, beta, M, plan->out_feat, stream);
+    }
+    TlProblem pr;
+    pr.Y = static_cast<f16 *>(Y);
+    pr.cptr = plan->d_cptr;
+    pr.row_offset = plan->d_row_offset;
+    pr.data = plan->d_data;
+    pr.bias = plan->d_bias;
+    pr.N = plan->out_feat;
+    pr.nbr = nbr;
+    return tile_launch_ln(pr, static_cast<const f16 *>(X), M, plan->in_feat, plan->KC, plan->nchunk,
+                          static_cast<const f16 *>(skip), static_cast<const f16 *>(gamma),
+                          static_cast<const f16 *>(beta), static_cast<hipStream_t>(stream));
 }
 
 extern "C" int et_tile_plan_run(const et_tile_plan *plan, void *Y, const void *X, int M, int gelu,

@@ -54,6 +54,14 @@ class Linear_tile:
         check(lib().et_linear_tile_run_rows(self._h, _dp(out), _dp(x), rows, _stream()))
         return out
 
+    def run_ln(self, x, skip, gamma, beta, out=None, rows=None):
+        """LayerNorm(half(linear(x)) + skip) * gamma + beta in one launch"""
+        rows = x.shape[0] if rows is None else rows
+        out = out if out is not None else torch.empty((x.shape[0], self.out_feat), dtype=torch.float16, device=x.device)
+        check(lib().et_linear_tile_run_rows_ln(self._h, _dp(out), _dp(x), _dp(skip), _dp(gamma), _dp(beta),
+                                               rows, _stream()))
+        return out
+
     def _release(self):  # ownership moved into an encoder
         self._h = None
 

@@ -41,6 +41,15 @@ class Linear_tile {
         etChk(et_tile_plan_run(plan, out, in, rows, is_gelu ? 1 : 0, stream));
     }
     // several linears over the same input in one launch (Q, K, V)
+    // this linear, the skip connection and LayerNorm in one launch:
+    // out = LayerNorm(half(linear(in)) + skip); see et_tile_plan_run_ln
+    void run_rows_ln(half *out, half *in, const half *skip, const half *gamma, const half *beta,
+                     int rows, void *stream) const {
+        etRequire(!is_gelu, "Linear_tile::run_rows_ln: not available for the GELU linear");
+        etChk(et_tile_plan_run_ln(plan, out, in, skip, gamma, beta, rows, stream));
+    }
+    bool ln_fusable() const { return et_tile_plan_ln_fusable(plan) != 0; }
+
     static void run_multi(const Linear_tile *const *lin, half *const *outs, int n, half *in, int rows,
                           void *stream) {
         const et_tile_plan *plans[4];

@@ -84,11 +84,10 @@ class Encoder_base {
     // O projection, skip-LN with the layer input, FFN1+GELU, FFN2, skip-LN.
     void tail(half *out, half *in, half *attn, const Linear_tile &O, const Linear_tile &M1,
               const Linear_tile &M2, int nrows) {
-        O.run_rows(buffers[0], attn, nrows, stream);
-        etChk(et_skip_layernorm(buffers[0], in, ln_gamma[0].get(), ln_beta[0].get(), nrows, d_model, stream));
+        // (each projection, its skip connection and LayerNorm are one launch)
+        O.run_rows_ln(buffers[0], attn, in, ln_gamma[0].get(), ln_beta[0].get(), nrows, stream);
         M1.run_rows(buffers[1], buffers[0], nrows, stream); // spans buffers[1..4]
-        M2.run_rows(out, buffers[1], nrows, stream);
-        etChk(et_skip_layernorm(out, buffers[0], ln_gamma[1].get(), ln_beta[1].get(), nrows, d_model, stream));
+        M2.run_rows_ln(out, buffers[1], buffers[0], ln_gamma[1].get(), ln_beta[1].get(), nrows, stream);
     }
 };
 
@@ -218,11 +217,17 @@ class Encoder_length : public Encoder_base {
             Linear_tile::run_multi(qkv, outs, 3, in_p, n, stream);
             etChk(et_OTF_attention_varlen(buffers[3], buffers[0], buffers[1], buffers[2], mask_ptr(),
                                           d_cu.get(), seq_len, d_model, nheads, batch, log2_scale, stream));
-            O_linear.run_rows(buffers[0], buffers[3], n, stream);
-            etChk(et_skip_layernorm(buffers[0], in_p, ln_gamma[0].get(), ln_beta[0].get(), n, d_model, stream));
+            O_linear.run_rows_ln(buffers[0], buffers[3], in_p, ln_gamma[0].get(), ln_beta[0].get(), n, stream);
             MLP1_linear.run_rows(buffers[1], buffers[0], n, stream);
-            MLP2_linear.run_rows(out, buffers[1], n, stream);
-            etChk(et_skip_layernorm(buffers[0], out, ln_gamma[1].get(), ln_beta[1].get(), n, d_model, stream));
+            if (MLP2_linear.ln_fusable()) {
+                // in place over the skip operand: a workgroup reads its rows of
+                // unit 0 before it writes them
+                MLP2_linear.run_rows_ln(buffers[0], buffers[1], buffers[0], ln_gamma[1].get(),
+                                        ln_beta[1].get(), n, stream);
+            } else {
+                MLP2_linear.run_rows(out, buffers[1], n, stream);
+                etChk(et_skip_layernorm(buffers[0], out, ln_gamma[1].get(), ln_beta[1].get(), n, d_model, stream));
+            }
             etChk(et_unpack_rows(out, buffers[0], d_cu.get(), batch, seq_len, d_model, stream));
             return;
         }

@@ -145,6 +145,17 @@ void et_tile_plan_destroy(et_tile_plan *plan);
 /* Linear_tile::run (encoder/Linear.h:36-45); gelu selects the GELU variant. */
 int et_tile_plan_run(const et_tile_plan *plan, void *Y, const void *X, int M,
                      int gelu, void *stream);
+/* Linear_tile::run followed by skip_layernorm_kernelLauncher on its output
+ * (encoder/encoder.cu:33-35 and 41-44; kernels/kernels.h:3-5) in ONE launch:
+ *   Y = LayerNorm(half(X W^T + bias) + skip) * gamma + beta,
+ * the sum rounded to half once, as the reference does.  One workgroup holds
+ * whole rows, so this needs out_feat <= 1536 (et_tile_plan_ln_fusable); wider
+ * plans run the two kernels one after the other, and then Y must not alias
+ * skip.  With the fused kernel Y may be the same buffer as skip. */
+int et_tile_plan_run_ln(const et_tile_plan *plan, void *Y, const void *X,
+                        const void *skip, const void *gamma, const void *beta,
+                        int M, void *stream);
+int et_tile_plan_ln_fusable(const et_tile_plan *plan);
 /* n (<= 4) planned linears with the same in_feat applied to the same X in ONE
  * launch (the Q/K/V projections, encoder/encoder.cu:22-26, which the
  * reference spreads over three streams). */

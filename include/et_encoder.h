@@ -32,6 +32,10 @@ void et_linear_tile_destroy(et_linear_tile *h);
 int et_linear_tile_run(const et_linear_tile *h, void *out, const void *in, void *stream);
 /* same on `rows` rows instead of the constructor's size */
 int et_linear_tile_run_rows(const et_linear_tile *h, void *out, const void *in, int rows, void *stream);
+/* the linear, the skip connection and LayerNorm in one launch
+ * (et_tile_plan_run_ln): out = LayerNorm(half(linear(in)) + skip) */
+int et_linear_tile_run_rows_ln(const et_linear_tile *h, void *out, const void *in, const void *skip,
+                               const void *gamma, const void *beta, int rows, void *stream);
 /* n <= 4 linears over one input in one launch (Q/K/V, encoder/encoder.cu:22-26) */
 int et_linear_tile_run_multi(const et_linear_tile *const *hs, void *const *outs, int n,
                              const void *in, int rows, void *stream);

@@ -91,6 +91,47 @@ def test_tile_linear_raw_and_planned(K, M, N, Kd, sp, gelu):
     check_close(got2, want64, max_abs=tol, mean_rel=5e-4, what="tile planned vs f64")
 
 
+LN_CASES = [
+    # M, N, K, sparsity
+    (128, 768, 768, 0.8),     # O projection + LayerNorm (resident panel, 3 block-rows per wave)
+    (100, 768, 3072, 0.8),    # FFN2 + LayerNorm, K in chunks, ragged M
+    (64, 256, 256, 0.5),      # one block-row per wave
+    (40, 512, 1024, 0.6),     # two block-rows per wave, chunked K
+    (33, 1024, 512, 0.7),     # four
+    (70, 1536, 768, 0.9),     # six: the widest fused row
+    (20, 48, 64, 0.0),        # most waves own nothing
+    (50, 2048, 256, 0.8),     # too wide for one workgroup: two launches
+]
+
+
+@pytest.mark.parametrize("M,N,Kd,sp", LN_CASES)
+def test_tile_linear_fused_skip_layernorm(K, M, N, Kd, sp):
+    """Linear_tile.run_ln == skip_layernorm(tile_linear(x), skip) of the oracle"""
+    from et_amd.encoder import Linear_tile
+    r = rng(900 + M + N)
+    lin = make_tile_linear(r, N, Kd, sp, seed=3 * M + N + Kd, std=0.05, bias_std=0.2)
+    X, skip = randn_h(r, (M, Kd)), randn_h(r, (M, N))
+    g, b = randn_h(r, (N,), 0.3) + np.float16(1), randn_h(r, (N,), 0.3)
+    y = orc.tile_linear(X, lin["row_ptr"], lin["row_offset"], lin["data"], lin["bias"], N)
+    want = orc.skip_layernorm(y, skip, g, b)
+    want64 = orc.skip_layernorm(y, skip, g, b, f64=True)
+    lt = Linear_tile(Kd, N, M, lin["row_offset"].size, lin["data"], lin["row_ptr"], lin["row_offset"], lin["bias"], False)
+    got = host(lt.run_ln(dev(X), dev(skip), dev(g), dev(b)))
+    check_close(got, want64, what="fused linear+LN vs f64")
+    check_close(got, want, what="fused linear+LN vs f32")
+    # against the two separate launches of this library: same linear, same
+    # LayerNorm arithmetic, only the summation order of the row statistics differs
+    two = lt.run(dev(X))
+    K.skip_layernorm(two, dev(skip), dev(g), dev(b))
+    two = host(two)
+    assert np.abs(got.astype(np.float32) - two.astype(np.float32)).max() <= 2.0 ** -7
+    assert (got != two).mean() < 0.02
+    if N <= 1536:  # fused: the output may overwrite the skip operand
+        sk = dev(skip)
+        lt.run_ln(dev(X), sk, dev(g), dev(b), out=sk)
+        assert np.array_equal(host(sk), got)
+
+
 def test_tile_linear_closed_form_reference_smoke_inputs(K):
     """weights = bias = 0.1 (test/gen_linear.cu:8,10): Y = 0.1*sum_{kept k} X + 0.1"""
     r = rng(12)
