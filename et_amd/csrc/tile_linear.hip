@@ -26,6 +26,7 @@
 #include "common.h"
 
 #include <algorithm>
+#include <type_traits>
 #include <cstdlib>
 #include <cstring>
 #include <numeric>
@@ -208,25 +209,180 @@ __device__ __forceinline__ void tl_epilogue_wave(const TlArgs &a, const TlCtx &x
     }
 }
 
+// ---------------------------------------------------------------------------
+// The pair stream shared by the plan kernels.
+//
+// A wave owns NB CONSECUTIVE block-rows, and the plan stores tiles in (chunk,
+// block-row) order with even segments, so the wave's work for a chunk is ONE
+// contiguous run of tile pairs [q0, qend): 1 KB of W per pair at an address
+// linear in the pair index, plus one int per half-wave giving the LDS byte
+// offset of that tile's X columns.  The run is consumed through a TL_DEPTH-stage
+// register pipeline (stage = pair index mod TL_DEPTH), every load unconditional
+// with a clamped address, so TL_DEPTH pairs are always in flight per wave and
+// the waits are counted, not drained.  X operands are read from LDS one stage
+// ahead.  Products accumulate into one running 32x16 accumulator; when the
+// stream crosses a block-row boundary (a scalar compare per pair) flush(j,
+// cur0, cur1) receives block-row j's finished sums.  All control flow in here
+// is wave-uniform and straight-line per stage: loops or conditional loads
+// would make the compiler drain every load instead of counting.
+// ---------------------------------------------------------------------------
+#ifndef TL_DEPTH
+#define TL_DEPTH 4
+#endif
+static_assert(TL_DEPTH % 2 == 0, "the X operand ping-pong needs an even pipeline depth");
+
+template <int I> using tl_ic = std::integral_constant<int, I>;
+template <int B, int E, class F>
+__device__ __forceinline__ void tl_static_for(F &&f) {
+    if constexpr (B < E) {
+        f(tl_ic<B>());
+        tl_static_for<B + 1, E>(f);
+    }
+}
+
+// the first TL_DEPTH pairs of a stream (an empty stream still loads pair q0:
+// the plan keeps a spare pair behind the last one)
+// One pair's operands: 16 bytes of W per lane and the lane's X offset.  The
+// pair's address is wave-uniform (scalar registers) and the lane's part a
+// 32-bit offset, so the loads need no vector address arithmetic.
+__device__ __forceinline__ void tl_load_pair(const f16 *data, const int *poff, int q, unsigned lane_w,
+                                             unsigned hi, f16x8 &w, int &o) {
+    const char *wq = reinterpret_cast<const char *>(data) + (size_t)q * 1024; // uniform
+    const char *oq = reinterpret_cast<const char *>(poff) + (size_t)q * 8;    // uniform
+    // (the empty asm keeps the compiler from folding the lane offsets into
+    // loop-invariant 64-bit vector addresses, which costs two 64-bit vector
+    // adds per pair instead of none)
+    unsigned lo = hi * 4u, lw = lane_w * 2u;
+    asm("" : "+v"(lo), "+v"(lw));
+    o = *reinterpret_cast<const int *>(oq + lo);
+    w = *reinterpret_cast<const f16x8 *>(wq + lw);
+}
+
+__device__ __forceinline__ void tl_preload(const f16 *data, const int *poff, unsigned lane_w, unsigned hi,
+                                           int q0, int qlast, f16x8 (&w)[TL_DEPTH], int (&o)[TL_DEPTH]) {
+#pragma unroll
+    for (int i = 0; i < TL_DEPTH; i++)
+        tl_load_pair(data, poff, min(q0 + i, qlast), lane_w, hi, w[i], o[i]);
+}
+
+// bvec: lane j holds the first pair of block-row j, lane NB the end of the
+// last one (read back with v_readlane)
+template <int NB, class Flush>
+__device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f16 *data,
+                                          const int *poff, unsigned lane_w, unsigned hi, int q0,
+                                          int qend, int qlast, int bvec, f16x8 (&w)[TL_DEPTH],
+                                          int (&o)[TL_DEPTH], Flush &&flush) {
+    if (q0 >= qend)
+        return;
+    f32x4 cur0 = f32x4{0.f, 0.f, 0.f, 0.f}, cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
+    int j = 0;
+    int bend = __builtin_amdgcn_readlane(bvec, 1);
+#pragma unroll
+    for (int t = 0; t < NB - 1; t++) { // leading empty block-rows
+        j += (bend == q0 && j + 1 < NB) ? 1 : 0;
+        bend = __builtin_amdgcn_readlane(bvec, j + 1);
+    }
+    f16x8 xa[2], xb[2];
+    xa[0] = *reinterpret_cast<const f16x8 *>(xlane + o[0]);
+    xb[0] = *reinterpret_cast<const f16x8 *>(xlane + o[0] + xrow16);
+    xa[1] = xb[1] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    int q = q0;
+    auto stage = [&](auto ic) {
+        constexpr int I = decltype(ic)::value;
+        constexpr int S = I % TL_DEPTH, SN = (I + 1) % TL_DEPTH, P = I & 1;
+        xa[P ^ 1] = *reinterpret_cast<const f16x8 *>(xlane + o[SN]);
+        xb[P ^ 1] = *reinterpret_cast<const f16x8 *>(xlane + o[SN] + xrow16);
+        // keep the reads above the MFMAs: left alone, the scheduler sinks them
+        // to the end of the stage and every stage then waits out the LDS latency
+        __builtin_amdgcn_sched_barrier(0);
+        cur0 = mfma16x16x32(w[S], xa[P], cur0);
+        cur1 = mfma16x16x32(w[S], xb[P], cur1);
+        tl_load_pair(data, poff, min(q + I + TL_DEPTH, qlast), lane_w, hi, w[S], o[S]);
+        if (q + I + 1 == bend) { // block-row j is complete
+            flush(j, cur0, cur1);
+            cur0 = f32x4{0.f, 0.f, 0.f, 0.f};
+            cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
+            j++;
+            bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));
+#pragma unroll
+            for (int t = 0; t < NB - 2; t++) { // skip empty block-rows
+                j += (bend == q + I + 1 && j + 1 < NB) ? 1 : 0;
+                bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));
+            }
+        }
+    };
+    for (; q + TL_DEPTH <= qend; q += TL_DEPTH) // straight-line body: counted waits
+        tl_static_for<0, TL_DEPTH>(stage);
+    tl_static_for<0, TL_DEPTH - 1>([&](auto ic) {
+        if (q + decltype(ic)::value < qend)
+            stage(ic);
+    });
+}
+
+// flush for kernels that keep NB static accumulators: acc[j] += cur with a
+// 0/1 mask per accumulator (branch-free; a branch per j makes the compiler
+// keep a copy of every accumulator per pipeline stage)
+template <int NB>
+__device__ __forceinline__ void tl_flush_acc(f32x4 (&acc)[NB][2], int j, f32x4 cur0, f32x4 cur1) {
+#pragma unroll
+    for (int k = 0; k < NB; k++) {
+        const float mk = (k == j) ? 1.0f : 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            acc[k][0][r] = __builtin_fmaf(cur0[r], mk, acc[k][0][r]);
+            acc[k][1][r] = __builtin_fmaf(cur1[r], mk, acc[k][1][r]);
+        }
+    }
+}
+
 // Fused skip connection + LayerNorm over a workgroup's 32 finished rows (the
 // math of skip_layernorm.hip: x = half(y + skip), fp32 mean and biased
 // two-pass variance, eps 1e-6).  The workgroup covers the whole row: wave k's
-// staging tile holds columns [k*16*NB, (k+1)*16*NB).  Wave w normalises rows
-// w*32/NW .. one after the other, a row spread over its 64 lanes in 16-byte
-// pieces; the caller has put a barrier between the staging writes and this.
-template <int NB, int NW>
-__device__ __forceinline__ void tl_ln_rows(const TlArgs &a, const f16 *stage0, int wave, int lane,
-                                           int m0, f16 *Y, int N) {
+// staging tile holds columns [k*16*NB, (k+1)*16*NB), k < NW.  Wave w of the NLW
+// waves that take part normalises rows w, w+NLW, ..., a row spread over its 64
+// lanes in 16-byte pieces.  The operands that come from global memory (the
+// skip rows, gamma, beta) are requested by tl_ln_fetch, which a wave calls
+// BEFORE the barrier that ends the staging writes, so that their latency runs
+// under the wait for the other waves.
+template <int NB, int NW, int NLW>
+struct TlLnOperands {
+    static constexpr int NCH = (NW * NB * 2 + 63) / 64;    // 16-byte pieces per lane and row
+    static constexpr int ROWS = (TL_BM + NLW - 1) / NLW;   // rows per wave
+    f16x8 skip[ROWS][NCH], gamma[NCH], beta[NCH];
+};
+
+template <int NB, int NW, int NLW>
+__device__ __forceinline__ void tl_ln_fetch(TlLnOperands<NB, NW, NLW> &op, const TlArgs &a, int wave,
+                                            int lane, int m0, int N) {
+    constexpr int NCH = TlLnOperands<NB, NW, NLW>::NCH;
+    constexpr int ROWS = TlLnOperands<NB, NW, NLW>::ROWS;
+    const int npiece = N >> 3;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int ch = min(lane + 64 * i, npiece - 1); // (clamped pieces are never used)
+#pragma unroll
+        for (int k = 0; k < ROWS; k++) {
+            const long row = min((long)m0 + wave + k * NLW, (long)a.M - 1);
+            op.skip[k][i] = *reinterpret_cast<const f16x8 *>(a.skip + row * N + ch * 8);
+        }
+        op.gamma[i] = *reinterpret_cast<const f16x8 *>(a.gamma + ch * 8);
+        op.beta[i] = *reinterpret_cast<const f16x8 *>(a.beta + ch * 8);
+    }
+}
+
+template <int NB, int NW, int NLW>
+__device__ __forceinline__ void tl_ln_rows(const TlLnOperands<NB, NW, NLW> &op, const TlArgs &a,
+                                           const f16 *stage0, int wave, int lane, int m0, f16 *Y, int N) {
     constexpr int lds = 16 * NB + 8;
-    constexpr int RPW = TL_BM / NW;
-    constexpr int NCH = (NW * NB * 2 + 63) / 64; // 16-byte pieces per lane and row
+    constexpr int NCH = TlLnOperands<NB, NW, NLW>::NCH;
+    constexpr int ROWS = TlLnOperands<NB, NW, NLW>::ROWS;
     const int npiece = N >> 3;
     const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int rr = 0; rr < RPW; rr++) {
-        const int r = wave * RPW + rr;
+    for (int k = 0; k < ROWS; k++) {
+        const int r = wave + k * NLW;
         const long row = (long)m0 + r;
-        if (row >= a.M)
+        if (r >= TL_BM || row >= a.M)
             break;
         f16x8 xv[NCH];
         float sum = 0.f;
@@ -238,8 +394,7 @@ __device__ __forceinline__ void tl_ln_rows(const TlArgs &a, const f16 *stage0, i
                 const int tile = ch / (2 * NB), c = ch - tile * (2 * NB);
                 const f16x8 y = *reinterpret_cast<const f16x8 *>(
                     stage0 + tile * tl_wave_stage_halves<NB>() + r * lds + c * 8);
-                const f16x8 sk = *reinterpret_cast<const f16x8 *>(a.skip + row * N + ch * 8);
-                xv[i] = y + sk; // half add, one rounding (kernels/skip_layernorm.cu:20)
+                xv[i] = y + op.skip[k][i]; // half add, one rounding (kernels/skip_layernorm.cu:20)
             }
 #pragma unroll
             for (int j = 0; j < 8; j++)
@@ -261,12 +416,11 @@ __device__ __forceinline__ void tl_ln_rows(const TlArgs &a, const f16 *stage0, i
         for (int i = 0; i < NCH; i++) {
             const int ch = lane + 64 * i;
             if (ch < npiece) {
-                const f16x8 gg = *reinterpret_cast<const f16x8 *>(a.gamma + ch * 8);
-                const f16x8 bb = *reinterpret_cast<const f16x8 *>(a.beta + ch * 8);
                 f16x8 o;
 #pragma unroll
                 for (int j = 0; j < 8; j++)
-                    o[j] = (f16)(((float)xv[i][j] - mean) * rstd * (float)gg[j] + (float)bb[j]);
+                    o[j] = (f16)(((float)xv[i][j] - mean) * rstd * (float)op.gamma[i][j] +
+                                 (float)op.beta[i][j]);
                 *reinterpret_cast<f16x8 *>(Y + row * N + ch * 8) = o;
             }
         }
@@ -326,7 +480,6 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_plan_kernel(const TlArgs 
     const int xrow16 = 16 * x.ldx * 2; // bytes between the two 16-row subtiles
     f16 *const stage0 = xs + TL_BM * x.ldx;
     f16 *const stage = stage0 + x.wave * tl_wave_stage_halves<NB>();
-    const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     const int per_rp = a.ncg * a.nlin;
 #ifdef TL_TRACE
     const unsigned long long tt0 = TL_TICK();
@@ -385,8 +538,7 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_plan_kernel(const TlArgs 
             if (x.bn0 + j < nbr)
                 b4[j] = *reinterpret_cast<const f16x4 *>(bias + (x.bn0 + j) * 16 + x.g4 * 4);
         }
-        const f16 *wbase = data + hi * 256 + x.c16 * 16 + x.khalf8; // + pair * 512
-        const int *obase = poff + hi;                               // + pair * 2
+        const unsigned lane_w = hi * 256 + x.c16 * 16 + x.khalf8; // lane's halves inside a 1 KB tile pair
 
         for (int c = 0; c < a.nchunk; c++) {
 #ifdef TL_TRACE
@@ -411,89 +563,19 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_plan_kernel(const TlArgs 
                 __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's part has landed
                 __syncthreads();                    // ... and everyone else's
             }
-            // the first four pairs of the stream
+            // the first pairs of the stream
             const int q0 = __builtin_amdgcn_readfirstlane(bvec);
             const int qend = __builtin_amdgcn_readlane(bvec, NB);
             const int qlast = max(qend - 1, q0);
-            f16x8 w0 = zero8, w1 = zero8, w2 = zero8, w3 = zero8;
-            int o0 = 0, o1 = 0, o2 = 0, o3 = 0;
-            if (q0 < qend) {
-                const int qa = q0, qb = min(q0 + 1, qlast), qc = min(q0 + 2, qlast), qd = min(q0 + 3, qlast);
-                o0 = obase[qa * 2];
-                w0 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qa * 512);
-                o1 = obase[qb * 2];
-                w1 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qb * 512);
-                o2 = obase[qc * 2];
-                w2 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qc * 512);
-                o3 = obase[qd * 2];
-                w3 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qd * 512);
-            }
+            f16x8 w[TL_DEPTH];
+            int o[TL_DEPTH];
+            tl_preload(data, poff, lane_w, hi, q0, qlast, w, o);
 #ifdef TL_TRACE
             const unsigned long long tb = TL_TICK();
             tpanel += tb - ta;
 #endif
-
-            if (q0 < qend) {
-                f32x4 cur0 = f32x4{0.f, 0.f, 0.f, 0.f}, cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
-                int j = 0;
-                int bend = __builtin_amdgcn_readlane(bvec, 1);
-                // leading empty block-rows (straight-line scalar code: loops
-                // in here would defeat the counted waits of the pipeline)
-#pragma unroll
-                for (int t = 0; t < NB - 1; t++) {
-                    j += (bend == q0 && j + 1 < NB) ? 1 : 0;
-                    bend = __builtin_amdgcn_readlane(bvec, j + 1);
-                }
-                // X operands are read one stage ahead (ping-pong xa0/xb0 <-> xa1/xb1)
-                f16x8 xa0 = *reinterpret_cast<const f16x8 *>(xlane + o0);
-                f16x8 xb0 = *reinterpret_cast<const f16x8 *>(xlane + o0 + xrow16);
-                f16x8 xa1 = zero8, xb1 = zero8;
-#define TL_STAGE(W_, O_, ONEXT_, XA_, XB_, XAN_, XBN_, I_)                                        \
-    {                                                                                             \
-        XAN_ = *reinterpret_cast<const f16x8 *>(xlane + ONEXT_);                                  \
-        XBN_ = *reinterpret_cast<const f16x8 *>(xlane + ONEXT_ + xrow16);                         \
-        cur0 = mfma16x16x32(W_, XA_, cur0);                                                       \
-        cur1 = mfma16x16x32(W_, XB_, cur1);                                                       \
-        {                                                                                         \
-            const int qn = min(q + (I_) + 4, qlast);                                              \
-            O_ = obase[qn * 2];                                                                   \
-            W_ = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qn * 512);                      \
-        }                                                                                         \
-        if (q + (I_) + 1 == bend) { /* block-row j is complete: acc[j] += cur, branch-free */     \
-            _Pragma("unroll") for (int k = 0; k < NB; k++) {                                      \
-                const float mk = (k == j) ? 1.0f : 0.0f;                                          \
-                _Pragma("unroll") for (int r = 0; r < 4; r++) {                                   \
-                    acc[k][0][r] = __builtin_fmaf(cur0[r], mk, acc[k][0][r]);                     \
-                    acc[k][1][r] = __builtin_fmaf(cur1[r], mk, acc[k][1][r]);                     \
-                }                                                                                 \
-            }                                                                                     \
-            cur0 = f32x4{0.f, 0.f, 0.f, 0.f};                                                     \
-            cur1 = f32x4{0.f, 0.f, 0.f, 0.f};                                                     \
-            j++;                                                                                  \
-            bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));                               \
-            _Pragma("unroll") for (int t = 0; t < NB - 2; t++) { /* skip empty block-rows */      \
-                j += (bend == q + (I_) + 1 && j + 1 < NB) ? 1 : 0;                                \
-                bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));                           \
-            }                                                                                     \
-        }                                                                                         \
-    }
-                int q = q0;
-                for (; q + 4 <= qend; q += 4) { // straight-line body: counted waits
-                    TL_STAGE(w0, o0, o1, xa0, xb0, xa1, xb1, 0)
-                    TL_STAGE(w1, o1, o2, xa1, xb1, xa0, xb0, 1)
-                    TL_STAGE(w2, o2, o3, xa0, xb0, xa1, xb1, 2)
-                    TL_STAGE(w3, o3, o0, xa1, xb1, xa0, xb0, 3)
-                }
-                if (q < qend) {
-                    TL_STAGE(w0, o0, o1, xa0, xb0, xa1, xb1, 0)
-                    if (q + 1 < qend) {
-                        TL_STAGE(w1, o1, o2, xa1, xb1, xa0, xb0, 1)
-                        if (q + 2 < qend)
-                            TL_STAGE(w2, o2, o3, xa0, xb0, xa1, xb1, 2)
-                    }
-                }
-#undef TL_STAGE
-            }
+            tl_stream<NB>(xlane, xrow16, data, poff, lane_w, hi, q0, qend, qlast, bvec, w, o,
+                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); });
 #ifdef TL_TRACE
             tlast = TL_TICK();
             tcomp += tlast - tb;
@@ -504,9 +586,11 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_plan_kernel(const TlArgs 
         const unsigned long long te = TL_TICK();
 #endif
         tl_epilogue_wave<NB, GELU, !LN>(a, x, stage, Yp, N, nbr, acc, b4);
-        if (LN) {
+        if constexpr (LN) {
+            TlLnOperands<NB, NW, NW> lnop;
+            tl_ln_fetch(lnop, a, x.wave, lane, x.m0, N);
             __syncthreads(); // every wave's part of the rows is staged
-            tl_ln_rows<NB, NW>(a, stage0, x.wave, lane, x.m0, Yp, N);
+            tl_ln_rows(lnop, a, stage0, x.wave, lane, x.m0, Yp, N);
             lds_used = true; // (the next item's panel load starts with a barrier)
         }
 #ifdef TL_TRACE
@@ -629,23 +713,15 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
         __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): this wave's part has landed */           \
         __syncthreads();                    /* ... and everyone else's */                         \
     }
-    // the first four pairs of an item's stream
+    // the first pairs of an item's stream
 #define TL_PRELOAD(t_, bvec_)                                                                     \
     {                                                                                             \
         q0 = __builtin_amdgcn_readfirstlane(bvec_);                                               \
         qend = __builtin_amdgcn_readlane(bvec_, NB);                                              \
         qlast = max(qend - 1, q0);                                                                \
-        wbase = (t_).data + lane_w;                                                               \
-        obase = (t_).poff + hi;                                                                   \
-        const int qb = min(q0 + 1, qlast), qc = min(q0 + 2, qlast), qd = min(q0 + 3, qlast);      \
-        o0 = obase[q0 * 2];                                                                       \
-        w0 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)q0 * 512);                          \
-        o1 = obase[qb * 2];                                                                       \
-        w1 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qb * 512);                          \
-        o2 = obase[qc * 2];                                                                       \
-        w2 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qc * 512);                          \
-        o3 = obase[qd * 2];                                                                       \
-        w3 = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qd * 512);                          \
+        wdata = (t_).data;                                                                        \
+        wpoff = (t_).poff;                                                                        \
+        tl_preload(wdata, wpoff, lane_w, hi, q0, qlast, w, o);                                    \
     }
 
     // Per-linear arguments are read from the kernel-argument segment with a
@@ -693,12 +769,10 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
     TL_BIAS(b4, cur)
     TL_PANEL(cur.rp)
     int q0, qend, qlast;
-    const f16 *wbase;
-    const int *obase;
-    f16x8 w0, w1, w2, w3;
-    int o0, o1, o2, o3;
-    // (an empty stream still loads pair q0: cptr's last entry is the padded
-    // tile count, and the plan's arrays hold one spare pair behind it)
+    const f16 *wdata;
+    const int *wpoff;
+    f16x8 w[TL_DEPTH];
+    int o[TL_DEPTH];
     TL_PRELOAD(cur, bvec)
 #ifdef TL_TRACE
     tlast = TL_TICK();
@@ -716,62 +790,18 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
         const unsigned long long ta = TL_TICK();
         tgap += ta - tlast;
 #endif
-        if (q0 < qend) {
-            f32x4 cur0 = f32x4{0.f, 0.f, 0.f, 0.f}, cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
-            int j = 0;
-            int bend = __builtin_amdgcn_readlane(bvec, 1);
-            // leading empty block-rows (straight-line scalar code: loops in
-            // here would defeat the counted waits of the pipeline)
+        // a finished block-row goes straight to the wave's staging tile
+        tl_stream<NB>(xlane, xrow16, wdata, wpoff, lane_w, hi, q0, qend, qlast, bvec, w, o,
+                      [&](int j, f32x4 c0, f32x4 c1) {
+                          // bias of block-row j as a 0/1-masked sum (exact); a chain
+                          // of selects over b4[] would be turned into an indexed
+                          // load and put the array into scratch memory
+                          f16x4 bj = f16x4{0, 0, 0, 0};
 #pragma unroll
-            for (int t = 0; t < NB - 1; t++) {
-                j += (bend == q0 && j + 1 < NB) ? 1 : 0;
-                bend = __builtin_amdgcn_readlane(bvec, j + 1);
-            }
-            f16x8 xa0 = *reinterpret_cast<const f16x8 *>(xlane + o0);
-            f16x8 xb0 = *reinterpret_cast<const f16x8 *>(xlane + o0 + xrow16);
-            f16x8 xa1 = zero8, xb1 = zero8;
-#define TL_STAGE(W_, O_, ONEXT_, XA_, XB_, XAN_, XBN_, I_)                                        \
-    {                                                                                             \
-        XAN_ = *reinterpret_cast<const f16x8 *>(xlane + ONEXT_);                                  \
-        XBN_ = *reinterpret_cast<const f16x8 *>(xlane + ONEXT_ + xrow16);                         \
-        cur0 = mfma16x16x32(W_, XA_, cur0);                                                       \
-        cur1 = mfma16x16x32(W_, XB_, cur1);                                                       \
-        {                                                                                         \
-            const int qn = min(q + (I_) + 4, qlast);                                              \
-            O_ = obase[qn * 2];                                                                   \
-            W_ = *reinterpret_cast<const f16x8 *>(wbase + (size_t)qn * 512);                      \
-        }                                                                                         \
-        if (q + (I_) + 1 == bend) { /* block-row j is complete */                                 \
-            f16x4 bj = b4[0];                                                                     \
-            _Pragma("unroll") for (int k = 1; k < NB; k++) bj = (j == k) ? b4[k] : bj;            \
-            tl_stage_tile<GELU>(stage_lane + j * 16, lds, cur0, cur1, bj);                        \
-            cur0 = f32x4{0.f, 0.f, 0.f, 0.f};                                                     \
-            cur1 = f32x4{0.f, 0.f, 0.f, 0.f};                                                     \
-            j++;                                                                                  \
-            bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));                               \
-            _Pragma("unroll") for (int t = 0; t < NB - 2; t++) { /* skip empty block-rows */      \
-                j += (bend == q + (I_) + 1 && j + 1 < NB) ? 1 : 0;                                \
-                bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));                           \
-            }                                                                                     \
-        }                                                                                         \
-    }
-            int q = q0;
-            for (; q + 4 <= qend; q += 4) { // straight-line body: counted waits
-                TL_STAGE(w0, o0, o1, xa0, xb0, xa1, xb1, 0)
-                TL_STAGE(w1, o1, o2, xa1, xb1, xa0, xb0, 1)
-                TL_STAGE(w2, o2, o3, xa0, xb0, xa1, xb1, 2)
-                TL_STAGE(w3, o3, o0, xa1, xb1, xa0, xb0, 3)
-            }
-            if (q < qend) {
-                TL_STAGE(w0, o0, o1, xa0, xb0, xa1, xb1, 0)
-                if (q + 1 < qend) {
-                    TL_STAGE(w1, o1, o2, xa1, xb1, xa0, xb0, 1)
-                    if (q + 2 < qend)
-                        TL_STAGE(w2, o2, o3, xa0, xb0, xa1, xb1, 2)
-                }
-            }
-#undef TL_STAGE
-        }
+                          for (int k = 0; k < NB; k++)
+                              bj += b4[k] * ((j == k) ? (f16)1 : (f16)0);
+                          tl_stage_tile<GELU>(stage_lane + j * 16, lds, c0, c1, bj);
+                      });
 #ifdef TL_TRACE
         const unsigned long long tb = TL_TICK();
         tcomp += tb - ta;
@@ -787,10 +817,12 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
         if (same_panel)
             TL_PRELOAD(nxt, bvec_n)
 
-        if (LN) {
+        if constexpr (LN) {
             // the workgroup holds whole rows: skip connection + LayerNorm here
+            TlLnOperands<NB, NW, NW> lnop;
+            tl_ln_fetch(lnop, a, wave, lane, cur.rp * TL_BM, cur.N);
             __syncthreads(); // every wave's part of the rows is staged
-            tl_ln_rows<NB, NW>(a, stage0, wave, lane, cur.rp * TL_BM, cur.Y, cur.N);
+            tl_ln_rows(lnop, a, stage0, wave, lane, cur.rp * TL_BM, cur.Y, cur.N);
             if (has_next && same_panel)
                 __syncthreads(); // the staging tiles are free again
         } else {
@@ -840,6 +872,174 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
 #endif
 #undef TL_BVEC
 #undef TL_KARG
+}
+
+// ---------------------------------------------------------------------------
+// Chunked fused kernel: linear + skip + LayerNorm for K beyond one LDS panel
+// (FFN2 of BERT-base, K = 3072, N = 768).  One workgroup per row panel holds
+// whole rows: twelve computing waves of NB block-rows each and a thirteenth
+// wave that does nothing but fetch.  K is walked in chunks through two LDS
+// panel buffers; the fetching wave requests chunk c+1 (global -> LDS DMA) as
+// soon as the computing waves have left chunk c-1, so the fetch runs under
+// chunk c's MFMAs.  It has to be a wave of its own: loads return in order
+// within a wave, so a panel request in a computing wave's queue would hold
+// back every weight pair requested after it.  One LDS-only barrier per chunk
+// hands over both "chunk c has landed" and "buffer (c+1)&1 is free".  The
+// computing waves run the pair stream and 4-stage pipeline of the plan kernel,
+// restarted per chunk with the first pairs requested before the barrier.
+// ---------------------------------------------------------------------------
+constexpr int TL_CWAVES = 12;
+constexpr int TL_CTHREADS = (TL_CWAVES + 1) * 64;
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences
+// global memory, which would make every wave drain the weight pairs it has
+// just requested; here only the panel buffers in LDS change hands.
+__device__ __forceinline__ void tl_barrier_lds() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+template <int NB>
+__global__ void __launch_bounds__(TL_CTHREADS) tile_linear_chunked_ln_kernel(const TlArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
+    f16 *xs = reinterpret_cast<f16 *>(tl_smem);
+    const int rp = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3);
+    if (rp >= a.total)
+        return;
+    TlCtx x;
+    x.lin = 0;
+    x.cg = 0;
+    x.m0 = rp * TL_BM;
+    x.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    x.lane = threadIdx.x & 63;
+    x.c16 = x.lane & 15;
+    x.g4 = x.lane >> 4;
+    x.khalf8 = (x.g4 & 1) * 8;
+    x.hi = x.lane >> 5;
+    x.ldx = a.KC + ((a.KC & 31) ? 0 : TL_PAD);
+    x.bn_wg = 0;
+    x.bn0 = x.wave * NB;
+    x.ld_r = x.ld_c = 0;
+    const int lane = x.lane;
+    const int pbuf = TL_BM * x.ldx; // halves per panel buffer
+    f16 *const stage0 = xs + 2 * pbuf;
+    f16 *const Yp = a.Y[0];
+    const int N = a.N[0];
+    const int nbr = N >> 4;
+#ifdef TL_TRACE
+    const unsigned long long tt0 = TL_TICK();
+    unsigned long long tpanel = 0, tcomp = 0, tepi = 0, tgap = 0, tlast = tt0;
+#endif
+
+    if (x.wave == TL_CWAVES) {
+        // ---- the fetching wave ----
+#define TL_FETCH(c_)                                                                              \
+    {                                                                                             \
+        const int pk0 = (c_) * a.KC;                                                              \
+        const int pcpr = min(a.KC, a.K - pk0) >> 3; /* 16-byte pieces per row, <= 124 */          \
+        f16 *dst = xs + ((c_) & 1) * pbuf;                                                        \
+        const int nrow = min(TL_BM, a.M - x.m0);                                                  \
+        for (int row = 0; row < nrow; row++) {                                                    \
+            const f16 *src = a.X + (size_t)(x.m0 + row) * a.K + pk0;                              \
+            if (lane < pcpr)                                                                      \
+                load_lds16(src + lane * 8, dst + row * x.ldx);                                    \
+            if (64 + lane < pcpr)                                                                 \
+                load_lds16(src + (64 + lane) * 8, dst + row * x.ldx + 512);                       \
+        }                                                                                         \
+    }
+        TL_FETCH(0)
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+        if (a.nchunk > 1)
+            TL_FETCH(1)
+        tl_barrier_lds(); // chunk 0 is in LDS
+        for (int c = 1; c < a.nchunk; c++) {
+#ifdef TL_TRACE
+            tlast = TL_TICK();
+#endif
+            __builtin_amdgcn_s_waitcnt(0x0F70); // chunk c has landed
+#ifdef TL_TRACE
+            { const unsigned long long t = TL_TICK(); tpanel += t - tlast; tlast = t; }
+#endif
+            tl_barrier_lds();                   // ... and every wave has left chunk c-1
+#ifdef TL_TRACE
+            tgap += TL_TICK() - tlast;
+#endif
+            if (c + 1 < a.nchunk)
+                TL_FETCH(c + 1)
+        }
+#undef TL_FETCH
+    } else {
+        // ---- the computing waves ----
+        const int *const cptr = a.cptr[0];
+        const int hi = x.hi;
+        f32x4 acc[NB][2];
+        f16x4 b4[NB];
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            acc[j][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+            acc[j][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+            b4[j] = f16x4{0, 0, 0, 0};
+            if (x.bn0 + j < nbr)
+                b4[j] = *reinterpret_cast<const f16x4 *>(a.bias[0] + (x.bn0 + j) * 16 + x.g4 * 4);
+        }
+        const int xrow16 = 16 * x.ldx * 2; // bytes between the two 16-row subtiles
+        const f16 *const data = a.data[0];
+        const int *const poff = a.row_offset[0];
+        const unsigned lane_w = hi * 256 + x.c16 * 16 + x.khalf8; // lane's halves inside a 1 KB tile pair
+        const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        // pair-index boundaries of the wave's block-rows in the current chunk
+        // (see tile_linear_plan_kernel); the next chunk's are requested a chunk ahead
+        int bvec = cptr[min(x.bn0 + min(lane, NB), nbr)] >> 1;
+
+        for (int c = 0; c < a.nchunk; c++) {
+            const char *xlane =
+                reinterpret_cast<const char *>(xs + (c & 1) * pbuf + x.c16 * x.ldx + x.khalf8);
+            const int q0 = __builtin_amdgcn_readfirstlane(bvec);
+            const int qend = __builtin_amdgcn_readlane(bvec, NB);
+            const int qlast = max(qend - 1, q0);
+            f16x8 w[TL_DEPTH];
+            int o[TL_DEPTH];
+            tl_preload(data, poff, lane_w, hi, q0, qlast, w, o);
+            const int cn = min(c + 1, a.nchunk - 1);
+            const int bvec_n = cptr[cn * nbr + min(x.bn0 + min(lane, NB), nbr)] >> 1;
+            const int bcur = bvec;
+#ifdef TL_TRACE
+            tlast = TL_TICK();
+#endif
+            tl_barrier_lds();
+#ifdef TL_TRACE
+            const unsigned long long tb = TL_TICK();
+            tgap += tb - tlast;
+#endif
+
+            tl_stream<NB>(xlane, xrow16, data, poff, lane_w, hi, q0, qend, qlast, bcur, w, o,
+                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); });
+#ifdef TL_TRACE
+            tcomp += TL_TICK() - tb;
+#endif
+            bvec = bvec_n;
+        }
+        f16 *stage = stage0 + x.wave * tl_wave_stage_halves<NB>();
+        tl_epilogue_wave<NB, false, false>(a, x, stage, Yp, N, nbr, acc, b4);
+    }
+#ifdef TL_TRACE
+    tlast = TL_TICK();
+#endif
+    TlLnOperands<NB, TL_CWAVES, TL_CWAVES + 1> lnop;
+    tl_ln_fetch(lnop, a, x.wave, lane, x.m0, N);
+    __syncthreads(); // every computing wave's part of the rows is staged
+    tl_ln_rows(lnop, a, stage0, x.wave, lane, x.m0, Yp, N);
+#ifdef TL_TRACE
+    tepi = TL_TICK() - tlast;
+    if (g_trace && lane == 0) {
+        unsigned hwid, xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        unsigned long long *t = g_trace + ((size_t)blockIdx.x * 16 + x.wave) * 8;
+        t[0] = tt0; t[1] = tpanel; t[2] = tcomp; t[3] = tepi; t[4] = TL_TICK(); t[5] = hwid; t[6] = xcc; t[7] = tgap;
+    }
+#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -1005,6 +1205,17 @@ static int ln_block_rows(int nbr) {
     return need <= 3 ? need : need == 4 ? 4 : need <= 6 ? 6 : 0;
 }
 
+template <int NB>
+static int launch_chunked_ln_inst(const TlArgs &a, size_t lds, hipStream_t st) {
+    auto k = tile_linear_chunked_ln_kernel<NB>;
+    ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_CTHREADS), lds, st, a);
+    return launch_status("tile_linear+LayerNorm (chunked) launch");
+}
+
+static int g_tile_ln_chunked = 1;
+
 static int tile_launch_ln(const TlProblem &p, const f16 *X, int M, int K, int KC, int nchunk,
                           const f16 *skip, const f16 *gamma, const f16 *beta, hipStream_t st) {
     TlArgs a;
@@ -1030,9 +1241,21 @@ static int tile_launch_ln(const TlProblem &p, const f16 *X, int M, int K, int KC
     a.skip = skip;
     a.gamma = gamma;
     a.beta = beta;
+    const size_t lds_x = (size_t)TL_BM * (KC + ((KC & 31) ? 0 : TL_PAD)) * sizeof(f16);
+    // K in chunks and rows narrow enough for twelve waves of <= 4 block-rows:
+    // the double-buffered kernel with a fetching wave
+    const int cnb = (p.nbr + TL_CWAVES - 1) / TL_CWAVES;
+    if (nchunk > 1 && cnb <= 4 && g_tile_ln_chunked) {
+        const size_t lds = 2 * lds_x + (size_t)TL_CWAVES * TL_BM * (16 * cnb + 8) * sizeof(f16);
+        switch (cnb) {
+        case 1: return launch_chunked_ln_inst<1>(a, lds, st);
+        case 2: return launch_chunked_ln_inst<2>(a, lds, st);
+        case 3: return launch_chunked_ln_inst<3>(a, lds, st);
+        default: return launch_chunked_ln_inst<4>(a, lds, st);
+        }
+    }
     const int nb = ln_block_rows(p.nbr);
-    const size_t lds = (size_t)TL_BM * (KC + ((KC & 31) ? 0 : TL_PAD)) * sizeof(f16) +
-                       (size_t)TL_LN_WAVES * TL_BM * (16 * nb + 8) * sizeof(f16);
+    const size_t lds = lds_x + (size_t)TL_LN_WAVES * TL_BM * (16 * nb + 8) * sizeof(f16);
     switch (nb) {
     case 1: return launch_ln_inst<1>(a, lds, st);
     case 2: return launch_ln_inst<2>(a, lds, st);
@@ -1174,6 +1397,10 @@ extern "C" int et_tuning_set(const char *key, int value) {
     }
     if (key && !strcmp(key, "tile_ipw")) {
         et::g_tile_ipw = value;
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "tile_ln_chunked")) {
+        et::g_tile_ln_chunked = value;
         return ET_OK;
     }
     if (key && !strcmp(key, "tile_fuse_ln")) {
