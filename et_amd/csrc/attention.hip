@@ -16,10 +16,14 @@
 //     (xor 16, xor 32) and the running statistics are per-lane scalars.
 //   O^T(d x queries) = V^T * P^T : the P values a lane already holds are, as
 //     they stand, the B operand (8 k-slots = 4 keys of subtile 2kk + 4 keys
-//     of subtile 2kk+1); the matching A operand is read from a V tile that was
-//     transposed while being staged into LDS.  P never goes through LDS and
-//     the O accumulator's query index is again the lane's c, so the online
-//     rescale is a per-lane multiply.
+//     of subtile 2kk+1); the matching A operand is a V^T fragment, which the
+//     LDS transpose read (ds_read_b64_tr_b16) produces from a V tile kept in
+//     its natural [key][d] layout (the pruned variant transposes V while
+//     staging it instead).  P never goes through LDS and the O accumulator's
+//     query index is again the lane's c, so the online rescale is a per-lane
+//     multiply.
+// K and V tiles of the unpruned variants are staged by DMA (global -> LDS
+// without registers), double-buffered, one tile ahead of the MFMAs.
 #include "common.h"
 
 #include <cmath>
@@ -65,7 +69,14 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
     constexpr int LDV = AT_KT + 8;
     constexpr int QB = AT_WAVES * 16 * QS; // queries per workgroup
     constexpr int LDO = HD + 8;
-    constexpr int KBUF = AT_KT * LDK, VBUF = HD * LDV;
+    // Unpruned operands are staged by DMA (global -> LDS, no registers) in their
+    // natural [key][d] layout, K and V alike; the transposed V^T fragments the
+    // second contraction needs are then produced by the LDS transpose read
+    // (ds_read_b64_tr_b16).  The pruned variant gathers ragged column sets and
+    // keeps the register path, which transposes V while storing it.
+    constexpr bool DMA = !PRUNED;
+    constexpr int LDVN = HD + 16; // V row stride in the natural layout (as LDK)
+    constexpr int KBUF = AT_KT * LDK, VBUF = DMA ? AT_KT * LDVN : HD * LDV;
     constexpr int SM_KV = 2 * (KBUF + VBUF); // double-buffered key/value tiles
     constexpr int SM_O = QB * LDO;
     constexpr int SM = SM_KV > SM_O ? SM_KV : SM_O;
@@ -228,17 +239,50 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 }
             }
         };
+        // DMA staging of one tile: every instruction moves 64 x 16 bytes to 1 KB
+        // of consecutive LDS, so a lane's LDS position decides which (row,
+        // column) it fetches; lanes that land in the row padding fetch the
+        // row's first bytes.  Rows at or beyond len re-read the last valid row
+        // (their scores are masked to -inf / their P is 0).
+        auto dma_tile = [&](int kb, int buf) {
+            constexpr int ROWB = LDK * 2;                // LDS bytes per row, K and V alike
+            constexpr int NINST = AT_KT * ROWB / 1024;   // per operand
+            static_assert(AT_KT * ROWB % 1024 == 0, "tile is a whole number of DMA instructions");
+            constexpr int NTOT = (SHAREDQK ? 1 : 2) * NINST;
+            f16 *ks = smem + buf * (KBUF + VBUF);
+            f16 *vs = ks + KBUF;
+#pragma unroll
+            for (int i0 = 0; i0 < NTOT; i0 += AT_WAVES) {
+                const int i = i0 + wave;
+                if (NTOT % AT_WAVES != 0 && i >= NTOT)
+                    break;
+                const bool isv = SHAREDQK || i >= NINST;
+                const int ii = (!SHAREDQK && isv) ? i - NINST : i;
+                const int p = ii * 1024 + lane * 16;
+                const int row = p / ROWB, cb = p - row * ROWB;
+                const int rr = min(kb + row, len - 1);
+                const int col = cb < HD * 2 ? (cb >> 1) : 0;
+                const f16 *src = isv ? a.V + (size_t)(row0 + rr) * a.ldv + vc0 + col
+                                     : a.K + (size_t)(row0 + rr) * a.ldq + qc0 + col;
+                load_lds16(src, (isv ? vs : ks) + ii * 512);
+            }
+        };
         typedef std::integral_constant<bool, true> yes_t;
         typedef std::integral_constant<bool, false> no_t;
 
         const int nt = (len + AT_KT - 1) / AT_KT;
         // all of this wave's query rows valid?  (wave-uniform)
         const bool wave_rows_ok = q0 + (wave + 1) * QS * 16 <= len;
-        if (AT_KT <= len)
-            load_tile(0, yes_t{});
-        else
-            load_tile(0, no_t{});
-        store_tile(0);
+        if (DMA) {
+            dma_tile(0, 0);
+            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+        } else {
+            if (AT_KT <= len)
+                load_tile(0, yes_t{});
+            else
+                load_tile(0, no_t{});
+            store_tile(0);
+        }
         __syncthreads();
 
         // Additive mask values of one tile, in the score layout.  They are
@@ -411,9 +455,23 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 for (int d = 0; d < DV; d++)
 #pragma unroll
                     for (int kk = 0; kk < 2; kk++) {
-                        const f16 *vrow = vt + (d * 16 + c16) * LDV + kk * 32 + g4 * 4;
-                        const f16x4 v0 = *reinterpret_cast<const f16x4 *>(vrow);
-                        const f16x4 v1 = *reinterpret_cast<const f16x4 *>(vrow + 16);
+                        f16x4 v0, v1;
+                        if (DMA) {
+                            // natural layout [key][d]: the transpose read hands lane
+                            // c of a 16-lane group the 4 consecutive keys of column
+                            // d0+c when lane i of the group addresses row i/4,
+                            // columns 4(i%4)..+3.  The B operand's 8 k-slots are
+                            // keys 4g..4g+3 of subtile 2kk and of subtile 2kk+1.
+                            typedef short s16x4 __attribute__((ext_vector_type(4)));
+                            typedef __attribute__((address_space(3))) s16x4 *lds4;
+                            const f16 *vrow = vt + (kk * 32 + g4 * 4 + (c16 >> 2)) * LDVN + d * 16 + (c16 & 3) * 4;
+                            v0 = __builtin_bit_cast(f16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds4)vrow));
+                            v1 = __builtin_bit_cast(f16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds4)(vrow + 16 * LDVN)));
+                        } else {
+                            const f16 *vrow = vt + (d * 16 + c16) * LDV + kk * 32 + g4 * 4;
+                            v0 = *reinterpret_cast<const f16x4 *>(vrow);
+                            v1 = *reinterpret_cast<const f16x4 *>(vrow + 16);
+                        }
                         vfr[d][kk] = f16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
                     }
 #pragma unroll
@@ -431,8 +489,14 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
             const f16 *ks = smem + (t & 1) * (KBUF + VBUF);
             const f16 *vt = ks + KBUF;
             const bool more = t + 1 < nt;
-            if (more) { // tile t+1: global loads in flight while tile t is consumed
-                if (kb + 2 * AT_KT <= len)
+            // tile t+1 goes into the other buffer (last read in iteration t-1,
+            // which every wave left before the previous barrier) while tile t is
+            // consumed: by DMA straight away, or through registers that are
+            // stored after the tile body
+            if (more) {
+                if (DMA)
+                    dma_tile(kb + AT_KT, (t + 1) & 1);
+                else if (kb + 2 * AT_KT <= len)
                     load_tile(kb + AT_KT, yes_t{});
                 else
                     load_tile(kb + AT_KT, no_t{});
@@ -441,10 +505,12 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 tile_body(kb, ks, vt, yes_t{});
             else
                 tile_body(kb, ks, vt, no_t{});
-            // publish tile t+1 into the other buffer (last read in iteration
-            // t-1, which every wave left before the previous barrier)
-            if (more)
-                store_tile((t + 1) & 1);
+            if (more) {
+                if (DMA)
+                    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's part of tile t+1 has landed
+                else
+                    store_tile((t + 1) & 1);
+            }
             __syncthreads();
         }
 
@@ -552,15 +618,16 @@ qk_scores_kernel(f16 *__restrict__ QK, const f16 *__restrict__ Q, const f16 *__r
 }
 
 // LDS bytes of one workgroup (mirrors the constants inside the kernel)
-template <int HD, int QS, int NW> constexpr size_t attn_lds_bytes() {
-    constexpr int KV = 2 * (AT_KT * (HD + 16) + HD * (AT_KT + 8));
+template <int HD, int QS, int NW, bool PRUNED> constexpr size_t attn_lds_bytes() {
+    // (must agree with the kernel's KBUF / VBUF)
+    constexpr int KV = 2 * (AT_KT * (HD + 16) + (PRUNED ? HD * (AT_KT + 8) : AT_KT * (HD + 16)));
     constexpr int O = NW * 16 * QS * (HD + 8);
     return sizeof(f16) * (size_t)(KV > O ? KV : O);
 }
 
 template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK>
 static void attn_launch_one(const AttnArgs &a, hipStream_t st) {
-    constexpr size_t lds = attn_lds_bytes<HD, QS, NW>();
+    constexpr size_t lds = attn_lds_bytes<HD, QS, NW, PRUNED>();
     auto kern = attention_kernel<HD, QS, NW, PRUNED, SHAREDQK>;
     if (lds > 64 * 1024) { // above the default dynamic-LDS limit: opt in once per kernel
         static bool done = false;
