@@ -124,6 +124,9 @@ def main():
     # ---- same launch sequence with HIP events around every kernel
     L = mk_linears()
     mask = torch.from_numpy(mask_h).to(dev)
+    # as Encoder_base does at construction: let the launcher skip the mask's all-zero tiles
+    mask_summary = K.attention_mask_summary(mask, S)
+    K.attention_mask_summary_attach(mask, S, mask_summary)
     gam = [torch.from_numpy(t).to(dev) for t in ln]
     b = [torch.empty((T, D), dtype=torch.float16, device=dev) for _ in range(4)]
     ffn = torch.empty((T, DFF), dtype=torch.float16, device=dev)

@@ -27,7 +27,9 @@
 #include "common.h"
 
 #include <cmath>
+#include <mutex>
 #include <type_traits>
+#include <vector>
 
 namespace et {
 
@@ -38,6 +40,11 @@ struct AttnArgs {
     const f16 *Q, *K, *V, *QK, *mask;
     const int *seq_lens, *cu_seqlens;
     const int *qk_head_ptr, *v_col_id, *v_head_ptr;
+    // optional: one bit per (16 query rows, 64-key tile) of the mask, set when
+    // any of its elements is non-zero (et_attention_mask_summary); msum_words
+    // 32-bit words per group of 16 rows
+    const unsigned *msum;
+    int msum_words;
     int ldq, ldv, ldo, seq_len, nhead, batch, nqb, total, per_xcd;
     float log2_scale, scale;
 };
@@ -285,6 +292,30 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
         }
         __syncthreads();
 
+        // Does key tile t hold a non-zero mask element for this wave's query
+        // rows?  (wave-uniform; all-zero tiles skip the mask loads and adds,
+        // which changes no result bit: s + 0 == s.)  The summary words of the
+        // first 64 tiles are fetched once, up front; longer sequences do not
+        // use the summary.
+        unsigned mw0 = 0xFFFFFFFFu, mw1 = 0xFFFFFFFFu;
+        if (a.msum && a.msum_words <= 2) {
+            unsigned w0 = 0, w1 = 0;
+#pragma unroll
+            for (int qs = 0; qs < QS; qs++) {
+                const int g = (q0 + (wave * QS + qs) * 16) >> 4;
+                if (g * 16 < a.seq_len) {
+                    w0 |= a.msum[(size_t)g * a.msum_words];
+                    if (a.msum_words > 1)
+                        w1 |= a.msum[(size_t)g * a.msum_words + 1];
+                }
+            }
+            mw0 = __builtin_amdgcn_readfirstlane(w0);
+            mw1 = __builtin_amdgcn_readfirstlane(w1);
+        }
+        auto tile_has_mask = [&](int t) -> bool {
+            return t >= 64 || (((t < 32 ? mw0 : mw1) >> (t & 31)) & 1u);
+        };
+
         // Additive mask values of one tile, in the score layout.  They are
         // requested one tile ahead (right after the previous tile consumed
         // its own) so the L2 latency is covered by a whole tile of work.
@@ -317,7 +348,8 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
         };
         const bool vec_ok = (!a.mask || mask_vec) && (!SHAREDQK || qk_vec);
         auto fast_tile = [&](int kb) { return kb + AT_KT <= len && wave_rows_ok && vec_ok; };
-        if (a.mask) {
+        bool has_mask_cur = a.mask && tile_has_mask(0);
+        if (has_mask_cur) {
             if (fast_tile(0))
                 load_mask(0, yes_t{});
             else
@@ -327,8 +359,10 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
         // One key tile.  FAST: all 64 keys and all of the wave's query rows are
         // valid and the vector paths apply, so the body has no per-lane
         // predicates at all.
-        auto tile_body = [&](int kb, const f16 *ks, const f16 *vt, auto fast_c) {
+        bool has_mask_next = false;
+        auto tile_body = [&](int kb, const f16 *ks, const f16 *vt, auto fast_c, auto masked_c) {
             constexpr bool FAST = decltype(fast_c)::value;
+            constexpr bool MASKED = decltype(masked_c)::value; // this tile's mask values are in mk
             // ---- scores, transposed: st[ksub][qs][r] = S[q = c16][key = 16 ksub + 4 g4 + r]
             f32x4 st[4][QS];
             if (!SHAREDQK) {
@@ -383,7 +417,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
             // more than 8 binades (P then stays <= 256, exact enough in half),
             // so after the first tiles the accumulator rescale is skipped.
             f16x8 pf[QS][2];
-            if (a.mask) {
+            if (MASKED) {
 #pragma unroll
                 for (int qs = 0; qs < QS; qs++)
 #pragma unroll
@@ -391,7 +425,10 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
 #pragma unroll
                         for (int r = 0; r < 4; r++)
                             st[ksub][qs][r] += (float)mk[qs][ksub][r];
-                if (kb + AT_KT < len) { // next tile's mask
+            }
+            if (a.mask) { // next tile's mask
+                has_mask_next = kb + AT_KT < len && tile_has_mask((kb + AT_KT) / AT_KT);
+                if (has_mask_next) {
                     if (fast_tile(kb + AT_KT))
                         load_mask(kb + AT_KT, yes_t{});
                     else
@@ -501,10 +538,18 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 else
                     load_tile(kb + AT_KT, no_t{});
             }
-            if (fast_tile(kb))
-                tile_body(kb, ks, vt, yes_t{});
-            else
-                tile_body(kb, ks, vt, no_t{});
+            if (has_mask_cur) {
+                if (fast_tile(kb))
+                    tile_body(kb, ks, vt, yes_t{}, yes_t{});
+                else
+                    tile_body(kb, ks, vt, no_t{}, yes_t{});
+            } else {
+                if (fast_tile(kb))
+                    tile_body(kb, ks, vt, yes_t{}, no_t{});
+                else
+                    tile_body(kb, ks, vt, no_t{}, no_t{});
+            }
+            has_mask_cur = has_mask_next;
             if (more) {
                 if (DMA)
                     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's part of tile t+1 has landed
@@ -658,6 +703,59 @@ static float head_scale(int hd) {
     return (float)(f16)sqrtf(1.0f / (float)hd);
 }
 
+// ---- mask summary: one bit per (16 query rows, 64-key tile) ----------------
+// One wave per group of 16 rows; per tile a lane tests 16 elements (row
+// lane/4, keys 16*(lane%4)..+15) and the wave's ballot gives the bit.
+__global__ void __launch_bounds__(64) mask_summary_kernel(const f16 *mask, int seq_len, unsigned *out,
+                                                          int words) {
+    const int g = blockIdx.x;
+    const int lane = threadIdx.x;
+    const int row = g * 16 + (lane >> 2);
+    const int nt = (seq_len + AT_KT - 1) / AT_KT;
+    const uint16_t *m = reinterpret_cast<const uint16_t *>(mask);
+    for (int w = 0; w < words; w++) {
+        unsigned bits = 0;
+        for (int t = w * 32; t < min(nt, w * 32 + 32); t++) {
+            bool nz = false;
+            if (row < seq_len) {
+                const int k0 = t * AT_KT + (lane & 3) * 16;
+                for (int j = 0; j < 16; j++)
+                    if (k0 + j < seq_len && (m[(size_t)row * seq_len + k0 + j] & 0x7FFFu) != 0)
+                        nz = true; // anything but +0 / -0
+            }
+            if (__builtin_amdgcn_ballot_w64(nz) != 0)
+                bits |= 1u << (t & 31);
+        }
+        if (lane == 0)
+            out[(size_t)g * words + w] = bits;
+    }
+}
+
+static int mask_summary_words(int seq_len) { return ((seq_len + AT_KT - 1) / AT_KT + 31) / 32; }
+
+// summaries registered for a mask pointer (et_attention_mask_summary_attach)
+struct MaskSummaryEntry {
+    const void *mask;
+    const unsigned *summary;
+    int seq_len;
+};
+static std::mutex g_msum_mutex;
+static std::vector<MaskSummaryEntry> g_msum;
+
+static void attach_mask_summary(AttnArgs &a) {
+    a.msum = nullptr;
+    a.msum_words = 0;
+    if (!a.mask)
+        return;
+    std::lock_guard<std::mutex> lock(g_msum_mutex);
+    for (const MaskSummaryEntry &e : g_msum)
+        if (e.mask == a.mask && e.seq_len == a.seq_len) {
+            a.msum = e.summary;
+            a.msum_words = mask_summary_words(a.seq_len);
+            return;
+        }
+}
+
 static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedqk,
                               hipStream_t st, const char *who) {
     ET_REQUIRE(a.out && a.V, ET_ERR_INVALID_ARG, "%s: null pointer", who);
@@ -676,6 +774,7 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
     }
     a.ldo = d_model;
     a.scale = head_scale(hd);
+    attach_mask_summary(a);
     // 128 query rows per workgroup when that still fills the chip, else 64
     int variant = 0;
     {
@@ -822,4 +921,34 @@ extern "C" int et_qk_scores(void *QK, const void *Q, const void *K, int seq_len,
     else
         hipLaunchKernelGGL(qk_scores_kernel<128>, grid, block, 0, st, o, q, k, seq_len, d_model, nhead, scale);
     return launch_status("et_qk_scores");
+}
+
+extern "C" size_t et_attention_mask_summary_bytes(int seq_len) {
+    if (seq_len <= 0)
+        return 0;
+    return (size_t)((seq_len + 15) / 16) * et::mask_summary_words(seq_len) * sizeof(unsigned);
+}
+
+extern "C" int et_attention_mask_summary(const void *mask, int seq_len, void *summary, void *stream) {
+    using namespace et;
+    ET_REQUIRE(mask && summary, ET_ERR_INVALID_ARG, "et_attention_mask_summary: null pointer");
+    ET_REQUIRE(seq_len > 0, ET_ERR_INVALID_ARG, "et_attention_mask_summary: seq_len=%d", seq_len);
+    hipLaunchKernelGGL(mask_summary_kernel, dim3((seq_len + 15) / 16), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const f16 *>(mask), seq_len,
+                       static_cast<unsigned *>(summary), mask_summary_words(seq_len));
+    return launch_status("et_attention_mask_summary launch");
+}
+
+extern "C" int et_attention_mask_summary_attach(const void *mask, int seq_len, const void *summary) {
+    using namespace et;
+    ET_REQUIRE(mask && seq_len > 0, ET_ERR_INVALID_ARG, "et_attention_mask_summary_attach: bad arguments");
+    std::lock_guard<std::mutex> lock(g_msum_mutex);
+    for (size_t i = 0; i < g_msum.size(); i++)
+        if (g_msum[i].mask == mask && g_msum[i].seq_len == seq_len) {
+            g_msum.erase(g_msum.begin() + i);
+            break;
+        }
+    if (summary)
+        g_msum.push_back({mask, static_cast<const unsigned *>(summary), seq_len});
+    return ET_OK;
 }

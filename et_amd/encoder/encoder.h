@@ -26,6 +26,7 @@ class Encoder_base {
     Weight<half> ln_beta[2];
     Weight<half> mask;  // [seq_len x seq_len] additive, shared by heads and batch
     bool has_mask;
+    unsigned *mask_summary; // which 16x64 regions of the mask are non-zero (et_attention_mask_summary)
     void *stream;       // hipStream_t; NULL = default stream
     float log2_scale;   // 1 = base-2 softmax of the reference, log2(e) = textbook
     // per-sequence lengths (optional)
@@ -44,14 +45,28 @@ class Encoder_base {
         : d_model(d_model_), seq_len(seq_len_), nheads(nheads_), batch(batch_), buffer(buffer_),
           ln_gamma{Weight<half>(ln_gamma_1, d_model_), Weight<half>(ln_gamma_2, d_model_)},
           ln_beta{Weight<half>(ln_beta_1, d_model_), Weight<half>(ln_beta_2, d_model_)},
-          has_mask(mask_ != nullptr), stream(nullptr), log2_scale(1.0f),
+          has_mask(mask_ != nullptr), mask_summary(nullptr), stream(nullptr), log2_scale(1.0f),
           total_rows(batch_ * seq_len_) {
-        if (mask_)
+        if (mask_) {
             mask = Weight<half>(mask_, seq_len_ * seq_len_);
+            // the mask never changes after construction: let the attention
+            // launchers skip its all-zero tiles
+            etChk(et_malloc((void **)&mask_summary, et_attention_mask_summary_bytes(seq_len_)));
+            etChk(et_attention_mask_summary(mask.get(), seq_len_, mask_summary, nullptr));
+            etChk(et_device_synchronize());
+            etChk(et_attention_mask_summary_attach(mask.get(), seq_len_, mask_summary));
+        }
         for (int i = 0; i < buffer_num; i++)
             buffers[i] = buffer + (size_t)i * batch * seq_len * d_model;
     }
-    virtual ~Encoder_base() {}
+    virtual ~Encoder_base() {
+        if (mask_summary) {
+            et_attention_mask_summary_attach(mask.get(), seq_len, nullptr);
+            et_free(mask_summary);
+        }
+    }
+    Encoder_base(const Encoder_base &) = delete;
+    Encoder_base &operator=(const Encoder_base &) = delete;
     virtual void run(half *out, half *in) = 0; // device pointers; out may alias in
     static size_t buffer_size(int d_model_, int seq_len_, int /*nheads_*/, int batch_ = 1) {
         return (size_t)buffer_num * d_model_ * seq_len_ * batch_ * sizeof(half);

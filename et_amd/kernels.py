@@ -125,3 +125,16 @@ def scatter_cols(x, col_id, width):
     out = torch.empty((rows, width), dtype=torch.float16, device=x.device)
     check(lib().et_scatter_cols(_h(out), _h(x), _i32(col_id), rows, col_id.numel(), ld, width, _stream()))
     return out
+
+
+def attention_mask_summary(mask, seq_len):
+    """Per-(16 rows x 64 keys) non-zero bits of an additive mask; attach() lets the
+    attention launchers skip the all-zero tiles of that mask tensor."""
+    nbytes = lib().et_attention_mask_summary_bytes(seq_len)
+    out = torch.empty((nbytes // 4,), dtype=torch.int32, device=mask.device)
+    check(lib().et_attention_mask_summary(_h(mask), seq_len, _p(out), _stream()))
+    return out
+
+
+def attention_mask_summary_attach(mask, seq_len, summary):
+    check(lib().et_attention_mask_summary_attach(_h(mask), seq_len, None if summary is None else _p(summary)))

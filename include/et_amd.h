@@ -86,6 +86,19 @@ int et_OTF_attention(void *out, const void *Q, const void *K, const void *V,
                      int batch, const int *seq_lens, float log2_scale,
                      void *stream);
 
+/* Optional accelerator for masks with all-zero regions (the usual padding
+ * mask): a summary holds one bit per (16 query rows, 64 keys) of the mask,
+ * set when any element there is not +-0.  A launcher that is handed a mask
+ * pointer with an attached summary skips the mask loads and additions for
+ * all-zero tiles; s + 0 == s, so no result bit changes.  The caller computes
+ * the summary once (device buffer of et_attention_mask_summary_bytes), attaches
+ * it to the mask pointer, and detaches it (summary = NULL) before the mask
+ * changes or is freed.  No counterpart in the reference, which adds the mask
+ * unconditionally (kernels/attention.cu:79-84). */
+size_t et_attention_mask_summary_bytes(int seq_len);
+int et_attention_mask_summary(const void *mask, int seq_len, void *summary, void *stream);
+int et_attention_mask_summary_attach(const void *mask, int seq_len, const void *summary);
+
 /* Variable-length (packed) form of et_OTF_attention for the
  * sequence-length-aware path: rows of sequence b are
  * cu_seqlens[b]..cu_seqlens[b+1]-1 of out/Q/K/V (no padding rows exist);

@@ -251,6 +251,45 @@ def test_otf_attention_closed_forms(K):
     assert np.abs(got.astype(np.float64) - 1).max() <= 2.0 ** -10   # rows of P sum to 1
 
 
+@pytest.mark.parametrize("S", [512, 200, 2100])
+def test_attention_mask_summary(K, S):
+    """summary bits == any non-zero element per (16 rows, 64 keys); attention with an attached
+    summary is bit-identical to attention without, for zero, block-structured and dense masks"""
+    r = rng(45 + S)
+    H, d, B = 4, 256, 1
+    nt, ng = (S + 63) // 64, (S + 15) // 16
+    words = (nt + 31) // 32
+    mask = np.zeros((S, S), np.float16)
+    mask[:, S - S // 3:] = -30000.0               # padding-style: the last third of the keys
+    mask[37, 5] = 0.25                            # one stray element
+    mask[S - 1, 0] = np.float16(-0.0)             # -0 counts as zero
+    md = dev(mask)
+    summ = K.attention_mask_summary(md, S)
+    got_bits = host(summ).view(np.uint32).reshape(ng, words)
+    want_bits = np.zeros((ng, words), np.uint32)
+    nz = (mask.view(np.uint16) & 0x7FFF) != 0
+    for g in range(ng):
+        for t in range(nt):
+            if nz[g * 16:(g + 1) * 16, t * 64:(t + 1) * 64].any():
+                want_bits[g, t // 32] |= np.uint32(1) << np.uint32(t % 32)
+    assert np.array_equal(got_bits, want_bits)
+    if S > 1024:
+        return
+    Q, Kk, V = (randn_h(r, (B * S, d)) for _ in range(3))
+    for m in (mask, np.zeros((S, S), np.float16), randn_h(r, (S, S))):
+        md = dev(m)
+        plain = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), md, S, H, B, None, 1.0))
+        summ = K.attention_mask_summary(md, S)
+        K.attention_mask_summary_attach(md, S, summ)
+        try:
+            fast = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), md, S, H, B, None, 1.0))
+        finally:
+            K.attention_mask_summary_attach(md, S, None)
+        assert np.array_equal(plain, fast)
+        want = orc.otf_attention(Q, Kk, V, m, S, H, B, None, 1.0, f64=True)
+        check_close(fast, want, max_abs=5e-3, mean_rel=1e-3, what="attention with mask summary")
+
+
 def test_otf_attention_varlen_equals_padded(K):
     r = rng(42)
     S, H, d, B = 256, 12, 768, 4
