@@ -244,11 +244,20 @@ int et_stream_destroy(void *stream);
 int et_stream_synchronize(void *stream);
 int et_device_synchronize(void);
 /* Launch-heuristic overrides for benchmarking sweeps; value 0 restores the
- * automatic choice.  Keys: "tile_nb" (block-rows of W per wave in the tile
- * linear: 1,2,3,4,6), "tile_min_wgs" (workgroups the automatic choice aims
- * for), "attn_variant" (0: 4 waves x 32 query rows, 1: 8 waves x 16 rows,
- * 2: 4 waves x 16 rows; -1 automatic).  Not thread-safe; results never depend
- * on these beyond fp32 summation order. */
+ * automatic choice unless noted.  Keys:
+ *   "tile_nb"         block-rows of W per wave in the tile linear (1, 2, 3; the
+ *                     raw launchers also take 4 and 6)
+ *   "tile_min_wgs"    workgroups the automatic choices aim for (default 512)
+ *   "tile_ipw"        work items per persistent workgroup of a planned linear
+ *   "tile_fuse_ln"    0: et_tile_plan_run_ln runs the linear and the LayerNorm
+ *                     as two launches; 1 (default): fused where the rows fit
+ *   "tile_ln_chunked" 0: fused LayerNorm with K > 992 uses the single-buffer
+ *                     kernel; 1 (default): the double-buffered one
+ *   "ln_rows"         rows per wave of et_skip_layernorm (1, 2, 4)
+ *   "attn_variant"    0: 4 waves x 32 query rows, 1: 8 waves x 16 rows,
+ *                     2: 4 waves x 16 rows; -1 automatic
+ * Not thread-safe; results never depend on these beyond fp32 summation
+ * order. */
 int et_tuning_set(const char *key, int value);
 /* number of compute units of the current device (0 if none) */
 int et_device_cu_count(void);
