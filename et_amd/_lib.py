@@ -37,6 +37,14 @@ PROTOTYPES = {
     "et_tile_plan_ln_fusable": (_i, [_vp]),
     "et_tile_plan_run_multi": (_i, [C.POINTER(_vp), C.POINTER(_vp), _i, _vp, _i, _vp]),
     "et_tile_plan_query": (_i, [_vp, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
+    "et_prune_tile_mat": (_i, [_vp, _i, _i, _f, _ip, _ip]),
+    "et_prune_row_mat": (_i, [_vp, _i, _i, _f, _ip]),
+    "et_tile_mat_save": (_i, [C.c_char_p, _i, _i, _i, _ip, _ip, _vp, _vp]),
+    "et_tile_mat_peek": (_i, [C.c_char_p, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
+    "et_tile_mat_load": (_i, [C.c_char_p, _ip, _ip, _vp, _vp]),
+    "et_row_mat_save": (_i, [C.c_char_p, _i, _i, _i, _ip, _vp, _vp]),
+    "et_row_mat_peek": (_i, [C.c_char_p, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
+    "et_row_mat_load": (_i, [C.c_char_p, _ip, _vp, _vp]),
     "et_gen_sparse_tile_mat": (_i, [_i, _i, _f, _u64, _ip, _ip]),
     "et_gen_sparse_row_mat": (_i, [_i, _f, _u64, _ip]),
     "et_gen_head_balanced_rows": (_i, [_i, _i, _i, _u64, _ip]),

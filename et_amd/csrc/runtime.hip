@@ -94,6 +94,7 @@ const char *et_strerror(int code) {
     case ET_ERR_UNSUPPORTED: return "unsupported shape";
     case ET_ERR_HIP: return "HIP runtime error";
     case ET_ERR_FORMAT: return "malformed pruned-weight format";
+    case ET_ERR_IO: return "file could not be opened, read or written";
     default: return "unknown error";
     }
 }

@@ -59,3 +59,69 @@ def head_ptr(row_id, nhead: int, head_dim: int):
     hp = np.zeros(nhead + 1, np.int32)
     check(lib().et_head_ptr(_ptr(row_id), int(row_id.size), nhead, head_dim, _ptr(hp)))
     return hp
+
+
+def prune_tile_mat(W, sparsity: float):
+    """magnitude pruning of dense half W[N x K] -> (row_ptr, row_offset): the tiles with the largest L2 norm"""
+    W = np.ascontiguousarray(W)
+    assert W.dtype == np.float16 and W.ndim == 2
+    N, K = W.shape
+    row_ptr = np.zeros(N // 16 + 1, np.int32)
+    row_offset = np.zeros(max((N // 16) * (K // 16), 1), np.int32)
+    nt = check(lib().et_prune_tile_mat(_ptr(W), N, K, sparsity, _ptr(row_ptr), _ptr(row_offset)))
+    return row_ptr, row_offset[:nt].copy()
+
+
+def prune_row_mat(W, sparsity: float):
+    """magnitude pruning of dense half W[N x K] -> sorted ids of the rows with the largest L2 norm"""
+    W = np.ascontiguousarray(W)
+    assert W.dtype == np.float16 and W.ndim == 2
+    row_id = np.zeros(max(W.shape[0], 1), np.int32)
+    n = check(lib().et_prune_row_mat(_ptr(W), W.shape[0], W.shape[1], sparsity, _ptr(row_id)))
+    return row_id[:n].copy()
+
+
+def tile_mat_save(path, in_feat, out_feat, row_ptr, row_offset, data, bias):
+    row_ptr = np.ascontiguousarray(row_ptr, np.int32)
+    row_offset = np.ascontiguousarray(row_offset, np.int32)
+    data = np.ascontiguousarray(data, np.float16)
+    bias = np.ascontiguousarray(bias, np.float16)
+    check(lib().et_tile_mat_save(str(path).encode(), in_feat, out_feat, int(row_offset.size), _ptr(row_ptr),
+                                 _ptr(row_offset), _ptr(data), _ptr(bias)))
+
+
+def tile_mat_load(path):
+    """-> dict(in_feat, out_feat, row_ptr, row_offset, data, bias)"""
+    import ctypes as C
+    a, b, c = C.c_int(), C.c_int(), C.c_int()
+    check(lib().et_tile_mat_peek(str(path).encode(), C.byref(a), C.byref(b), C.byref(c)))
+    in_feat, out_feat, nt = a.value, b.value, c.value
+    row_ptr = np.zeros(out_feat // 16 + 1, np.int32)
+    row_offset = np.zeros(max(nt, 1), np.int32)
+    data = np.zeros(max(nt, 1) * 256, np.float16)
+    bias = np.zeros(out_feat, np.float16)
+    check(lib().et_tile_mat_load(str(path).encode(), _ptr(row_ptr), _ptr(row_offset), _ptr(data), _ptr(bias)))
+    return dict(in_feat=in_feat, out_feat=out_feat, row_ptr=row_ptr, row_offset=row_offset[:nt].copy(),
+                data=data[:nt * 256].copy(), bias=bias)
+
+
+def row_mat_save(path, in_feat, out_feat, row_id, weight, bias):
+    row_id = np.ascontiguousarray(row_id, np.int32)
+    weight = np.ascontiguousarray(weight, np.float16)
+    bias = np.ascontiguousarray(bias, np.float16)
+    assert weight.size == row_id.size * in_feat
+    check(lib().et_row_mat_save(str(path).encode(), in_feat, out_feat, int(row_id.size), _ptr(row_id),
+                                _ptr(weight), _ptr(bias)))
+
+
+def row_mat_load(path):
+    """-> dict(in_feat, out_feat, row_id, weight[nrow x in_feat], bias)"""
+    import ctypes as C
+    a, b, c = C.c_int(), C.c_int(), C.c_int()
+    check(lib().et_row_mat_peek(str(path).encode(), C.byref(a), C.byref(b), C.byref(c)))
+    in_feat, out_feat, n = a.value, b.value, c.value
+    row_id = np.zeros(max(n, 1), np.int32)
+    weight = np.zeros((max(n, 1), in_feat), np.float16)
+    bias = np.zeros(out_feat, np.float16)
+    check(lib().et_row_mat_load(str(path).encode(), _ptr(row_id), _ptr(weight), _ptr(bias)))
+    return dict(in_feat=in_feat, out_feat=out_feat, row_id=row_id[:n].copy(), weight=weight[:n].copy(), bias=bias)

@@ -24,7 +24,8 @@ extern "C" {
 #define ET_ERR_ALIGNMENT (-2)   /* pointer or leading dimension not 16-byte aligned */
 #define ET_ERR_UNSUPPORTED (-3) /* shape outside what the kernels cover */
 #define ET_ERR_HIP (-4)         /* a HIP runtime call failed; see et_last_error() */
-#define ET_ERR_FORMAT (-5)      /* malformed tile_mat / row_mat index arrays */
+#define ET_ERR_FORMAT (-5)      /* malformed tile_mat / row_mat index arrays or container file */
+#define ET_ERR_IO (-6)          /* a file could not be opened, read or written */
 
 /* Human-readable text for a code; message of the last failure on this thread. */
 const char *et_strerror(int code);
@@ -197,6 +198,36 @@ int et_gen_sparse_row_mat(int nrow, float sparsity, uint64_t seed,
  * nhead*keep.  Balanced variant used for per-head Q/K pruning. */
 int et_gen_head_balanced_rows(int nhead, int head_dim, int keep, uint64_t seed,
                               int *row_id);
+/* Magnitude-based selection in place of the random one: from dense row-major
+ * W[N x K] (halves) keep the int(total*(1.0-sparsity)) 16x16 tiles (resp.
+ * int(N*(1.0-sparsity)) rows) with the largest sum of squares (accumulated in
+ * double, row-major; ties keep the lower index; NaN counts as 0).  Tiles are
+ * listed by ascending column inside a block-row, row_id ascending.  Counts
+ * follow test/tile_mat.cu:10-11 and test/row_mat.cu:7; the reference itself
+ * only selects at random (test/tile_mat.cu:16, test/row_mat.cu:11).  Returns
+ * the number kept; follow with et_tile_pack / a row gather for the values. */
+int et_prune_tile_mat(const void *W, int N, int K, float sparsity, int *row_ptr,
+                      int *row_offset);
+int et_prune_row_mat(const void *W, int N, int K, float sparsity, int *row_id);
+
+/* On-disk container of a pruned linear (the reference keeps none): 64-byte
+ * little-endian header (magic, version 1, in_feat, out_feat, count, payload
+ * bytes, FNV-1a 64 of the payload) followed by
+ *   tile_mat: row_ptr[out_feat/16+1], row_offset[ntile], data[ntile*256], bias[out_feat]
+ *   row_mat : row_id[nrow], weight[nrow x in_feat] (compact rows), bias[out_feat]
+ * _peek reads the sizes so that the caller can allocate; _load verifies size,
+ * checksum and the format's invariants (ET_ERR_FORMAT) and fills the arrays. */
+int et_tile_mat_save(const char *path, int in_feat, int out_feat, int ntile,
+                     const int *row_ptr, const int *row_offset, const void *data,
+                     const void *bias);
+int et_tile_mat_peek(const char *path, int *in_feat, int *out_feat, int *ntile);
+int et_tile_mat_load(const char *path, int *row_ptr, int *row_offset, void *data,
+                     void *bias);
+int et_row_mat_save(const char *path, int in_feat, int out_feat, int nrow,
+                    const int *row_id, const void *weight, const void *bias);
+int et_row_mat_peek(const char *path, int *in_feat, int *out_feat, int *nrow);
+int et_row_mat_load(const char *path, int *row_id, void *weight, void *bias);
+
 /* 0 if (row_ptr,row_offset) is a well-formed tile_mat of W[N x K]
  * (the asserts of test/tile_mat.cu:31-33 plus range/alignment/duplicates). */
 int et_tile_mat_validate(int N, int K, int ntile, const int *row_ptr,

@@ -343,6 +343,69 @@ void orc_gelu(const h16 *in, h16 *out, long n) {
         out[i] = gelu_h(in[i]);
 }
 
+/* ------------------------------------------------------------------ */
+/* Magnitude pruning (the selection rule of the product library's      */
+/* et_prune_tile_mat / et_prune_row_mat, restated with a full sort):    */
+/* keep the int(total*(1.0-sparsity)) units with the largest sum of      */
+/* squares (double, row-major), ties to the lower index.  Counts as     */
+/* test/tile_mat.cu:10-11 and test/row_mat.cu:7.                        */
+/* ------------------------------------------------------------------ */
+typedef struct { double key; int idx; } prune_item;
+static int prune_cmp(const void *a, const void *b) {
+    const prune_item *x = (const prune_item *)a, *y = (const prune_item *)b;
+    if (x->key != y->key) return x->key > y->key ? -1 : 1;
+    return x->idx < y->idx ? -1 : (x->idx > y->idx);
+}
+static int int_cmp(const void *a, const void *b) {
+    const int x = *(const int *)a, y = *(const int *)b;
+    return x < y ? -1 : (x > y);
+}
+static double sq_h(h16 v) {
+    uint16_t u; memcpy(&u, &v, 2);
+    if ((u & 0x7C00) == 0x7C00 && (u & 0x3FF)) return 0.0;          /* NaN counts as 0 */
+    double d = ((u & 0x7FFF) == 0x7C00) ? 4294967296.0 : (double)h2f(v); /* Inf as 2^32 */
+    return d * d;
+}
+int orc_prune_tile_mat(const h16 *W, int N, int K, float sparsity, int *row_ptr, int *row_offset) {
+    const int brows = N / 16, bcols = K / 16, total = brows * bcols;
+    const int ntile = (int)(total * (1.0 - (double)sparsity));
+    prune_item *it = (prune_item *)malloc(sizeof(prune_item) * (size_t)(total > 0 ? total : 1));
+    for (int t = 0; t < total; t++) {
+        const int y = t / bcols, x = t % bcols;
+        double acc = 0.0;
+        for (int n = 0; n < 16; n++)
+            for (int k = 0; k < 16; k++)
+                acc += sq_h(W[(size_t)(y * 16 + n) * K + x * 16 + k]);
+        it[t].key = acc; it[t].idx = t;
+    }
+    qsort(it, (size_t)total, sizeof(prune_item), prune_cmp);
+    int *kept = (int *)malloc(sizeof(int) * (size_t)(ntile > 0 ? ntile : 1));
+    for (int i = 0; i < ntile; i++) kept[i] = it[i].idx;
+    qsort(kept, (size_t)ntile, sizeof(int), int_cmp);
+    for (int y = 0; y <= brows; y++) row_ptr[y] = 0;
+    for (int i = 0; i < ntile; i++) {
+        row_ptr[kept[i] / bcols + 1]++;
+        row_offset[i] = (kept[i] % bcols) * 16;
+    }
+    for (int y = 0; y < brows; y++) row_ptr[y + 1] += row_ptr[y];
+    free(kept); free(it);
+    return ntile;
+}
+int orc_prune_row_mat(const h16 *W, int N, int K, float sparsity, int *row_id) {
+    const int keep = (int)(N * (1.0 - (double)sparsity));
+    prune_item *it = (prune_item *)malloc(sizeof(prune_item) * (size_t)(N > 0 ? N : 1));
+    for (int n = 0; n < N; n++) {
+        double acc = 0.0;
+        for (int k = 0; k < K; k++) acc += sq_h(W[(size_t)n * K + k]);
+        it[n].key = acc; it[n].idx = n;
+    }
+    qsort(it, (size_t)N, sizeof(prune_item), prune_cmp);
+    for (int i = 0; i < keep; i++) row_id[i] = it[i].idx;
+    qsort(row_id, (size_t)keep, sizeof(int), int_cmp);
+    free(it);
+    return keep;
+}
+
 #define REAL float
 #define SUF(name) name##_f32
 #define TOH(x) f2h((float)(x))

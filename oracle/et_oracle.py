@@ -94,6 +94,24 @@ def gen_sparse_tile_mat(nrow, ncol, sparsity, seed):
     return row_ptr, row_offset[:nt].copy()
 
 
+def prune_tile_mat(W, sparsity):
+    """magnitude pruning: the tiles of dense half W[N x K] with the largest L2 norm -> (row_ptr, row_offset)"""
+    W = _h(W)
+    N, K = W.shape
+    row_ptr = np.zeros(N // 16 + 1, np.int32)
+    row_offset = np.zeros(max((N // 16) * (K // 16), 1), np.int32)
+    nt = lib().orc_prune_tile_mat(_p(W), N, K, C.c_float(sparsity), _p(row_ptr), _p(row_offset))
+    return row_ptr, row_offset[:nt].copy()
+
+
+def prune_row_mat(W, sparsity):
+    """magnitude pruning: sorted ids of the rows of dense half W[N x K] with the largest L2 norm"""
+    W = _h(W)
+    row_id = np.zeros(max(W.shape[0], 1), np.int32)
+    n = lib().orc_prune_row_mat(_p(W), W.shape[0], W.shape[1], C.c_float(sparsity), _p(row_id))
+    return row_id[:n].copy()
+
+
 def gen_sparse_row_mat(nrow, sparsity, seed):
     """-> sorted row_id[nn_row] int32; test/row_mat.cu:5-14"""
     row_id = np.zeros(max(nrow, 1), np.int32)

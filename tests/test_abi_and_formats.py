@@ -11,6 +11,7 @@ import pytest
 
 import oracle.et_oracle as orc
 from et_amd import _lib, formats
+from helpers import rng
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -97,3 +98,55 @@ def test_argument_errors_return_codes_without_a_device():
     h = C.c_void_p()
     rc = l.et_tile_plan_create(C.byref(h), 32, 32, int(ro.size), data.ctypes.data, rp.ctypes.data, bad.ctypes.data, bias.ctypes.data)
     assert rc == -5 and not h.value
+
+
+def test_magnitude_pruner_matches_the_oracle_bit_for_bit():
+    from et_amd import formats
+    r = rng(81)
+    for N, K, sp in [(96, 128, 0.5), (768, 768, 0.8), (64, 64, 0.0), (64, 64, 1.0), (3072, 768, 0.9)]:
+        W = (r.standard_normal((N, K)) * 0.05).astype(np.float16)
+        W[::7] *= np.float16(3)
+        rp, ro = formats.prune_tile_mat(W, sp)
+        rp2, ro2 = orc.prune_tile_mat(W, sp)
+        assert np.array_equal(rp, rp2) and np.array_equal(ro, ro2)
+        assert np.array_equal(formats.prune_row_mat(W, sp), orc.prune_row_mat(W, sp))
+    W = np.ones((64, 64), np.float16)
+    W[5, 5] = np.float16(np.nan)
+    W[40, 40] = np.float16(np.inf)
+    for a, b in zip(formats.prune_tile_mat(W, 0.75), orc.prune_tile_mat(W, 0.75)):
+        assert np.array_equal(a, b)
+    assert np.array_equal(formats.prune_row_mat(W, 0.9), orc.prune_row_mat(W, 0.9))
+
+
+def test_pruned_weight_containers_round_trip_and_reject_damage(tmp_path):
+    from et_amd import formats
+    from et_amd._lib import EtError
+    r = rng(82)
+    N, K = 96, 64
+    W = (r.standard_normal((N, K)) * 0.1).astype(np.float16)
+    bias = (r.standard_normal(N) * 0.1).astype(np.float16)
+    rp, ro = formats.prune_tile_mat(W, 0.6)
+    data = formats.tile_pack(W, rp, ro)
+    p = tmp_path / "w.ettile"
+    formats.tile_mat_save(p, K, N, rp, ro, data, bias)
+    back = formats.tile_mat_load(p)
+    assert (back["in_feat"], back["out_feat"]) == (K, N)
+    for k, v in (("row_ptr", rp), ("row_offset", ro), ("data", data), ("bias", bias)):
+        assert np.array_equal(back[k].view(np.uint8), np.ascontiguousarray(v).view(np.uint8)), k
+    ids = formats.prune_row_mat(W, 0.7)
+    q = tmp_path / "w.etrow"
+    formats.row_mat_save(q, K, N, ids, W[ids], bias)
+    back = formats.row_mat_load(q)
+    assert np.array_equal(back["row_id"], ids) and np.array_equal(back["weight"], W[ids]) and np.array_equal(back["bias"], bias)
+    # damage: one flipped payload byte, truncation, trailing bytes, the other kind's file, no file
+    raw = p.read_bytes()
+    for bad in (raw[:100] + bytes([raw[100] ^ 1]) + raw[101:], raw[:-3], raw + b"x", q.read_bytes()):
+        (tmp_path / "bad").write_bytes(bad)
+        with pytest.raises(EtError) as e:
+            formats.tile_mat_load(tmp_path / "bad")
+        assert e.value.code == -5
+    with pytest.raises(EtError) as e:
+        formats.tile_mat_load(tmp_path / "missing")
+    assert e.value.code == -6
+    with pytest.raises(EtError):                                      # unsorted row ids are refused on save
+        formats.row_mat_save(tmp_path / "x", K, N, ids[::-1], W[ids], bias)

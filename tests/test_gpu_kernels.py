@@ -91,6 +91,33 @@ def test_tile_linear_raw_and_planned(K, M, N, Kd, sp, gelu):
     check_close(got2, want64, max_abs=tol, mean_rel=5e-4, what="tile planned vs f64")
 
 
+def test_magnitude_pruned_linear_through_container(K, tmp_path):
+    """dense W -> et_prune_tile_mat -> et_tile_pack -> container file -> Linear_tile == oracle on the same tile_mat,
+    and == the dense product with the dropped tiles zeroed"""
+    from et_amd import formats
+    from et_amd.encoder import Linear_tile
+    r = rng(77)
+    M, N, Kd = 200, 768, 768
+    W = (r.standard_normal((N, Kd)) * 0.05 * (1 + (np.arange(N)[:, None] // 16 + np.arange(Kd)[None, :] // 16) % 5)).astype(np.float16)
+    bias = randn_h(r, (N,), 0.2)
+    rp, ro = formats.prune_tile_mat(W, 0.8)
+    assert ro.size == 460
+    formats.tile_mat_save(tmp_path / "o.ettile", Kd, N, rp, ro, formats.tile_pack(W, rp, ro), bias)
+    t = formats.tile_mat_load(tmp_path / "o.ettile")
+    X = randn_h(r, (M, Kd))
+    lt = Linear_tile(Kd, N, M, t["row_offset"].size, t["data"], t["row_ptr"], t["row_offset"], t["bias"], False)
+    got = host(lt.run(dev(X)))
+    want = orc.tile_linear(X, t["row_ptr"], t["row_offset"], t["data"], t["bias"], N, f64=True)
+    tol = max(np.abs(want.astype(np.float64)).max() * 2.0 ** -10, 1e-3)
+    check_close(got, want, max_abs=tol, mean_rel=5e-4, what="magnitude-pruned linear")
+    Wz = np.zeros_like(W)
+    for bn in range(N // 16):
+        for o in t["row_offset"][t["row_ptr"][bn]:t["row_ptr"][bn + 1]]:
+            Wz[bn * 16:(bn + 1) * 16, o:o + 16] = W[bn * 16:(bn + 1) * 16, o:o + 16]
+    dense = X.astype(np.float64) @ Wz.astype(np.float64).T + bias.astype(np.float64)
+    check_close(got, dense.astype(np.float16), max_abs=tol, mean_rel=5e-4, what="vs dense with zeroed tiles")
+
+
 LN_CASES = [
     # M, N, K, sparsity
     (128, 768, 768, 0.8),     # O projection + LayerNorm (resident panel, 3 block-rows per wave)

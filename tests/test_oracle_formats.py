@@ -175,3 +175,43 @@ def test_head_ptr_csr():
     bal = orc.gen_head_balanced_rows(12, 64, 32, seed=4)
     assert orc.head_ptr(bal, 12, 64).tolist() == [32 * h for h in range(13)]
     assert (np.diff(bal) > 0).all()
+
+
+# ------------------------------------------------------------------ magnitude pruning
+def test_prune_tile_mat_keeps_the_largest_tiles():
+    """norms made distinct and well separated, so any correct ranking gives the same set"""
+    r = rng(71)
+    N, K = 96, 128
+    nb = (N // 16) * (K // 16)
+    scale = r.permutation(nb).astype(np.float64) + 1.0           # tile t gets magnitude ~ scale[t]
+    W = np.zeros((N, K), np.float16)
+    for t in range(nb):
+        y, x = divmod(t, K // 16)
+        W[y * 16:(y + 1) * 16, x * 16:(x + 1) * 16] = (scale[t] * (0.9 + 0.01 * r.random((16, 16)))).astype(np.float16)
+    for sp in (0.0, 0.25, 0.5, 0.8, 0.97, 1.0):
+        rp, ro = orc.prune_tile_mat(W, sp)
+        keep = int(nb * (1.0 - float(np.float32(sp))))
+        assert ro.size == keep and rp[-1] == keep and rp[0] == 0
+        assert orc.tile_mat_validate(N, K, rp, ro) == 0
+        want = np.sort(np.argsort(-scale, kind="stable")[:keep])      # the `keep` largest tiles, row-major
+        got = np.concatenate([[bn * (K // 16) + o // 16 for o in ro[rp[bn]:rp[bn + 1]]] for bn in range(N // 16)]).astype(int) if keep else np.array([], int)
+        assert np.array_equal(got, want)
+        for bn in range(N // 16):                                    # ascending columns inside a block-row
+            assert (np.diff(ro[rp[bn]:rp[bn + 1]]) > 0).all()
+
+
+def test_prune_ties_keep_the_lower_index_and_rows():
+    W = np.ones((64, 64), np.float16)                               # every tile / row has the same norm
+    rp, ro = orc.prune_tile_mat(W, 0.5)
+    assert np.array_equal(rp, [0, 4, 8, 8, 8]) and np.array_equal(ro, list(range(0, 64, 16)) * 2)
+    assert np.array_equal(orc.prune_row_mat(W, 0.75), np.arange(16))
+    r = rng(72)
+    W = (r.standard_normal((200, 48)) * (1 + np.arange(200)[:, None] % 7)).astype(np.float16)
+    ids = orc.prune_row_mat(W, 0.7)
+    n2 = (W.astype(np.float64) ** 2).sum(1)
+    assert ids.size == int(200 * (1.0 - float(np.float32(0.7)))) and (np.diff(ids) > 0).all()
+    assert n2[ids].min() >= np.delete(n2, ids).max()                # nothing dropped outranks anything kept
+    W[3, 5] = np.float16(np.nan)                                     # NaN contributes nothing; Inf dominates
+    W[7, 0] = np.float16(np.inf)
+    ids = orc.prune_row_mat(W, 0.99)                                  # int(200*(1-float(0.99f))) = 1 row
+    assert ids.tolist() == [7]
