@@ -21,6 +21,7 @@ PROTOTYPES = {
     "et_skip_layernorm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "et_tile_spmm_add_bias": (_i, [_vp, _vp, _ip, _ip, _vp, _i, _i, _i, _vp, _vp]),
     "et_tile_spmm_add_bias_gelu": (_i, [_vp, _vp, _ip, _ip, _vp, _i, _i, _i, _vp, _vp]),
+    "et_row_spmm_add_bias_gelu": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "et_row_spmm_add_bias": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "et_OTF_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _ip, _f, _vp]),
     "et_attention_mask_summary_bytes": (C.c_size_t, [_i]),
@@ -62,11 +63,14 @@ PROTOTYPES = {
     "et_linear_tile_run_rows_ln": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
     "et_linear_tile_run_multi": (_i, [C.POINTER(_vp), C.POINTER(_vp), _i, _vp, _i, _vp]),
     "et_linear_row_create": (_i, [C.POINTER(_vp), _i, _i, _i, _vp, _ip, _i, _vp, _i]),
+    "et_linear_row_set_gelu": (_i, [_vp, _i]),
     "et_linear_row_destroy": (None, [_vp]),
     "et_linear_row_run": (_i, [_vp, _vp, _vp, _vp]),
     "et_linear_row_query": (_i, [_vp, C.POINTER(_i), C.POINTER(_i), C.POINTER(_vp), C.POINTER(_vp)]),
     "et_encoder_create": (_i, [C.POINTER(_vp), _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                 _vp, _vp, _vp, _vp, _vp]),
+    "et_encoder_attnaware_create": (_i, [C.POINTER(_vp), _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                          _vp, _vp, _vp, _vp, _vp]),
     "et_encoder_destroy": (None, [_vp]),
     "et_encoder_buffer_size": (_sz, [_i, _i, _i, _i, _i]),
     "et_encoder_run": (_i, [_vp, _vp, _vp]),

@@ -128,6 +128,14 @@ int et_linear_row_create(et_linear_row **h, int in_feat, int out_feat, int size,
                                           H(bias), nhead)};
     });
 }
+int et_linear_row_set_gelu(et_linear_row *h, int on) {
+    if (!h) {
+        et::set_error("et_linear_row_set_gelu: null handle");
+        return ET_ERR_INVALID_ARG;
+    }
+    h->impl.is_gelu = on != 0;
+    return ET_OK;
+}
 void et_linear_row_destroy(et_linear_row *h) { delete h; }
 int et_linear_row_run(const et_linear_row *h, void *out, const void *in, void *stream) {
     if (!h) {
@@ -198,6 +206,37 @@ int et_encoder_create(et_encoder **h, int kind, int d_model, int seq_len, int nh
             delete static_cast<et_linear_row *>(v);
         else
             delete static_cast<et_linear_tile *>(v);
+        delete o;
+        delete mlp1;
+        delete mlp2;
+    }
+    return rc;
+}
+int et_encoder_attnaware_create(et_encoder **h, int d_model, int seq_len, int nheads, int batch,
+                                void *buffer, et_linear_row *q, et_linear_row *k, et_linear_tile *v,
+                                et_linear_row *o, et_linear_row *mlp1, et_linear_row *mlp2, const void *g1,
+                                const void *b1, const void *g2, const void *b2, const void *mask) {
+    if (!h || !buffer || !q || !k || !v || !o || !mlp1 || !mlp2 || !g1 || !b1 || !g2 || !b2) {
+        et::set_error("et_encoder_attnaware_create: null pointer");
+        return ET_ERR_INVALID_ARG;
+    }
+    if (d_model <= 0 || seq_len <= 0 || nheads <= 0 || batch <= 0 || d_model % nheads) {
+        et::set_error("et_encoder_attnaware_create: d_model=%d seq_len=%d nheads=%d batch=%d", d_model,
+                      seq_len, nheads, batch);
+        return ET_ERR_INVALID_ARG;
+    }
+    *h = nullptr;
+    const int rc = guarded([&] {
+        std::unique_ptr<Encoder_base> e(new Encoder_attnaware(
+            d_model, seq_len, nheads, static_cast<half *>(buffer), std::move(q->impl), std::move(k->impl),
+            std::move(v->impl), std::move(o->impl), std::move(mlp1->impl), std::move(mlp2->impl), H(g1), H(b1),
+            H(g2), H(b2), H(mask), batch));
+        *h = new et_encoder{ET_ENCODER_ATTNAWARE, std::move(e)};
+    });
+    if (rc == ET_OK) { // the linears were moved in: release the emptied shells
+        delete q;
+        delete k;
+        delete v;
         delete o;
         delete mlp1;
         delete mlp2;

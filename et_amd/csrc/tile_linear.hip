@@ -1438,9 +1438,9 @@ extern "C" int et_tile_spmm_add_bias_gelu(void *Y, const void *X, const int *W_r
                                stream, "et_tile_spmm_add_bias_gelu");
 }
 
-extern "C" int et_row_spmm_add_bias(void *out, const void *in, const void *weight,
-                                    const void *bias, int M, int N, int K, void *stream) {
-    using namespace et;
+namespace et {
+static int row_linear(void *out, const void *in, const void *weight, const void *bias, int M, int N,
+                      int K, bool gelu, void *stream) {
     ET_REQUIRE(out && in && weight && bias, ET_ERR_INVALID_ARG, "et_row_spmm_add_bias: null pointer");
     ET_REQUIRE(M >= 0 && N > 0 && K > 0, ET_ERR_INVALID_ARG,
                "et_row_spmm_add_bias: M=%d N=%d K=%d", M, N, K);
@@ -1460,8 +1460,19 @@ extern "C" int et_row_spmm_add_bias(void *out, const void *in, const void *weigh
     p.nbr = N / 16;
     int KC, nchunk;
     chunking(K, &KC, &nchunk);
-    return tile_launch(&p, 1, static_cast<const f16 *>(in), M, K, KC, nchunk, false, TL_DENSE,
+    return tile_launch(&p, 1, static_cast<const f16 *>(in), M, K, KC, nchunk, gelu, TL_DENSE,
                        static_cast<hipStream_t>(stream));
+}
+} // namespace et
+
+extern "C" int et_row_spmm_add_bias(void *out, const void *in, const void *weight,
+                                    const void *bias, int M, int N, int K, void *stream) {
+    return et::row_linear(out, in, weight, bias, M, N, K, false, stream);
+}
+
+extern "C" int et_row_spmm_add_bias_gelu(void *out, const void *in, const void *weight,
+                                         const void *bias, int M, int N, int K, void *stream) {
+    return et::row_linear(out, in, weight, bias, M, N, K, true, stream);
 }
 
 // ---------------------------------------------------------------------------

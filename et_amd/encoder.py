@@ -84,7 +84,7 @@ def run_multi(linears, x, outs=None):
 class Linear_row:
     """encoder/Linear.h:48-72"""
 
-    def __init__(self, in_feat, out_feat, size, weight, row_id, nrow, bias, nhead):
+    def __init__(self, in_feat, out_feat, size, weight, row_id, nrow, bias, nhead, is_gelu=False):
         weight, row_id, bias = _np(weight, np.float16), _np(row_id, np.int32), _np(bias, np.float16)
         assert weight.size == nrow * in_feat and row_id.size == nrow and bias.size == nrow
         self.in_feat, self.out_feat, self.size, self.nhead = in_feat, out_feat, size, nhead
@@ -92,6 +92,8 @@ class Linear_row:
         check(lib().et_linear_row_create(C.byref(h), in_feat, out_feat, size, _hp(weight), _hp(row_id), nrow,
                                          _hp(bias), nhead))
         self._h = h
+        if is_gelu:
+            check(lib().et_linear_row_set_gelu(h, 1))
         a, b = C.c_int(), C.c_int()
         check(lib().et_linear_row_query(h, C.byref(a), C.byref(b), None, None))
         self.nrow, self.row_id_size = a.value, b.value
@@ -126,11 +128,14 @@ class _Encoder:
         assert mask is None or mask.size == seq_len * seq_len
         lin = [Q_linear, K_linear, V_linear, O_linear, MLP1_linear, MLP2_linear]
         h = C.c_void_p()
-        check(lib().et_encoder_create(C.byref(h), self.kind, d_model, seq_len, nheads, batch, buffer.data_ptr(),
-                                      *[l._h for l in lin], *[_hp(t) for t in ln], _hp(mask)))
+        self._create(h, d_model, seq_len, nheads, batch, buffer, lin, ln, mask)
         for l in lin:
             l._release()
         self._h = h
+
+    def _create(self, h, d_model, seq_len, nheads, batch, buffer, lin, ln, mask):
+        check(lib().et_encoder_create(C.byref(h), self.kind, d_model, seq_len, nheads, batch, buffer.data_ptr(),
+                                      *[l._h for l in lin], *[_hp(t) for t in ln], _hp(mask)))
 
     @classmethod
     def buffer_size(cls, d_model, seq_len, nheads, batch=1):
@@ -167,6 +172,16 @@ class Encoder_tile(_Encoder):
 class Encoder_prune(_Encoder):
     """encoder/encoder.h:79-100; V_linear is a Linear_row"""
     kind = ENCODER_PRUNE
+
+
+class Encoder_attnaware(_Encoder):
+    """Attention-aware pruning through the whole layer: Q/K row-pruned to the same columns per head, V a tile
+    linear, O/FFN1(GELU)/FFN2 row-pruned (no counterpart in the reference)"""
+    kind = ENCODER_TILE  # same workspace as the tile encoder
+
+    def _create(self, h, d_model, seq_len, nheads, batch, buffer, lin, ln, mask):
+        check(lib().et_encoder_attnaware_create(C.byref(h), d_model, seq_len, nheads, batch, buffer.data_ptr(),
+                                                *[l._h for l in lin], *[_hp(t) for t in ln], _hp(mask)))
 
 
 class Encoder_length(_Encoder):

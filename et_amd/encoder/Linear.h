@@ -79,16 +79,17 @@ class Linear_row {
     int nrow;        // row_id_size rounded up to a multiple of 16
     int row_id_size; // surviving rows
     Weight<half> bias;
+    bool is_gelu;    // added: GELU on the compact output (a row-pruned FFN1)
 
     static int multiple_16(int x) { return ((x + 15) / 16) * 16; }
 
     // weight_: HOST [row_id_size_ x in_feat_]; row_id_: HOST, ascending; bias_: HOST [row_id_size_]
     Linear_row(int in_feat_, int out_feat_, int size_, half *weight_, int *row_id_, int row_id_size_,
-               half *bias_, int nhead_)
+               half *bias_, int nhead_, bool is_gelu_ = false)
         : in_feat(in_feat_), out_feat(out_feat_), size(size_), nhead(nhead_),
           weight(in_feat_ * multiple_16(row_id_size_)), row_id(row_id_, row_id_size_ > 0 ? row_id_size_ : 1),
           head_ptr(nhead_ + 1), nrow(multiple_16(row_id_size_)), row_id_size(row_id_size_),
-          bias(multiple_16(row_id_size_)) {
+          bias(multiple_16(row_id_size_)), is_gelu(is_gelu_) {
         // padded rows must contribute nothing: zero the buffers first
         etChk(et_fill_zero(weight.get(), sizeof(half) * (size_t)in_feat * nrow, nullptr));
         etChk(et_fill_zero(bias.get(), sizeof(half) * (size_t)nrow, nullptr));
@@ -103,10 +104,15 @@ class Linear_row {
     Linear_row(const Linear_row &) = delete;
 
     // encoder/Linear.h:68-71; the cuBLAS handle becomes a stream
-    void run(half *out, half *in, void *stream) const {
-        etChk(et_row_spmm_add_bias(out, in, weight.get(), bias.get(), size, nrow, in_feat, stream));
-    }
+    void run(half *out, half *in, void *stream) const { run_rows(out, in, size, stream); }
     void run_rows(half *out, half *in, int rows, void *stream) const {
-        etChk(et_row_spmm_add_bias(out, in, weight.get(), bias.get(), rows, nrow, in_feat, stream));
+        if (is_gelu)
+            etChk(et_row_spmm_add_bias_gelu(out, in, weight.get(), bias.get(), rows, nrow, in_feat, stream));
+        else
+            etChk(et_row_spmm_add_bias(out, in, weight.get(), bias.get(), rows, nrow, in_feat, stream));
+    }
+    // out[rows x out_feat] = the compact result expanded to model width, pruned columns zero
+    void scatter(half *out, const half *compact, int rows, void *stream) const {
+        etChk(et_scatter_cols(out, compact, row_id.get(), rows, row_id_size, nrow, out_feat, stream));
     }
 };

@@ -172,6 +172,56 @@ class Encoder_prune : public Encoder_base {
     }
 };
 
+// Attention-aware pruning carried through the whole layer (no counterpart in
+// the reference, which row-prunes only V, encoder/encoder.h:84): Q and K are
+// row-pruned to the SAME column set per head, so the scores contract over the
+// kept columns only; O, FFN1 and FFN2 are row-pruned too.  A row linear emits
+// a compact [rows x nrow] result (kernels/linear.cu:30-32): O's and FFN2's
+// are expanded back to model width (pruned columns zero) before the skip
+// connection, FFN1's compact hidden feeds an FFN2 whose input columns were
+// gathered to match (MLP2.in_feat == MLP1.nrow).
+class Encoder_attnaware : public Encoder_base {
+  private:
+    Linear_row Q_linear, K_linear;
+    Linear_tile V_linear;
+    Linear_row O_linear, MLP1_linear, MLP2_linear;
+
+  public:
+    Encoder_attnaware(int d_model_, int seq_len_, int nheads_, half *buffer_, Linear_row &&Q_linear_,
+                      Linear_row &&K_linear_, Linear_tile &&V_linear_, Linear_row &&O_linear_,
+                      Linear_row &&MLP1_linear_, Linear_row &&MLP2_linear_, half *ln_gamma_1,
+                      half *ln_beta_1, half *ln_gamma_2, half *ln_beta_2, half *mask_, int batch_ = 1)
+        : Encoder_base(d_model_, seq_len_, nheads_, buffer_, ln_gamma_1, ln_beta_1, ln_gamma_2,
+                       ln_beta_2, mask_, batch_),
+          Q_linear(std::move(Q_linear_)), K_linear(std::move(K_linear_)),
+          V_linear(std::move(V_linear_)), O_linear(std::move(O_linear_)),
+          MLP1_linear(std::move(MLP1_linear_)), MLP2_linear(std::move(MLP2_linear_)) {
+        etRequire(Q_linear.row_id_size == K_linear.row_id_size && Q_linear.nrow <= d_model,
+                  "Encoder_attnaware: Q and K must keep the same columns");
+        etRequire(MLP1_linear.is_gelu, "Encoder_attnaware: MLP1_linear must be the GELU variant");
+        etRequire(MLP2_linear.in_feat == MLP1_linear.nrow,
+                  "Encoder_attnaware: MLP2 must take MLP1's compact hidden as input");
+        etRequire(MLP1_linear.nrow <= 3 * d_model && O_linear.out_feat == d_model && MLP2_linear.out_feat == d_model,
+                  "Encoder_attnaware: widths do not fit the workspace");
+    }
+    void run(half *out, half *in) override {
+        const int n = rows();
+        Q_linear.run_rows(buffers[0], in, n, stream); // compact [n x nrow]
+        K_linear.run_rows(buffers[1], in, n, stream);
+        V_linear.run_rows(buffers[2], in, n, stream);
+        etChk(et_Prune_attention(buffers[3], buffers[0], buffers[1], buffers[2], Q_linear.head_ptr.get(),
+                                 Q_linear.nrow, nullptr, nullptr, d_model, mask_ptr(), seq_len, d_model,
+                                 nheads, batch, lens_ptr(), log2_scale, stream));
+        O_linear.run_rows(buffers[0], buffers[3], n, stream);
+        O_linear.scatter(buffers[1], buffers[0], n, stream);
+        etChk(et_skip_layernorm(buffers[1], in, ln_gamma[0].get(), ln_beta[0].get(), n, d_model, stream));
+        MLP1_linear.run_rows(buffers[2], buffers[1], n, stream); // compact hidden, spans units 2..4
+        MLP2_linear.run_rows(buffers[0], buffers[2], n, stream);
+        MLP2_linear.scatter(out, buffers[0], n, stream);
+        etChk(et_skip_layernorm(out, buffers[1], ln_gamma[1].get(), ln_beta[1].get(), n, d_model, stream));
+    }
+};
+
 // Sequence-aware encoder (encoder/encoder.h:102-134, encoder/encoder.cu:116-149).
 // The reference's version writes scaled Q K^T for all heads to memory and runs
 // a second attention kernel on it; that path is kept behind use_shared_qk.

@@ -70,6 +70,11 @@ int et_tile_spmm_add_bias_gelu(void *Y, const void *X, const int *W_row_ptr,
  * multiple of 16).  The cuBLAS handle/algo pair becomes a stream. */
 int et_row_spmm_add_bias(void *out, const void *in, const void *weight,
                          const void *bias, int M, int N, int K, void *stream);
+/* the same followed by the tanh-form GELU of kernels/linear.cu:36-48 (the
+ * reference's row linear has no GELU form; a row-pruned FFN1 needs it) */
+int et_row_spmm_add_bias_gelu(void *out, const void *in, const void *weight,
+                              const void *bias, int M, int N, int K,
+                              void *stream);
 
 /* Replaces OTF_attention_kernelLauncher (kernels/kernels.h:22-24,
  * kernels/attention.cu:122-134).  out, Q, K, V are [batch*seq_len x d_model];

@@ -45,6 +45,8 @@ int et_linear_tile_run_multi(const et_linear_tile *const *hs, void *const *outs,
  * ascending. */
 int et_linear_row_create(et_linear_row **h, int in_feat, int out_feat, int size, const void *weight,
                          const int *row_id, int row_id_size, const void *bias, int nhead);
+/* added: apply the tanh-form GELU to the compact output (a row-pruned FFN1) */
+int et_linear_row_set_gelu(et_linear_row *h, int on);
 void et_linear_row_destroy(et_linear_row *h);
 /* Linear_row::run(out, in, handle) — encoder/Linear.h:68-71; out is compact
  * [size x nrow]. */
@@ -55,7 +57,7 @@ int et_linear_row_run(const et_linear_row *h, void *out, const void *in, void *s
 int et_linear_row_query(const et_linear_row *h, int *nrow, int *row_id_size, const int **row_id_dev,
                         const int **head_ptr_dev);
 
-enum { ET_ENCODER_TILE = 0, ET_ENCODER_PRUNE = 1, ET_ENCODER_LENGTH = 2 };
+enum { ET_ENCODER_TILE = 0, ET_ENCODER_PRUNE = 1, ET_ENCODER_LENGTH = 2, ET_ENCODER_ATTNAWARE = 3 };
 
 /* Encoder_tile / Encoder_prune / Encoder_length constructors
  * (encoder/encoder.h:70-75, 93-98, 122-127) with the added trailing `batch`.
@@ -69,6 +71,16 @@ int et_encoder_create(et_encoder **h, int kind, int d_model, int seq_len, int nh
                       et_linear_tile *mlp1, et_linear_tile *mlp2, const void *ln_gamma_1,
                       const void *ln_beta_1, const void *ln_gamma_2, const void *ln_beta_2,
                       const void *mask);
+/* Encoder_attnaware: attention-aware pruning through the whole layer (no
+ * counterpart in the reference, which row-prunes only V).  q and k keep the
+ * same columns per head; o, mlp1 (GELU set) and mlp2 are row-pruned, with
+ * mlp2's in_feat equal to mlp1's padded row count.  Ownership as for
+ * et_encoder_create; kind of the result is ET_ENCODER_ATTNAWARE. */
+int et_encoder_attnaware_create(et_encoder **h, int d_model, int seq_len, int nheads, int batch,
+                                void *buffer, et_linear_row *q, et_linear_row *k, et_linear_tile *v,
+                                et_linear_row *o, et_linear_row *mlp1, et_linear_row *mlp2,
+                                const void *ln_gamma_1, const void *ln_beta_1, const void *ln_gamma_2,
+                                const void *ln_beta_2, const void *mask);
 void et_encoder_destroy(et_encoder *h);
 /* Encoder_base::buffer_size / Encoder_length::buffer_size
  * (encoder/encoder.h:51-53,129-133), times batch. */

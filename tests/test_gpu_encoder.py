@@ -87,6 +87,75 @@ def test_encoder_prune_layer():
     check_close(got, want, what="Encoder_prune")
 
 
+def test_encoder_attnaware_layer_config4_wiring():
+    """BASELINE config 4: Q/K keep 32 of 64 columns per head (same set), O/FFN1/FFN2 row-pruned at 70 %.
+    Oracle = its own ops chained step by step; invariant = the same layer with DENSE linears whose pruned
+    rows are zero (and, for FFN2, the dropped hidden units' columns)."""
+    from et_amd.encoder import Encoder_attnaware, Linear_row, Linear_tile
+    r = rng(650)
+    d, H, dff, S, B = 768, 12, 3072, 64, 2
+    hd, T = d // H, B * S
+    x = randn_h(r, (T, d))
+    mask = randn_h(r, (S, S), 0.5)
+    ln = [randn_h(r, (d,), 0.2) + np.float16(1), randn_h(r, (d,), 0.2), randn_h(r, (d,), 0.2) + np.float16(1), randn_h(r, (d,), 0.2)]
+    W = {k: randn_h(r, shp, 0.03) for k, shp in dict(q=(d, d), k=(d, d), v=(d, d), o=(d, d), m1=(dff, d), m2=(d, dff)).items()}
+    bsz = {k: randn_h(r, (W[k].shape[0],), 0.05) for k in W}
+    qk_id = orc.gen_head_balanced_rows(H, hd, 32, seed=11)       # 384 kept Q/K columns, 32 per head
+    o_id = orc.gen_sparse_row_mat(d, 0.7, seed=12)               # 230 rows
+    m1_id = orc.gen_sparse_row_mat(dff, 0.7, seed=13)            # 921 rows
+    m2_id = orc.gen_sparse_row_mat(d, 0.7, seed=14)              # 230 rows
+    pad16 = lambda n: (n + 15) // 16 * 16
+    # FFN2 sees the compact hidden: gather its input columns to the kept hidden units, pad to FFN1's padded width
+    W2c = np.zeros((m2_id.size, pad16(m1_id.size)), np.float16)
+    W2c[:, :m1_id.size] = W["m2"][m2_id][:, m1_id]
+
+    # ---- oracle, step by step
+    qc, kc = orc.row_linear(x, W["q"][qk_id], bsz["q"][qk_id]), orc.row_linear(x, W["k"][qk_id], bsz["k"][qk_id])
+    vfull = (x.astype(np.float32) @ W["v"].astype(np.float32).T + bsz["v"].astype(np.float32)).astype(np.float16)
+    z = orc.prune_attention(qc, kc, vfull, orc.head_ptr(qk_id, H, hd), None, None, mask, S, d, H, B)
+    def scatter(c, ids):
+        out = np.zeros((T, d), np.float16)
+        out[:, ids] = c[:, :ids.size]
+        return out
+    h1 = orc.skip_layernorm(scatter(orc.row_linear(z, W["o"][o_id], bsz["o"][o_id]), o_id), x, ln[0], ln[1])
+    hid = orc.gelu(orc.row_linear(h1, W["m1"][m1_id], bsz["m1"][m1_id]))
+    hid_p = np.zeros((T, pad16(m1_id.size)), np.float16)
+    hid_p[:, :m1_id.size] = hid
+    want = orc.skip_layernorm(scatter(orc.row_linear(hid_p, W2c, bsz["m2"][m2_id]), m2_id), h1, ln[2], ln[3])
+
+    # ---- invariant: dense linears with the pruned rows zeroed give the same layer (fp64)
+    def zero_rows(w, b, ids):
+        wz, bz = np.zeros_like(w, np.float64), np.zeros_like(b, np.float64)
+        wz[ids], bz[ids] = w[ids], b[ids]
+        return wz, bz
+    x64 = x.astype(np.float64)
+    lin = lambda inp, wb: (inp @ wb[0].T + wb[1]).astype(np.float16)
+    qd, kd = lin(x64, zero_rows(W["q"], bsz["q"], qk_id)), lin(x64, zero_rows(W["k"], bsz["k"], qk_id))
+    zd = orc.otf_attention(qd, kd, vfull, mask, S, H, B, None, 1.0, f64=True)
+    h1d = orc.skip_layernorm(lin(zd.astype(np.float64), zero_rows(W["o"], bsz["o"], o_id)), x, ln[0], ln[1], f64=True)
+    hidd = orc.gelu(lin(h1d.astype(np.float64), zero_rows(W["m1"], bsz["m1"], m1_id)))
+    hidd[:, np.setdiff1d(np.arange(dff), m1_id)] = 0               # gelu(0) = 0 anyway
+    outd = orc.skip_layernorm(lin(hidd.astype(np.float64), zero_rows(W["m2"], bsz["m2"], m2_id)), h1d, ln[2], ln[3], f64=True)
+    check_close(want, outd, what="config-4 oracle vs dense-with-zeroed-rows")
+
+    # ---- the class
+    vt = dict(N=d, K=d)
+    vt["row_ptr"], vt["row_offset"] = orc.gen_sparse_tile_mat(d, d, 0.0, seed=1)
+    vt["data"] = orc.tile_pack(W["v"], vt["row_ptr"], vt["row_offset"])
+    Lq = Linear_row(d, d, T, W["q"][qk_id], qk_id, qk_id.size, bsz["q"][qk_id], H)
+    Lk = Linear_row(d, d, T, W["k"][qk_id], qk_id, qk_id.size, bsz["k"][qk_id], H)
+    Lv = Linear_tile(d, d, T, vt["row_offset"].size, vt["data"], vt["row_ptr"], vt["row_offset"], bsz["v"], False)
+    Lo = Linear_row(d, d, T, W["o"][o_id], o_id, o_id.size, bsz["o"][o_id], H)
+    L1 = Linear_row(d, dff, T, W["m1"][m1_id], m1_id, m1_id.size, bsz["m1"][m1_id], H, is_gelu=True)
+    L2 = Linear_row(pad16(m1_id.size), d, T, W2c, m2_id, m2_id.size, bsz["m2"][m2_id], H)
+    assert (Lq.nrow, Lo.nrow, L1.nrow, L2.nrow) == (384, 240, 928, 240)
+    enc = Encoder_attnaware(d, S, H, workspace(Encoder_attnaware, d, S, H, B), Lq, Lk, Lv, Lo, L1, L2, *ln, mask, B)
+    xd = dev(x)
+    got = host(enc.run(torch.empty_like(xd), xd))
+    check_close(got, want, what="Encoder_attnaware")
+    check_close(got, outd, what="Encoder_attnaware vs dense-with-zeroed-rows")
+
+
 def test_encoder_length_paths():
     from et_amd.encoder import Encoder_length
     r = rng(700)
