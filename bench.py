@@ -270,6 +270,56 @@ def run_extras(torch, orc, K, dev):
     o = torch.empty_like(x)
     us = timeit(lambda: enc.run(o, x))
     out["config1_dense_layer_b1_s128"] = {"us": round(us, 2), "seqs_per_s": round(1e6 / us, 1)}
+
+    # config 4: attention-aware pruned layer, batch 32 x seq 256 (Q/K keep 32 of 64 columns per head,
+    # O/FFN1/FFN2 row-pruned at 70 %)
+    from et_amd.encoder import Encoder_attnaware, Linear_row
+    r = rng(9)
+    S, B = 256, 32
+    T = S * B
+    pad16 = lambda n: (n + 15) // 16 * 16
+    qk_id = orc.gen_head_balanced_rows(H, D // H, 32, seed=11)
+    o_id, m1_id, m2_id = (orc.gen_sparse_row_mat(n, 0.7, seed=s) for n, s in ((D, 12), (DFF, 13), (D, 14)))
+    rw = lambda n, k: randn_h(r, (n, k), 0.02)
+    zb = lambda n: np.zeros(n, np.float16)
+    vt = make_tile_linear(r, D, D, 0.0, seed=15, std=0.02)
+    Lq, Lk = (Linear_row(D, D, T, rw(qk_id.size, D), qk_id, qk_id.size, zb(qk_id.size), H) for _ in range(2))
+    Lv = Linear_tile(D, D, T, vt["row_offset"].size, vt["data"], vt["row_ptr"], vt["row_offset"], vt["bias"])
+    Lo = Linear_row(D, D, T, rw(o_id.size, D), o_id, o_id.size, zb(o_id.size), H)
+    L1 = Linear_row(D, DFF, T, rw(m1_id.size, D), m1_id, m1_id.size, zb(m1_id.size), H, is_gelu=True)
+    L2 = Linear_row(pad16(m1_id.size), D, T, rw(m2_id.size, pad16(m1_id.size)), m2_id, m2_id.size, zb(m2_id.size), H)
+    ws = torch.empty(Encoder_attnaware.buffer_size(D, S, H, B) // 2, dtype=torch.float16, device=dev)
+    ln1 = [np.ones(D, np.float16), np.zeros(D, np.float16)] * 2
+    enc4 = Encoder_attnaware(D, S, H, ws, Lq, Lk, Lv, Lo, L1, L2, *ln1, np.zeros((S, S), np.float16), B)
+    x = torch.from_numpy(randn_h(r, (T, D))).to(dev)
+    o = torch.empty_like(x)
+    us = timeit(lambda: enc4.run(o, x), reps=50)
+    out["config4_attention_aware_pruned_layer_b32_s256"] = {"us": round(us, 2), "seqs_per_s": round(B * 1e6 / us, 1)}
+    del enc4, ws
+
+    # config 5: 12-layer stack, batch 64, lengths ~ U{32..512} padded to 512: packed (length-aware) vs padded
+    from et_amd.encoder import Encoder_length, Encoder_stack
+    r = rng(10)
+    S, B, NL = 512, 64, 12
+    lens = r.integers(32, 513, size=B).astype(np.int32)
+    layers = []
+    for li in range(NL):
+        lins, ln = build_layer(orc, r, 0.8, seed=200 + 10 * li)
+        ws = torch.empty(Encoder_length.buffer_size(D, S, H, B) // 2, dtype=torch.float16, device=dev)
+        L = [Linear_tile(l["K"], l["N"], S * B, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], j == 4)
+             for j, l in enumerate(lins)]
+        layers.append((Encoder_length(D, S, H, ws, *L, *ln, np.zeros((S, S), np.float16), B), ws))
+    x = torch.from_numpy(randn_h(r, (S * B, D))).to(dev)
+    o = torch.empty_like(x)
+    stack = Encoder_stack([l for l, _ in layers], D, S, B)
+    res5 = {"lengths_sum": int(lens.sum()), "padded_rows": S * B}
+    for name, ll in (("padded", None), ("length_aware", lens)):
+        for l, _ in layers:
+            l.set_seq_lens(ll)
+        us = timeit(lambda: stack.run(o, x), reps=10, warm=3)
+        res5[name] = {"us_12_layers": round(us, 1), "seqs_per_s": round(B * 1e6 / us, 1)}
+    res5["padding_skip_speedup"] = round(res5["padded"]["us_12_layers"] / res5["length_aware"]["us_12_layers"], 3)
+    out["config5_length_aware_12_layer_stack_b64"] = res5
     return out
 
 

@@ -1270,6 +1270,7 @@ static int g_tile_nb = 0;
 static int g_tile_min_wgs = 512;
 static int g_tile_ipw = 0;
 static int g_tile_fuse_ln = 1;
+static int g_tile_ln_min_panels = 96;
 
 // Block-rows per wave.  Measured on the BERT-base shapes (rows 4096..8192):
 // three block-rows per wave is the best trade between panel re-reads (fewer
@@ -1318,14 +1319,26 @@ static int tile_launch(const TlProblem *probs, int nlin, const f16 *X, int M, in
     a.total = nrp * a.ncg * nlin;
     a.ipw = 1;
     if (mode == TL_PLAN && nchunk == 1) {
-        // persistent workgroups: as many items of one row panel per workgroup
-        // as still leaves every CU its share of workgroups
+        // Persistent workgroups: d items of one row panel per workgroup, d a
+        // divisor of the items per panel.  A workgroup costs one panel fetch
+        // (about 2/3 of an item) plus d items, and the launch runs in
+        // ceil(workgroups / resident slots) rounds; take the cheapest d.
         const int per_rp = a.ncg * nlin;
-        for (int d = per_rp; d > 1; d--)
-            if (per_rp % d == 0 && a.total / d >= g_tile_min_wgs) {
+        const long slots = g_tile_min_wgs; // two workgroups per CU
+        double best = 0.0;
+        for (int d = 1; d <= per_rp; d++) {
+            if (per_rp % d)
+                continue;
+            const long nwg = a.total / d;
+            const long rounds = (nwg + slots - 1) / slots;
+            const double cost = (double)rounds * (2.0 / 3.0 + d);
+            if (a.ipw == 1 && d == 1) {
+                best = cost;
+            } else if (cost < best * 0.999) {
+                best = cost;
                 a.ipw = d;
-                break;
             }
+        }
         if (g_tile_ipw > 0)
             a.ipw = g_tile_ipw;
     }
@@ -1401,6 +1414,10 @@ extern "C" int et_tuning_set(const char *key, int value) {
     }
     if (key && !strcmp(key, "tile_ln_chunked")) {
         et::g_tile_ln_chunked = value;
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "tile_ln_min_panels")) {
+        et::g_tile_ln_min_panels = value > 0 ? value : 96;
         return ET_OK;
     }
     if (key && !strcmp(key, "tile_fuse_ln")) {
@@ -1620,6 +1637,10 @@ extern "C" int et_tile_plan_ln_fusable(const et_tile_plan *plan) {
                : 0;
 }
 
+// The fused kernels run one workgroup per 32-row panel; with few rows that
+// leaves most CUs idle and the two-launch form (more, smaller workgroups) wins.
+static bool ln_fusion_pays(int M) { return M >= 32 * et::g_tile_ln_min_panels; }
+
 extern "C" int et_tile_plan_run_ln(const et_tile_plan *plan, void *Y, const void *X,
                                    const void *skip, const void *gamma, const void *beta, int M,
                                    void *stream) {
@@ -1632,8 +1653,8 @@ extern "C" int et_tile_plan_run_ln(const et_tile_plan *plan, void *Y, const void
     if (M == 0)
         return ET_OK;
     const int nbr = plan->out_feat / 16;
-    if (!et_tile_plan_ln_fusable(plan)) {
-        // rows too wide for one workgroup: the two kernels, one after the other
+    if (!et_tile_plan_ln_fusable(plan) || (!ln_fusion_pays(M) && Y != skip)) {
+        // rows too wide for one workgroup, or too few of them: the two kernels, one after the other
         ET_REQUIRE(Y != skip, ET_ERR_INVALID_ARG,
                    "et_tile_plan_run_ln: Y must not alias skip for out_feat=%d", plan->out_feat);
         const int rc = et_tile_plan_run(plan, Y, X, M, 0, stream);

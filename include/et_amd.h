@@ -287,6 +287,8 @@ int et_device_synchronize(void);
  *   "tile_ipw"        work items per persistent workgroup of a planned linear
  *   "tile_fuse_ln"    0: et_tile_plan_run_ln runs the linear and the LayerNorm
  *                     as two launches; 1 (default): fused where the rows fit
+ *   "tile_ln_min_panels" fewest 32-row panels for which et_tile_plan_run_ln
+ *                     fuses (default 96; below, two launches are faster)
  *   "tile_ln_chunked" 0: fused LayerNorm with K > 992 uses the single-buffer
  *                     kernel; 1 (default): the double-buffered one
  *   "ln_rows"         rows per wave of et_skip_layernorm (1, 2, 4)
