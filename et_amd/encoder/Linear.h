@@ -2,6 +2,7 @@
 // meaning as encoder/Linear.h of the reference; the device work goes through
 // the C ABI (et_amd.h).
 #pragma once
+#include <algorithm>
 #include <utility>
 #include <vector>
 
@@ -80,6 +81,10 @@ class Linear_row {
     int row_id_size; // surviving rows
     Weight<half> bias;
     bool is_gelu;    // added: GELU on the compact output (a row-pruned FFN1)
+    // the compact rows as a fully populated tile_mat: the planned tile kernels
+    // (panel in LDS, pipelined weight stream) then serve the dense product too;
+    // null when in_feat is not a multiple of 16
+    et_tile_plan *plan;
 
     static int multiple_16(int x) { return ((x + 15) / 16) * 16; }
 
@@ -89,7 +94,7 @@ class Linear_row {
         : in_feat(in_feat_), out_feat(out_feat_), size(size_), nhead(nhead_),
           weight(in_feat_ * multiple_16(row_id_size_)), row_id(row_id_, row_id_size_ > 0 ? row_id_size_ : 1),
           head_ptr(nhead_ + 1), nrow(multiple_16(row_id_size_)), row_id_size(row_id_size_),
-          bias(multiple_16(row_id_size_)), is_gelu(is_gelu_) {
+          bias(multiple_16(row_id_size_)), is_gelu(is_gelu_), plan(nullptr) {
         // padded rows must contribute nothing: zero the buffers first
         etChk(et_fill_zero(weight.get(), sizeof(half) * (size_t)in_feat * nrow, nullptr));
         etChk(et_fill_zero(bias.get(), sizeof(half) * (size_t)nrow, nullptr));
@@ -99,14 +104,38 @@ class Linear_row {
         std::vector<int> h_head_ptr(nhead + 1);
         etChk(et_head_ptr(row_id_, row_id_size, nhead, out_feat / nhead, h_head_ptr.data()));
         head_ptr.set(h_head_ptr.data());
+        if (in_feat % 16 == 0) {
+            const int bcols = in_feat / 16, brows = nrow / 16;
+            std::vector<half> wpad((size_t)nrow * in_feat, (half)0), bpad(nrow, (half)0);
+            std::copy(weight_, weight_ + (size_t)row_id_size * in_feat, wpad.begin());
+            std::copy(bias_, bias_ + row_id_size, bpad.begin());
+            std::vector<int> rp(brows + 1), ro((size_t)brows * bcols);
+            for (int y = 0; y <= brows; y++)
+                rp[y] = y * bcols;
+            for (int y = 0; y < brows; y++)
+                for (int x = 0; x < bcols; x++)
+                    ro[(size_t)y * bcols + x] = x * 16;
+            std::vector<half> data((size_t)brows * bcols * 256);
+            etChk(et_tile_pack(wpad.data(), nrow, in_feat, rp.data(), ro.data(), data.data()));
+            etChk(et_tile_plan_create(&plan, in_feat, nrow, brows * bcols, data.data(), rp.data(), ro.data(),
+                                      bpad.data()));
+        }
     }
-    Linear_row(Linear_row &&) noexcept = default;
+    Linear_row(Linear_row &&o) noexcept
+        : in_feat(o.in_feat), out_feat(o.out_feat), size(o.size), nhead(o.nhead), weight(std::move(o.weight)),
+          row_id(std::move(o.row_id)), head_ptr(std::move(o.head_ptr)), nrow(o.nrow),
+          row_id_size(o.row_id_size), bias(std::move(o.bias)), is_gelu(o.is_gelu), plan(o.plan) {
+        o.plan = nullptr;
+    }
     Linear_row(const Linear_row &) = delete;
+    ~Linear_row() { et_tile_plan_destroy(plan); }
 
     // encoder/Linear.h:68-71; the cuBLAS handle becomes a stream
     void run(half *out, half *in, void *stream) const { run_rows(out, in, size, stream); }
     void run_rows(half *out, half *in, int rows, void *stream) const {
-        if (is_gelu)
+        if (plan)
+            etChk(et_tile_plan_run(plan, out, in, rows, is_gelu ? 1 : 0, stream));
+        else if (is_gelu)
             etChk(et_row_spmm_add_bias_gelu(out, in, weight.get(), bias.get(), rows, nrow, in_feat, stream));
         else
             etChk(et_row_spmm_add_bias(out, in, weight.get(), bias.get(), rows, nrow, in_feat, stream));
