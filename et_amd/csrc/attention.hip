@@ -366,27 +366,30 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
             // ---- scores, transposed: st[ksub][qs][r] = S[q = c16][key = 16 ksub + 4 g4 + r]
             f32x4 st[4][QS];
             if (!SHAREDQK) {
-                // all K fragments of the tile are requested from LDS first, then
-                // the MFMAs run with the dependent pair (s, s+1) eight issues apart
-                f16x8 kfr[4][DK];
+                // K fragments are read one 16-key subtile ahead of the MFMAs that
+                // use them (two subtiles' worth of registers instead of four)
+                f16x8 kfr[2][DK];
 #pragma unroll
-                for (int ksub = 0; ksub < 4; ksub++)
+                for (int s = 0; s < DK; s++)
+                    kfr[0][s] = *reinterpret_cast<const f16x8 *>(ks + c16 * LDK + s * 32 + g4 * 8);
 #pragma unroll
-                    for (int s = 0; s < DK; s++)
-                        kfr[ksub][s] = *reinterpret_cast<const f16x8 *>(
-                            ks + (ksub * 16 + c16) * LDK + s * 32 + g4 * 8);
+                for (int ksub = 0; ksub < 4; ksub++) {
+                    if (ksub + 1 < 4) {
 #pragma unroll
-                for (int ksub = 0; ksub < 4; ksub++)
+                        for (int s = 0; s < DK; s++)
+                            kfr[(ksub + 1) & 1][s] = *reinterpret_cast<const f16x8 *>(
+                                ks + ((ksub + 1) * 16 + c16) * LDK + s * 32 + g4 * 8);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int qs = 0; qs < QS; qs++)
                         st[ksub][qs] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int s = 0; s < DK; s++)
-#pragma unroll
-                    for (int ksub = 0; ksub < 4; ksub++)
+                    for (int s = 0; s < DK; s++)
 #pragma unroll
                         for (int qs = 0; qs < QS; qs++)
-                            st[ksub][qs] = mfma16x16x32(kfr[ksub][s], qf[qs][s], st[ksub][qs]);
+                            st[ksub][qs] = mfma16x16x32(kfr[ksub & 1][s], qf[qs][s], st[ksub][qs]);
+                }
             } else {
 #pragma unroll
                 for (int qs = 0; qs < QS; qs++) {
@@ -485,11 +488,9 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                                        ph[kk * 4 + 2][0], ph[kk * 4 + 2][1], ph[kk * 4 + 3][0], ph[kk * 4 + 3][1]};
             }
 
-            // ---- O^T += V^T P^T, same ordering: all V^T fragments first
+            // ---- O^T += V^T P^T, V^T fragments read one 16-column subtile ahead
             {
-                f16x8 vfr[DV][2];
-#pragma unroll
-                for (int d = 0; d < DV; d++)
+                auto load_v = [&](int d, f16x8 (&dst)[2]) {
 #pragma unroll
                     for (int kk = 0; kk < 2; kk++) {
                         f16x4 v0, v1;
@@ -509,15 +510,22 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                             v0 = *reinterpret_cast<const f16x4 *>(vrow);
                             v1 = *reinterpret_cast<const f16x4 *>(vrow + 16);
                         }
-                        vfr[d][kk] = f16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                        dst[kk] = f16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
                     }
+                };
+                f16x8 vfr[2][2];
+                load_v(0, vfr[0]);
 #pragma unroll
-                for (int kk = 0; kk < 2; kk++)
+                for (int d = 0; d < DV; d++) {
+                    if (d + 1 < DV)
+                        load_v(d + 1, vfr[(d + 1) & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int d = 0; d < DV; d++)
+                    for (int kk = 0; kk < 2; kk++)
 #pragma unroll
                         for (int qs = 0; qs < QS; qs++)
-                            ot[d][qs] = mfma16x16x32(vfr[d][kk], pf[qs][kk], ot[d][qs]);
+                            ot[d][qs] = mfma16x16x32(vfr[d & 1][kk], pf[qs][kk], ot[d][qs]);
+                }
             }
         };
 

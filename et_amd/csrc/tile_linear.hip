@@ -245,10 +245,8 @@ __device__ __forceinline__ void tl_static_for(F &&f) {
 // One pair's operands: 16 bytes of W per lane and the lane's X offset.  The
 // pair's address is wave-uniform (scalar registers) and the lane's part a
 // 32-bit offset, so the loads need no vector address arithmetic.
-__device__ __forceinline__ void tl_load_pair(const f16 *data, const int *poff, int q, unsigned lane_w,
-                                             unsigned hi, f16x8 &w, int &o) {
-    const char *wq = reinterpret_cast<const char *>(data) + (size_t)q * 1024; // uniform
-    const char *oq = reinterpret_cast<const char *>(poff) + (size_t)q * 8;    // uniform
+__device__ __forceinline__ void tl_load_pair_at(const char *wq, const char *oq, unsigned lane_w,
+                                                unsigned hi, f16x8 &w, int &o) {
     // (the empty asm keeps the compiler from folding the lane offsets into
     // loop-invariant 64-bit vector addresses, which costs two 64-bit vector
     // adds per pair instead of none)
@@ -256,6 +254,11 @@ __device__ __forceinline__ void tl_load_pair(const f16 *data, const int *poff, i
     asm("" : "+v"(lo), "+v"(lw));
     o = *reinterpret_cast<const int *>(oq + lo);
     w = *reinterpret_cast<const f16x8 *>(wq + lw);
+}
+__device__ __forceinline__ void tl_load_pair(const f16 *data, const int *poff, int q, unsigned lane_w,
+                                             unsigned hi, f16x8 &w, int &o) {
+    tl_load_pair_at(reinterpret_cast<const char *>(data) + (size_t)q * 1024,
+                    reinterpret_cast<const char *>(poff) + (size_t)q * 8, lane_w, hi, w, o);
 }
 
 __device__ __forceinline__ void tl_preload(const f16 *data, const int *poff, unsigned lane_w, unsigned hi,
@@ -287,6 +290,10 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
     xb[0] = *reinterpret_cast<const f16x8 *>(xlane + o[0] + xrow16);
     xa[1] = xb[1] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     int q = q0;
+    // running (wave-uniform) addresses of pair q + TL_DEPTH: a stage adds a
+    // constant, which goes into the load's immediate offset
+    const char *wp = reinterpret_cast<const char *>(data) + (size_t)(q0 + TL_DEPTH) * 1024;
+    const char *op = reinterpret_cast<const char *>(poff) + (size_t)(q0 + TL_DEPTH) * 8;
     auto stage = [&](auto ic) {
         constexpr int I = decltype(ic)::value;
         constexpr int S = I % TL_DEPTH, SN = (I + 1) % TL_DEPTH, P = I & 1;
@@ -297,7 +304,10 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
         __builtin_amdgcn_sched_barrier(0);
         cur0 = mfma16x16x32(w[S], xa[P], cur0);
         cur1 = mfma16x16x32(w[S], xb[P], cur1);
-        tl_load_pair(data, poff, min(q + I + TL_DEPTH, qlast), lane_w, hi, w[S], o[S]);
+        // (not clamped to the end of the stream: its last stages request pairs
+        // that belong to other waves, or the spare pairs behind the array, and
+        // never use them)
+        tl_load_pair_at(wp + I * 1024, op + I * 8, lane_w, hi, w[S], o[S]);
         if (q + I + 1 == bend) { // block-row j is complete
             flush(j, cur0, cur1);
             cur0 = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -311,8 +321,11 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
             }
         }
     };
-    for (; q + TL_DEPTH <= qend; q += TL_DEPTH) // straight-line body: counted waits
+    for (; q + TL_DEPTH <= qend; q += TL_DEPTH) { // straight-line body: counted waits
         tl_static_for<0, TL_DEPTH>(stage);
+        wp += TL_DEPTH * 1024;
+        op += TL_DEPTH * 8;
+    }
     tl_static_for<0, TL_DEPTH - 1>([&](auto ic) {
         if (q + decltype(ic)::value < qend)
             stage(ic);
@@ -625,6 +638,15 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_plan_kernel(const TlArgs 
 //    item instead of three;
 //  * items that share the row panel reuse it without any barrier.
 // ---------------------------------------------------------------------------
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences
+// global memory, which would make every wave drain the weight pairs it has
+// just requested; this one is for hand-overs of LDS buffers.
+__device__ __forceinline__ void tl_barrier_lds() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 struct TlItem {
     int rp, lin, cg, bn0, nbr, N;
     f16 *Y;
@@ -764,6 +786,7 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
     const int per_rp = a.ncg * a.nlin;
     const int rp0 = it0 / per_rp, rest0 = it0 - rp0 * per_rp;
     TlItem cur = tl_item(rp0, rest0 / a.ncg, rest0 % a.ncg);
+
     int bvec = TL_BVEC(cur);
     f16x4 b4[NB];
     TL_BIAS(b4, cur)
@@ -890,15 +913,6 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
 // ---------------------------------------------------------------------------
 constexpr int TL_CWAVES = 12;
 constexpr int TL_CTHREADS = (TL_CWAVES + 1) * 64;
-
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences
-// global memory, which would make every wave drain the weight pairs it has
-// just requested; here only the panel buffers in LDS change hands.
-__device__ __forceinline__ void tl_barrier_lds() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
 
 template <int NB>
 __global__ void __launch_bounds__(TL_CTHREADS) tile_linear_chunked_ln_kernel(const TlArgs a) {
@@ -1549,11 +1563,14 @@ extern "C" int et_tile_plan_create(et_tile_plan **plan, int in_feat, int out_fea
         }
     }
     cptr[(size_t)nbr * nchunk] = (int)off.size();
-    // one spare all-zero pair behind the last one: the kernels request the
-    // first pairs of a wave's stream before they know whether it is empty
-    off.push_back(0);
-    off.push_back(0);
-    packed.insert(packed.end(), 512, (uint16_t)0);
+    // spare all-zero pairs behind the last one: the kernels request the first
+    // pairs of a wave's stream before they know whether it is empty, and a
+    // stream's last stages request up to 2*TL_DEPTH pairs past its end
+    for (int i = 0; i < 2 * TL_DEPTH + 1; i++) {
+        off.push_back(0);
+        off.push_back(0);
+        packed.insert(packed.end(), 512, (uint16_t)0);
+    }
 
     et_tile_plan *p = new et_tile_plan();
     memset(p, 0, sizeof(*p));
