@@ -141,10 +141,17 @@ def main():
          4 * B * S * S * D, 8 * B * S * D + 2 * S * S, "mfma"),
         ("tile_linear o (768->768) + skip + LayerNorm", lambda: L[3].run_ln(b[3], x, gam[0], gam[1], out=b[0]),
          tile_flops(T, nt[3]), tile_bytes(T, D, D, nt[3]) + 2 * T * D + 4 * D, "hbm"),
-        ("tile_linear ffn1+gelu (768->3072)", lambda: L[4].run(b[0], out=ffn), tile_flops(T, nt[4]), tile_bytes(T, DFF, D, nt[4]), "hbm"),
-        ("tile_linear ffn2 (3072->768) + skip + LayerNorm", lambda: L[5].run_ln(ffn, b[0], gam[2], gam[3], out=y),
-         tile_flops(T, nt[5]), tile_bytes(T, D, DFF, nt[5]) + 2 * T * D + 4 * D, "hbm"),
+        # the feed-forward block in one launch: X in, Y out, both weights once; the hidden activations stay in LDS
+        ("feed-forward 768->3072->768 (gelu) + skip + LayerNorm, fused", lambda: Linear_tile.run_ffn_ln(L[4], L[5], b[0], b[0], gam[2], gam[3], out=y),
+         tile_flops(T, nt[4]) + tile_flops(T, nt[5]),
+         tile_bytes(T, DFF, D, nt[4]) + tile_bytes(T, D, DFF, nt[5]) - 2 * 2 * T * DFF + 4 * D, "hbm"),
     ]
+    if not Linear_tile.ffn_fusable(L[4], L[5]):  # (tuning override): the two launches through a hidden buffer
+        steps_def[-1:] = [
+            ("tile_linear ffn1+gelu (768->3072)", lambda: L[4].run(b[0], out=ffn), tile_flops(T, nt[4]), tile_bytes(T, DFF, D, nt[4]), "hbm"),
+            ("tile_linear ffn2 (3072->768) + skip + LayerNorm", lambda: L[5].run_ln(ffn, b[0], gam[2], gam[3], out=y),
+             tile_flops(T, nt[5]), tile_bytes(T, D, DFF, nt[5]) + 2 * T * D + 4 * D, "hbm"),
+        ]
     nk = len(steps_def)
     reps = max(20, min(args.steps, 100))
     for _ in range(5):

@@ -91,6 +91,22 @@ int et_linear_tile_run_rows_ln(const et_linear_tile *h, void *out, const void *i
                             static_cast<const half *>(beta), rows, stream);
     });
 }
+int et_linear_tile_run_rows_ffn_ln(const et_linear_tile *first, const et_linear_tile *second, void *out,
+                                   const void *in, void *hidden, const void *skip, const void *gamma,
+                                   const void *beta, int rows, void *stream) {
+    if (!first || !second) {
+        et::set_error("et_linear_tile_run_rows_ffn_ln: null handle");
+        return ET_ERR_INVALID_ARG;
+    }
+    return guarded([&] {
+        Linear_tile::run_rows_ffn_ln(first->impl, second->impl, H(out), H(in), H(hidden),
+                                     static_cast<const half *>(skip), static_cast<const half *>(gamma),
+                                     static_cast<const half *>(beta), rows, stream);
+    });
+}
+int et_linear_tile_ffn_fusable(const et_linear_tile *first, const et_linear_tile *second) {
+    return first && second && Linear_tile::ffn_fusable(first->impl, second->impl) ? 1 : 0;
+}
 int et_linear_tile_run_multi(const et_linear_tile *const *hs, void *const *outs, int n, const void *in,
                              int rows, void *stream) {
     if (!hs || !outs || n < 1 || n > 4) {

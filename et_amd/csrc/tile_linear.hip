@@ -294,7 +294,7 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
     // constant, which goes into the load's immediate offset
     const char *wp = reinterpret_cast<const char *>(data) + (size_t)(q0 + TL_DEPTH) * 1024;
     const char *op = reinterpret_cast<const char *>(poff) + (size_t)(q0 + TL_DEPTH) * 8;
-    auto stage = [&](auto ic) {
+    auto stage = [&](auto ic, auto always) {
         constexpr int I = decltype(ic)::value;
         constexpr int S = I % TL_DEPTH, SN = (I + 1) % TL_DEPTH, P = I & 1;
         xa[P ^ 1] = *reinterpret_cast<const f16x8 *>(xlane + o[SN]);
@@ -304,10 +304,11 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
         __builtin_amdgcn_sched_barrier(0);
         cur0 = mfma16x16x32(w[S], xa[P], cur0);
         cur1 = mfma16x16x32(w[S], xb[P], cur1);
-        // (not clamped to the end of the stream: its last stages request pairs
-        // that belong to other waves, or the spare pairs behind the array, and
-        // never use them)
-        tl_load_pair_at(wp + I * 1024, op + I * 8, lane_w, hi, w[S], o[S]);
+        // pair q + I + TL_DEPTH; the last stages of a stream request nothing:
+        // a request still in flight when the stream ends would make the next
+        // use of these registers wait out a full memory latency
+        if (decltype(always)::value || q + I + TL_DEPTH < qend)
+            tl_load_pair_at(wp + I * 1024, op + I * 8, lane_w, hi, w[S], o[S]);
         if (q + I + 1 == bend) { // block-row j is complete
             flush(j, cur0, cur1);
             cur0 = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -321,14 +322,14 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
             }
         }
     };
-    for (; q + TL_DEPTH <= qend; q += TL_DEPTH) { // straight-line body: counted waits
-        tl_static_for<0, TL_DEPTH>(stage);
+    for (; q + 2 * TL_DEPTH <= qend; q += TL_DEPTH) { // straight-line body: counted waits
+        tl_static_for<0, TL_DEPTH>([&](auto ic) { stage(ic, std::true_type()); });
         wp += TL_DEPTH * 1024;
         op += TL_DEPTH * 8;
     }
-    tl_static_for<0, TL_DEPTH - 1>([&](auto ic) {
+    tl_static_for<0, 2 * TL_DEPTH - 1>([&](auto ic) {
         if (q + decltype(ic)::value < qend)
-            stage(ic);
+            stage(ic, std::false_type());
     });
 }
 
@@ -1057,6 +1058,227 @@ __global__ void __launch_bounds__(TL_CTHREADS) tile_linear_chunked_ln_kernel(con
 }
 
 // ---------------------------------------------------------------------------
+// Fused feed-forward block: Y = LayerNorm(skip + W2 * gelu(W1 * X + b1) + b2)
+// in ONE launch (encoder/encoder.cu:33-41 runs it as MLP1, MLP2 and
+// skip_layernorm with the [rows x ffn] intermediate written to and read back
+// from memory).  One workgroup of 16 waves per 32-row panel keeps the panel of
+// X in LDS and walks the hidden dimension in chunks of the second plan's
+// chunk width: phase p computes hidden columns [p*KC, (p+1)*KC) with the first
+// linear (bias, GELU, rounded to half exactly like the stored intermediate)
+// into one of two LDS buffers, then multiplies that buffer with chunk p of the
+// second linear into register accumulators that live across all phases.  The
+// hidden activations never leave the CU.  With two hidden buffers a single
+// barrier per phase is enough: phase p+1's first linear overwrites the buffer
+// that phase p-1's second linear read, and every wave has passed barrier p
+// since.  Each wave owns NB block-rows of either linear per phase; the first
+// pairs of a stream are requested one whole stream ahead (two register sets).
+// arguments: linear 0 = first (N[0] = hidden width), linear 1 = second
+// (N[1] = output width, Y[1] = output), K = input width, KC / nchunk = the
+// second plan's chunking.
+// ---------------------------------------------------------------------------
+constexpr int TL_FFN_WAVES = 16;
+constexpr int TL_FFN_MAX_PHASES = 16;
+
+// Workgroup-local event counters in LDS: every wave adds one when it has
+// finished a step, and a wave that needs everyone's result waits for the
+// count.  Unlike s_barrier this lets a wave run ahead with other work and
+// wait only when it is a whole step ahead of the slowest wave.
+__device__ __forceinline__ void tl_signal(unsigned *ctr, int lane) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local"); // this wave's LDS writes first
+    if (lane == 0)
+        __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void tl_wait_count(unsigned *ctr, unsigned target) {
+    while ((unsigned)__builtin_amdgcn_readfirstlane(
+               (int)__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) < target)
+        __builtin_amdgcn_s_sleep(1);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+template <int NB>
+__global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const TlArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
+    f16 *xs = reinterpret_cast<f16 *>(tl_smem);
+    const int rp = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3);
+    if (rp >= a.total)
+        return;
+    constexpr int NW = TL_FFN_WAVES;
+    TlCtx x;
+    x.lin = 1;
+    x.cg = 0;
+    x.m0 = rp * TL_BM;
+    x.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    x.lane = threadIdx.x & 63;
+    x.c16 = x.lane & 15;
+    x.g4 = x.lane >> 4;
+    x.khalf8 = (x.g4 & 1) * 8;
+    x.hi = x.lane >> 5;
+    x.ldx = a.K + ((a.K & 31) ? 0 : TL_PAD);
+    x.bn_wg = 0;
+    x.bn0 = x.wave * NB;
+    x.ld_r = x.ld_c = 0;
+    const int wave = x.wave, lane = x.lane, c16 = x.c16, g4 = x.g4, hi = x.hi;
+    const int ldx = x.ldx;
+    const int ldh = a.KC + ((a.KC & 31) ? 0 : TL_PAD);
+    f16 *const hs = xs + TL_BM * ldx; // two hidden buffers behind the X panel
+    const int hbuf = TL_BM * ldh;
+    // event counters behind the hidden buffers: [p] first linear of phase p
+    // done, [TL_FFN_MAX_PHASES + p] second linear of phase p done
+    unsigned *const ctr = reinterpret_cast<unsigned *>(hs + 2 * hbuf);
+    const int N1 = a.N[0], N2 = a.N[1], nbr1 = N1 >> 4, nbr2 = N2 >> 4;
+    const int hbr = a.KC >> 4; // hidden block-rows per phase
+    const unsigned lane_w = hi * 256 + c16 * 16 + x.khalf8;
+
+    // the X panel: wave w fetches rows 2w and 2w+1
+    {
+        const int pcpr = a.K >> 3;
+#pragma unroll
+        for (int rr = 0; rr < TL_BM / NW; rr++) {
+            const int r = wave * (TL_BM / NW) + rr;
+            if (x.m0 + r < a.M) {
+                const f16 *src = a.X + (size_t)(x.m0 + r) * a.K;
+                if (lane < pcpr)
+                    load_lds16(src + lane * 8, xs + r * ldx);
+                if (64 + lane < pcpr)
+                    load_lds16(src + (64 + lane) * 8, xs + r * ldx + 512);
+            }
+        }
+    }
+    if (threadIdx.x < 2 * TL_FFN_MAX_PHASES)
+        ctr[threadIdx.x] = 0;
+    const int *const cptr1 = a.cptr[0], *const cptr2 = a.cptr[1];
+    const f16 *const data1 = a.data[0], *const data2 = a.data[1];
+    const int *const poff1 = a.row_offset[0], *const poff2 = a.row_offset[1];
+    // pair-index boundaries of the wave's block-rows (lane j: start of block-row
+    // j, lane NB: end of the last one); block-rows past the phase's range or the
+    // matrix are empty
+    // (read with scalar loads: they do not queue behind the weight pairs in
+    // flight, and no wait for them drains those)
+    typedef const __attribute__((address_space(4))) int *ScalarInts;
+    auto bvec_of = [&](ScalarInts base, int i0, int lim) {
+        int v = 0;
+#pragma unroll
+        for (int k = NB; k >= 0; k--) {
+            const int s = base[min(i0 + k, lim)] >> 1;
+            v = (lane == k) ? s : v;
+        }
+        return v;
+    };
+#define TL_FFN_BVEC1(p_) bvec_of((ScalarInts)cptr1, (p_) * hbr + wave * NB, min(((p_) + 1) * hbr, nbr1))
+#define TL_FFN_BVEC2(p_) bvec_of((ScalarInts)cptr2 + (p_) * nbr2, wave * NB, nbr2)
+#define TL_FFN_BIAS1(dst_, p_)                                                                    \
+    _Pragma("unroll") for (int k = 0; k < NB; k++)                                                \
+        dst_[k] = *reinterpret_cast<const f16x4 *>(                                               \
+            a.bias[0] + min((p_) * hbr + wave * NB + k, nbr1 - 1) * 16 + g4 * 4);
+    f32x4 acc[NB][2];
+    f16x4 b2[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        acc[j][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+        acc[j][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+        b2[j] = f16x4{0, 0, 0, 0};
+        if (x.bn0 + j < nbr2)
+            b2[j] = *reinterpret_cast<const f16x4 *>(a.bias[1] + (x.bn0 + j) * 16 + g4 * 4);
+    }
+    const char *const xlane1 = reinterpret_cast<const char *>(xs + c16 * ldx + x.khalf8);
+    const int xrow1 = 16 * ldx * 2, xrow2 = 16 * ldh * 2;
+
+    // One stream of the first linear: hidden columns of phase p_ (bias, GELU,
+    // half) into hidden buffer p_ & 1.  w_/o_ hold its first pairs already.
+#define TL_FFN_FIRST(p_, bvec_, b1_, w_, o_)                                                      \
+    {                                                                                             \
+        f16 *const hlane = hs + ((p_) & 1) * hbuf + c16 * ldh + wave * NB * 16 + g4 * 4;          \
+        const int q0_ = __builtin_amdgcn_readfirstlane(bvec_), qe_ = __builtin_amdgcn_readlane(bvec_, NB); \
+        tl_stream<NB>(xlane1, xrow1, data1, poff1, lane_w, hi, q0_, qe_, max(qe_ - 1, q0_), bvec_, w_, o_, \
+                      [&](int j, f32x4 c0, f32x4 c1) {                                            \
+                          f16x4 bj = f16x4{0, 0, 0, 0};                                           \
+                          _Pragma("unroll") for (int k = 0; k < NB; k++)                          \
+                              bj += b1_[k] * ((j == k) ? (f16)1 : (f16)0);                        \
+                          tl_stage_tile<true>(hlane + j * 16, ldh, c0, c1, bj);                   \
+                      });                                                                         \
+        /* block-rows of this phase without any tile: bias only */                                \
+        const int lim1 = min(((p_) + 1) * hbr, nbr1);                                             \
+        _Pragma("unroll") for (int k = 0; k < NB; k++)                                            \
+            if ((p_) * hbr + wave * NB + k < lim1 &&                                              \
+                __builtin_amdgcn_readlane(bvec_, k) == __builtin_amdgcn_readlane(bvec_, k + 1))   \
+                tl_stage_tile<true>(hlane + k * 16, ldh, f32x4{0.f, 0.f, 0.f, 0.f},               \
+                                    f32x4{0.f, 0.f, 0.f, 0.f}, b1_[k]);                           \
+        tl_signal(ctr + (p_), lane);                                                              \
+    }
+#define TL_FFN_PRELOAD(data_, poff_, bvec_, w_, o_)                                               \
+    {                                                                                             \
+        const int q0_ = __builtin_amdgcn_readfirstlane(bvec_), qe_ = __builtin_amdgcn_readlane(bvec_, NB); \
+        tl_preload(data_, poff_, lane_w, hi, q0_, max(qe_ - 1, q0_), w_, o_);                     \
+    }
+
+    // The streams run in the order F(0), F(1), S(0), F(2), S(1), ..., S(last)
+    // (F = first linear, S = second): the first linear stays one phase ahead,
+    // so what a wave waits for was finished by most waves a stream ago.
+    // Register set A serves F(0) and every S, set B every later F.
+    f16x8 wA[TL_DEPTH], wB[TL_DEPTH];
+    int oA[TL_DEPTH], oB[TL_DEPTH];
+    int bvecF = TL_FFN_BVEC1(0);
+    f16x4 b1[NB];
+    TL_FFN_BIAS1(b1, 0)
+    int bvecFn = TL_FFN_BVEC1(min(1, a.nchunk - 1));
+    f16x4 b1n[NB];
+    TL_FFN_BIAS1(b1n, min(1, a.nchunk - 1))
+    int bvecS = TL_FFN_BVEC2(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's part of the panel has landed
+    TL_FFN_PRELOAD(data1, poff1, bvecF, wA, oA)
+    tl_barrier_lds(); // ... and everyone else's; the counters are zero
+    if (a.nchunk > 1)
+        TL_FFN_PRELOAD(data1, poff1, bvecFn, wB, oB)
+    TL_FFN_FIRST(0, bvecF, b1, wA, oA)
+
+    for (int p = 0; p < a.nchunk; p++) {
+        // operands of the streams after the next two
+        const int bvecSn = TL_FFN_BVEC2(min(p + 1, a.nchunk - 1));
+        const int bvecF2 = TL_FFN_BVEC1(min(p + 2, a.nchunk - 1));
+        f16x4 b1n2[NB];
+        TL_FFN_BIAS1(b1n2, min(p + 2, a.nchunk - 1))
+        TL_FFN_PRELOAD(data2, poff2, bvecS, wA, oA) // S(p), a stream ahead
+        if (p + 1 < a.nchunk) {
+            if (p >= 1) // F(p+1) overwrites the buffer that S(p-1) read
+                tl_wait_count(ctr + TL_FFN_MAX_PHASES + p - 1, NW);
+            TL_FFN_FIRST(p + 1, bvecFn, b1n, wB, oB)
+        }
+        if (p + 2 < a.nchunk)
+            TL_FFN_PRELOAD(data1, poff1, bvecF2, wB, oB) // F(p+2), a stream ahead
+        tl_wait_count(ctr + p, NW); // hidden buffer p & 1 is complete
+        {
+            const char *const xlane2 =
+                reinterpret_cast<const char *>(hs + (p & 1) * hbuf + c16 * ldh + x.khalf8);
+            const int q0_ = __builtin_amdgcn_readfirstlane(bvecS), qe_ = __builtin_amdgcn_readlane(bvecS, NB);
+            tl_stream<NB>(xlane2, xrow2, data2, poff2, lane_w, hi, q0_, qe_, max(qe_ - 1, q0_), bvecS, wA, oA,
+                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); });
+            tl_signal(ctr + TL_FFN_MAX_PHASES + p, lane);
+        }
+        bvecS = bvecSn;
+        bvecFn = bvecF2;
+#pragma unroll
+        for (int k = 0; k < NB; k++)
+            b1n[k] = b1n2[k];
+    }
+#undef TL_FFN_BVEC1
+#undef TL_FFN_BVEC2
+#undef TL_FFN_BIAS1
+#undef TL_FFN_FIRST
+#undef TL_FFN_PRELOAD
+
+    // output rows -> staging tiles over the (now unused) panel and hidden
+    // buffers, then skip connection + LayerNorm over whole rows
+    TlLnOperands<NB, NW, NW> lnop;
+    tl_ln_fetch(lnop, a, wave, lane, x.m0, N2);
+    tl_barrier_lds(); // every wave has left the hidden buffers
+    f16 *const stage0 = xs;
+    tl_epilogue_wave<NB, false, false>(a, x, stage0 + wave * tl_wave_stage_halves<NB>(), a.Y[1], N2, nbr2,
+                                       acc, b2);
+    __syncthreads(); // every wave's part of the rows is staged
+    tl_ln_rows(lnop, a, stage0, wave, lane, x.m0, a.Y[1], N2);
+}
+
+// ---------------------------------------------------------------------------
 // Generic kernel: the caller's own tile_mat (TL_RAW / TL_FILTER) or a dense
 // row-major weight (TL_DENSE).  Same mapping, plain per-block-row loops with
 // per-lane predicates.
@@ -1229,6 +1451,51 @@ static int launch_chunked_ln_inst(const TlArgs &a, size_t lds, hipStream_t st) {
 }
 
 static int g_tile_ln_chunked = 1;
+static int g_tile_fuse_ffn = 1; // et_tuning_set("tile_fuse_ffn")
+
+// LDS bytes of the fused feed-forward kernel: X panel, two hidden buffers (the
+// output staging tiles reuse their storage)
+static size_t ffn_lds_bytes(int K1, int KC2) {
+    const size_t ldx = K1 + ((K1 & 31) ? 0 : TL_PAD), ldh = KC2 + ((KC2 & 31) ? 0 : TL_PAD);
+    const size_t panels = (size_t)TL_BM * (ldx + 2 * ldh) * sizeof(f16) + 2 * TL_FFN_MAX_PHASES * sizeof(unsigned);
+    const size_t staging = (size_t)TL_FFN_WAVES * TL_BM * (16 * 3 + 8) * sizeof(f16);
+    return std::max(panels, staging);
+}
+
+static int tile_launch_ffn(const TlProblem &p1, const TlProblem &p2, const f16 *X, int M, int K1,
+                           int KC2, int nchunk2, const f16 *skip, const f16 *gamma, const f16 *beta,
+                           hipStream_t st) {
+    TlArgs a;
+    memset(&a, 0, sizeof(a));
+    for (int i = 0; i < TL_MAX_LIN; i++) {
+        const TlProblem &p = i == 0 ? p1 : p2;
+        a.Y[i] = p.Y;
+        a.cptr[i] = p.cptr;
+        a.row_offset[i] = p.row_offset;
+        a.data[i] = p.data;
+        a.bias[i] = p.bias;
+        a.N[i] = p.N;
+    }
+    a.X = X;
+    a.nlin = 2;
+    a.M = M;
+    a.K = K1;
+    a.KC = KC2;
+    a.nchunk = nchunk2;
+    a.ncg = 1;
+    a.total = (M + TL_BM - 1) / TL_BM;
+    a.ipw = 1;
+    a.per_xcd = (a.total + 7) / 8;
+    a.skip = skip;
+    a.gamma = gamma;
+    a.beta = beta;
+    const size_t lds = ffn_lds_bytes(K1, KC2);
+    auto k = tile_ffn_fused_kernel<3>;
+    ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_FFN_WAVES * 64), lds, st, a);
+    return launch_status("fused feed-forward launch");
+}
 
 static int tile_launch_ln(const TlProblem &p, const f16 *X, int M, int K, int KC, int nchunk,
                           const f16 *skip, const f16 *gamma, const f16 *beta, hipStream_t st) {
@@ -1424,6 +1691,10 @@ extern "C" int et_tuning_set(const char *key, int value) {
     }
     if (key && !strcmp(key, "tile_ipw")) {
         et::g_tile_ipw = value;
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "tile_fuse_ffn")) {
+        et::g_tile_fuse_ffn = value;
         return ET_OK;
     }
     if (key && !strcmp(key, "tile_ln_chunked")) {
@@ -1690,6 +1961,64 @@ extern "C" int et_tile_plan_run_ln(const et_tile_plan *plan, void *Y, const void
     return tile_launch_ln(pr, static_cast<const f16 *>(X), M, plan->in_feat, plan->KC, plan->nchunk,
                           static_cast<const f16 *>(skip), static_cast<const f16 *>(gamma),
                           static_cast<const f16 *>(beta), static_cast<hipStream_t>(stream));
+}
+
+extern "C" int et_tile_plan_ffn_fusable(const et_tile_plan *p1, const et_tile_plan *p2) {
+    using namespace et;
+    if (!p1 || !p2 || !g_tile_fuse_ffn)
+        return 0;
+    return p1->nchunk == 1 && p2->in_feat == p1->out_feat && p2->nchunk <= TL_FFN_MAX_PHASES &&
+                   p2->KC / 16 <= TL_FFN_WAVES * 3 &&
+                   p2->out_feat / 16 <= TL_FFN_WAVES * 3 && p2->out_feat % 8 == 0 &&
+                   ffn_lds_bytes(p1->in_feat, p2->KC) <= 160 * 1024
+               ? 1
+               : 0;
+}
+
+extern "C" int et_tile_plan_run_ffn_ln(const et_tile_plan *p1, const et_tile_plan *p2, void *Y,
+                                       const void *X, void *hidden, const void *skip,
+                                       const void *gamma, const void *beta, int M, void *stream) {
+    using namespace et;
+    ET_REQUIRE(p1 && p2 && Y && X && skip && gamma && beta, ET_ERR_INVALID_ARG,
+               "et_tile_plan_run_ffn_ln: null pointer");
+    ET_REQUIRE(M >= 0, ET_ERR_INVALID_ARG, "et_tile_plan_run_ffn_ln: M=%d", M);
+    ET_REQUIRE(p2->in_feat == p1->out_feat, ET_ERR_INVALID_ARG,
+               "et_tile_plan_run_ffn_ln: the second linear takes %d inputs, the first gives %d",
+               p2->in_feat, p1->out_feat);
+    ET_REQUIRE(aligned16(Y) && aligned16(X) && aligned16(skip) && aligned16(gamma) && aligned16(beta) &&
+                   aligned16(hidden),
+               ET_ERR_ALIGNMENT, "et_tile_plan_run_ffn_ln: pointers must be 16-byte aligned");
+    if (M == 0)
+        return ET_OK;
+    const bool fusable = et_tile_plan_ffn_fusable(p1, p2) != 0;
+    if (!fusable || (hidden && !ln_fusion_pays(M))) {
+        // the three steps one after the other, through the caller's buffer
+        ET_REQUIRE(hidden, ET_ERR_UNSUPPORTED,
+                   "et_tile_plan_run_ffn_ln: these shapes need the hidden buffer (%d x %d halves)", M,
+                   p1->out_feat);
+        const int rc = et_tile_plan_run(p1, hidden, X, M, 1, stream);
+        if (rc != ET_OK)
+            return rc;
+        return et_tile_plan_run_ln(p2, Y, hidden, skip, gamma, beta, M, stream);
+    }
+    TlProblem a, b;
+    a.Y = nullptr;
+    a.cptr = p1->d_cptr;
+    a.row_offset = p1->d_row_offset;
+    a.data = p1->d_data;
+    a.bias = p1->d_bias;
+    a.N = p1->out_feat;
+    a.nbr = p1->out_feat / 16;
+    b.Y = static_cast<f16 *>(Y);
+    b.cptr = p2->d_cptr;
+    b.row_offset = p2->d_row_offset;
+    b.data = p2->d_data;
+    b.bias = p2->d_bias;
+    b.N = p2->out_feat;
+    b.nbr = p2->out_feat / 16;
+    return tile_launch_ffn(a, b, static_cast<const f16 *>(X), M, p1->in_feat, p2->KC, p2->nchunk,
+                           static_cast<const f16 *>(skip), static_cast<const f16 *>(gamma),
+                           static_cast<const f16 *>(beta), static_cast<hipStream_t>(stream));
 }
 
 extern "C" int et_tile_plan_run(const et_tile_plan *plan, void *Y, const void *X, int M, int gelu,

@@ -62,6 +62,22 @@ class Linear_tile:
                                                rows, _stream()))
         return out
 
+    @staticmethod
+    def run_ffn_ln(first, second, x, skip, gamma, beta, out=None, hidden=None, rows=None):
+        """LayerNorm(half(second(gelu(first(x)))) + skip) * gamma + beta: the feed-forward block in one
+        launch.  `hidden` ([rows, first.out_feat]) is only used where the fused kernel does not apply;
+        None insists on the fused kernel."""
+        rows = x.shape[0] if rows is None else rows
+        out = out if out is not None else torch.empty((x.shape[0], second.out_feat), dtype=torch.float16, device=x.device)
+        check(lib().et_linear_tile_run_rows_ffn_ln(first._h, second._h, _dp(out), _dp(x),
+                                                   _dp(hidden) if hidden is not None else None, _dp(skip),
+                                                   _dp(gamma), _dp(beta), rows, _stream()))
+        return out
+
+    @staticmethod
+    def ffn_fusable(first, second):
+        return bool(lib().et_linear_tile_ffn_fusable(first._h, second._h))
+
     def _release(self):  # ownership moved into an encoder
         self._h = None
 

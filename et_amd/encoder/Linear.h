@@ -51,6 +51,21 @@ class Linear_tile {
     }
     bool ln_fusable() const { return et_tile_plan_ln_fusable(plan) != 0; }
 
+    // the feed-forward block in one launch: out = LayerNorm(half(second(gelu(first(in)))) + skip);
+    // `hidden` ([rows x first.out_feat]) is used only where the fused kernel does
+    // not apply or does not pay; see et_tile_plan_run_ffn_ln
+    static void run_rows_ffn_ln(const Linear_tile &first, const Linear_tile &second, half *out, half *in,
+                                half *hidden, const half *skip, const half *gamma, const half *beta,
+                                int rows, void *stream) {
+        etRequire(first.is_gelu && !second.is_gelu,
+                  "Linear_tile::run_rows_ffn_ln: the first linear must be the GELU variant, the second not");
+        etChk(et_tile_plan_run_ffn_ln(first.plan, second.plan, out, in, hidden, skip, gamma, beta, rows,
+                                      stream));
+    }
+    static bool ffn_fusable(const Linear_tile &first, const Linear_tile &second) {
+        return et_tile_plan_ffn_fusable(first.plan, second.plan) != 0;
+    }
+
     static void run_multi(const Linear_tile *const *lin, half *const *outs, int n, half *in, int rows,
                           void *stream) {
         const et_tile_plan *plans[4];

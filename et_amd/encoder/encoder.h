@@ -99,10 +99,12 @@ class Encoder_base {
     // O projection, skip-LN with the layer input, FFN1+GELU, FFN2, skip-LN.
     void tail(half *out, half *in, half *attn, const Linear_tile &O, const Linear_tile &M1,
               const Linear_tile &M2, int nrows) {
-        // (each projection, its skip connection and LayerNorm are one launch)
+        // (the projection, its skip connection and LayerNorm are one launch, and
+        // so is the whole feed-forward block; its hidden buffer, units 1..4, is
+        // only touched where the fused kernel does not apply)
         O.run_rows_ln(buffers[0], attn, in, ln_gamma[0].get(), ln_beta[0].get(), nrows, stream);
-        M1.run_rows(buffers[1], buffers[0], nrows, stream); // spans buffers[1..4]
-        M2.run_rows_ln(out, buffers[1], buffers[0], ln_gamma[1].get(), ln_beta[1].get(), nrows, stream);
+        Linear_tile::run_rows_ffn_ln(M1, M2, out, buffers[0], buffers[1], buffers[0], ln_gamma[1].get(),
+                                     ln_beta[1].get(), nrows, stream);
     }
 };
 
@@ -283,13 +285,17 @@ class Encoder_length : public Encoder_base {
             etChk(et_OTF_attention_varlen(buffers[3], buffers[0], buffers[1], buffers[2], mask_ptr(),
                                           d_cu.get(), seq_len, d_model, nheads, batch, log2_scale, stream));
             O_linear.run_rows_ln(buffers[0], buffers[3], in_p, ln_gamma[0].get(), ln_beta[0].get(), n, stream);
-            MLP1_linear.run_rows(buffers[1], buffers[0], n, stream);
-            if (MLP2_linear.ln_fusable()) {
+            if (Linear_tile::ffn_fusable(MLP1_linear, MLP2_linear) && MLP2_linear.ln_fusable()) {
                 // in place over the skip operand: a workgroup reads its rows of
-                // unit 0 before it writes them
+                // unit 0 before it writes them (fused or not, see run_rows_ln)
+                Linear_tile::run_rows_ffn_ln(MLP1_linear, MLP2_linear, buffers[0], buffers[0], buffers[1],
+                                             buffers[0], ln_gamma[1].get(), ln_beta[1].get(), n, stream);
+            } else if (MLP2_linear.ln_fusable()) {
+                MLP1_linear.run_rows(buffers[1], buffers[0], n, stream);
                 MLP2_linear.run_rows_ln(buffers[0], buffers[1], buffers[0], ln_gamma[1].get(),
                                         ln_beta[1].get(), n, stream);
             } else {
+                MLP1_linear.run_rows(buffers[1], buffers[0], n, stream);
                 MLP2_linear.run_rows(out, buffers[1], n, stream);
                 etChk(et_skip_layernorm(buffers[0], out, ln_gamma[1].get(), ln_beta[1].get(), n, d_model, stream));
             }

@@ -175,6 +175,23 @@ int et_tile_plan_run_ln(const et_tile_plan *plan, void *Y, const void *X,
                         const void *skip, const void *gamma, const void *beta,
                         int M, void *stream);
 int et_tile_plan_ln_fusable(const et_tile_plan *plan);
+/* The feed-forward block of a layer, encoder/encoder.cu:36-44 (MLP1_linear
+ * with GELU, MLP2_linear, skip_layernorm_kernelLauncher), in ONE launch:
+ *   Y = LayerNorm(half(gelu(X W1^T + b1) W2^T + b2) + skip) * gamma + beta.
+ * The hidden activations are rounded to half exactly as the reference stores
+ * them, but stay in LDS: a workgroup walks the hidden dimension in chunks and
+ * feeds every chunk straight into the second linear.  Needs
+ * et_tile_plan_ffn_fusable(first, second): in_feat of the first <= 992, hidden
+ * chunks and out_feat of the second <= 768 columns.  `hidden` is a device
+ * buffer of M x hidden-width halves for the cases where the fused kernel does
+ * not apply or does not pay (few rows): then the launches run one after the
+ * other through it.  It may be NULL, which forces the fused kernel and fails
+ * with ET_ERR_UNSUPPORTED where that does not apply.  Y may alias skip (and
+ * skip may be X, the usual residual) only when the fused kernel runs. */
+int et_tile_plan_run_ffn_ln(const et_tile_plan *first, const et_tile_plan *second,
+                            void *Y, const void *X, void *hidden, const void *skip,
+                            const void *gamma, const void *beta, int M, void *stream);
+int et_tile_plan_ffn_fusable(const et_tile_plan *first, const et_tile_plan *second);
 /* n (<= 4) planned linears with the same in_feat applied to the same X in ONE
  * launch (the Q/K/V projections, encoder/encoder.cu:22-26, which the
  * reference spreads over three streams). */
@@ -289,6 +306,8 @@ int et_device_synchronize(void);
  *                     as two launches; 1 (default): fused where the rows fit
  *   "tile_ln_min_panels" fewest 32-row panels for which et_tile_plan_run_ln
  *                     fuses (default 96; below, two launches are faster)
+ *   "tile_fuse_ffn"   0: et_tile_plan_ffn_fusable answers no (the feed-forward
+ *                     block runs as separate launches); 1 (default)
  *   "tile_ln_chunked" 0: fused LayerNorm with K > 992 uses the single-buffer
  *                     kernel; 1 (default): the double-buffered one
  *   "ln_rows"         rows per wave of et_skip_layernorm (1, 2, 4)

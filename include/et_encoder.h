@@ -36,6 +36,14 @@ int et_linear_tile_run_rows(const et_linear_tile *h, void *out, const void *in, 
  * (et_tile_plan_run_ln): out = LayerNorm(half(linear(in)) + skip) */
 int et_linear_tile_run_rows_ln(const et_linear_tile *h, void *out, const void *in, const void *skip,
                                const void *gamma, const void *beta, int rows, void *stream);
+/* the feed-forward block (encoder/encoder.cu:36-44: MLP1 with GELU, MLP2,
+ * skip + LayerNorm) in one launch (et_tile_plan_run_ffn_ln); `hidden`
+ * ([rows x first.out_feat] halves, may be NULL to insist on the fused kernel)
+ * is used only where that kernel does not apply */
+int et_linear_tile_run_rows_ffn_ln(const et_linear_tile *first, const et_linear_tile *second, void *out,
+                                   const void *in, void *hidden, const void *skip, const void *gamma,
+                                   const void *beta, int rows, void *stream);
+int et_linear_tile_ffn_fusable(const et_linear_tile *first, const et_linear_tile *second);
 /* n <= 4 linears over one input in one launch (Q/K/V, encoder/encoder.cu:22-26) */
 int et_linear_tile_run_multi(const et_linear_tile *const *hs, void *const *outs, int n,
                              const void *in, int rows, void *stream);

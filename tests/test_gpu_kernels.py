@@ -159,6 +159,55 @@ def test_tile_linear_fused_skip_layernorm(K, M, N, Kd, sp):
         assert np.array_equal(host(sk), got)
 
 
+FFN_CASES = [
+    # M, d (in = out), hidden, sparsity, fused kernel expected
+    (128, 768, 3072, 0.8, True),    # BERT-base block: four hidden chunks of 768
+    (100, 768, 3072, 0.5, True),    # ragged M, denser
+    (70, 256, 1024, 0.6, True),     # two chunks, narrow rows: most waves own nothing in the second linear
+    (33, 512, 768, 0.7, True),      # hidden width in ONE chunk
+    (40, 768, 1536 + 256, 0.8, True),  # last hidden chunk partial (256 of 768 columns)
+    (64, 64, 3072, 0.9, True),      # tiny model width, many empty block-rows
+    (50, 768, 896, 0.8, False),     # one hidden chunk of 896 columns: too wide for the fused kernel
+    (36, 1024, 2048, 0.8, False),   # model width beyond one LDS panel
+]
+
+
+@pytest.mark.parametrize("M,d,F,sp,fused", FFN_CASES)
+def test_tile_ffn_fused_gelu_linear_layernorm(K, M, d, F, sp, fused):
+    """Linear_tile.run_ffn_ln == skip_layernorm(tile_linear(gelu(tile_linear(x))), skip) of the oracle"""
+    from et_amd.encoder import Linear_tile
+    r = rng(1700 + M + d)
+    l1 = make_tile_linear(r, F, d, sp, seed=5 * M + F, std=0.05, bias_std=0.2)
+    l2 = make_tile_linear(r, d, F, sp, seed=7 * M + d, std=0.05, bias_std=0.2)
+    X = randn_h(r, (M, d))
+    g, b = randn_h(r, (d,), 0.3) + np.float16(1), randn_h(r, (d,), 0.3)
+    h = orc.tile_linear(X, l1["row_ptr"], l1["row_offset"], l1["data"], l1["bias"], F, gelu=True)
+    y = orc.tile_linear(h, l2["row_ptr"], l2["row_offset"], l2["data"], l2["bias"], d)
+    want = orc.skip_layernorm(y, X, g, b)
+    t1 = Linear_tile(d, F, M, l1["row_offset"].size, l1["data"], l1["row_ptr"], l1["row_offset"], l1["bias"], True)
+    t2 = Linear_tile(F, d, M, l2["row_offset"].size, l2["data"], l2["row_ptr"], l2["row_offset"], l2["bias"], False)
+    assert Linear_tile.ffn_fusable(t1, t2) == fused
+    xd = dev(X)
+    if fused:
+        got = host(Linear_tile.run_ffn_ln(t1, t2, xd, xd, dev(g), dev(b)))  # no hidden buffer: fused or error
+    else:
+        with pytest.raises(Exception):
+            Linear_tile.run_ffn_ln(t1, t2, xd, xd, dev(g), dev(b))
+        hid = torch.empty((M, F), dtype=torch.float16, device="cuda")
+        got = host(Linear_tile.run_ffn_ln(t1, t2, xd, xd, dev(g), dev(b), hidden=hid))
+    check_close(got, want, what="fused feed-forward vs oracle chain")
+    # against the separate launches of this library: the hidden activations are
+    # rounded to half at the same point, so only fp32 summation order differs
+    hid = t1.run(xd)
+    sep = host(t2.run_ln(hid, xd, dev(g), dev(b)))
+    assert np.abs(got.astype(np.float32) - sep.astype(np.float32)).max() <= 2.0 ** -6
+    assert (got != sep).mean() < 0.03
+    if fused:  # in place over the input, which is also the skip operand
+        xd2 = dev(X)
+        Linear_tile.run_ffn_ln(t1, t2, xd2, xd2, dev(g), dev(b), out=xd2)
+        assert np.array_equal(host(xd2), got)
+
+
 def test_tile_linear_closed_form_reference_smoke_inputs(K):
     """weights = bias = 0.1 (test/gen_linear.cu:8,10): Y = 0.1*sum_{kept k} X + 0.1"""
     r = rng(12)
