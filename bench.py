@@ -144,9 +144,18 @@ def main():
         # the feed-forward block in one launch: X in, Y out, both weights once; the hidden activations stay in LDS
         ("feed-forward 768->3072->768 (gelu) + skip + LayerNorm, fused", lambda: Linear_tile.run_ffn_ln(L[4], L[5], b[0], b[0], gam[2], gam[3], out=y),
          tile_flops(T, nt[4]) + tile_flops(T, nt[5]),
-         tile_bytes(T, DFF, D, nt[4]) + tile_bytes(T, D, DFF, nt[5]) - 2 * 2 * T * DFF + 4 * D, "hbm"),
+         tile_bytes(T, DFF, D, nt[4]) + tile_bytes(T, D, DFF, nt[5]) - 2 * 2 * T * DFF + 4 * D, "mfma"),
     ]
-    if not Linear_tile.ffn_fusable(L[4], L[5]):  # (tuning override): the two launches through a hidden buffer
+    if Linear_tile.tail_fusable(L[3], L[4], L[5]):
+        # steps 6-10 in one launch: attention output and layer input in, Y out, three weights once
+        steps_def[-2:] = [
+            ("layer tail: o + skip + LayerNorm + feed-forward (gelu) + skip + LayerNorm, fused",
+             lambda: Linear_tile.run_tail(L[3], L[4], L[5], b[3], x, gam[0], gam[1], gam[2], gam[3], out=y),
+             tile_flops(T, nt[3]) + tile_flops(T, nt[4]) + tile_flops(T, nt[5]),
+             tile_bytes(T, D, D, nt[3]) + 2 * T * D + tile_bytes(T, DFF, D, nt[4]) + tile_bytes(T, D, DFF, nt[5])
+             - 2 * 2 * T * DFF - 2 * 2 * T * D + 8 * D, "mfma"),
+        ]
+    elif not Linear_tile.ffn_fusable(L[4], L[5]):  # (tuning override): the two launches through a hidden buffer
         steps_def[-1:] = [
             ("tile_linear ffn1+gelu (768->3072)", lambda: L[4].run(b[0], out=ffn), tile_flops(T, nt[4]), tile_bytes(T, DFF, D, nt[4]), "hbm"),
             ("tile_linear ffn2 (3072->768) + skip + LayerNorm", lambda: L[5].run_ln(ffn, b[0], gam[2], gam[3], out=y),

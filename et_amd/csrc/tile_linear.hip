@@ -79,6 +79,7 @@ struct TlArgs {
     int ipw; // plan kernel: consecutive work items per (persistent) workgroup
     // fused skip + LayerNorm epilogue (plan kernels with LN = true)
     const f16 *skip, *gamma, *beta;
+    const f16 *gamma2, *beta2; // second LayerNorm of the fused layer tail
 };
 #define TL_SEL(f) (lin == 0 ? a.f[0] : lin == 1 ? a.f[1] : lin == 2 ? a.f[2] : a.f[3])
 
@@ -365,9 +366,12 @@ struct TlLnOperands {
     f16x8 skip[ROWS][NCH], gamma[NCH], beta[NCH];
 };
 
+// (skip0 / Y0 point at the panel's first row, in global memory or in LDS, with
+// row pitches ldskip / ldy in halves)
 template <int NB, int NW, int NLW>
-__device__ __forceinline__ void tl_ln_fetch(TlLnOperands<NB, NW, NLW> &op, const TlArgs &a, int wave,
-                                            int lane, int m0, int N) {
+__device__ __forceinline__ void tl_ln_fetch_at(TlLnOperands<NB, NW, NLW> &op, int M, int wave, int lane,
+                                               int m0, int N, const f16 *skip0, long ldskip,
+                                               const f16 *gamma, const f16 *beta) {
     constexpr int NCH = TlLnOperands<NB, NW, NLW>::NCH;
     constexpr int ROWS = TlLnOperands<NB, NW, NLW>::ROWS;
     const int npiece = N >> 3;
@@ -376,17 +380,35 @@ __device__ __forceinline__ void tl_ln_fetch(TlLnOperands<NB, NW, NLW> &op, const
         const int ch = min(lane + 64 * i, npiece - 1); // (clamped pieces are never used)
 #pragma unroll
         for (int k = 0; k < ROWS; k++) {
-            const long row = min((long)m0 + wave + k * NLW, (long)a.M - 1);
-            op.skip[k][i] = *reinterpret_cast<const f16x8 *>(a.skip + row * N + ch * 8);
+            const long r = min((long)wave + k * NLW, (long)M - 1 - m0);
+            op.skip[k][i] = *reinterpret_cast<const f16x8 *>(skip0 + r * ldskip + ch * 8);
         }
-        op.gamma[i] = *reinterpret_cast<const f16x8 *>(a.gamma + ch * 8);
-        op.beta[i] = *reinterpret_cast<const f16x8 *>(a.beta + ch * 8);
+        op.gamma[i] = *reinterpret_cast<const f16x8 *>(gamma + ch * 8);
+        op.beta[i] = *reinterpret_cast<const f16x8 *>(beta + ch * 8);
     }
 }
 
 template <int NB, int NW, int NLW>
+__device__ __forceinline__ void tl_ln_fetch(TlLnOperands<NB, NW, NLW> &op, const TlArgs &a, int wave,
+                                            int lane, int m0, int N) {
+    tl_ln_fetch_at(op, a.M, wave, lane, m0, N, a.skip + (long)m0 * N, (long)N, a.gamma, a.beta);
+}
+
+template <int NB, int NW, int NLW>
+__device__ __forceinline__ void tl_ln_rows_at(const TlLnOperands<NB, NW, NLW> &op, int M,
+                                              const f16 *stage0, int wave, int lane, int m0, int N,
+                                              f16 *Y0, long ldy);
+
+template <int NB, int NW, int NLW>
 __device__ __forceinline__ void tl_ln_rows(const TlLnOperands<NB, NW, NLW> &op, const TlArgs &a,
                                            const f16 *stage0, int wave, int lane, int m0, f16 *Y, int N) {
+    tl_ln_rows_at(op, a.M, stage0, wave, lane, m0, N, Y + (long)m0 * N, (long)N);
+}
+
+template <int NB, int NW, int NLW>
+__device__ __forceinline__ void tl_ln_rows_at(const TlLnOperands<NB, NW, NLW> &op, int M,
+                                              const f16 *stage0, int wave, int lane, int m0, int N,
+                                              f16 *Y0, long ldy) {
     constexpr int lds = 16 * NB + 8;
     constexpr int NCH = TlLnOperands<NB, NW, NLW>::NCH;
     constexpr int ROWS = TlLnOperands<NB, NW, NLW>::ROWS;
@@ -395,8 +417,7 @@ __device__ __forceinline__ void tl_ln_rows(const TlLnOperands<NB, NW, NLW> &op, 
 #pragma unroll
     for (int k = 0; k < ROWS; k++) {
         const int r = wave + k * NLW;
-        const long row = (long)m0 + r;
-        if (r >= TL_BM || row >= a.M)
+        if (r >= TL_BM || m0 + r >= M)
             break;
         f16x8 xv[NCH];
         float sum = 0.f;
@@ -435,7 +456,7 @@ __device__ __forceinline__ void tl_ln_rows(const TlLnOperands<NB, NW, NLW> &op, 
                 for (int j = 0; j < 8; j++)
                     o[j] = (f16)(((float)xv[i][j] - mean) * rstd * (float)op.gamma[i][j] +
                                  (float)op.beta[i][j]);
-                *reinterpret_cast<f16x8 *>(Y + row * N + ch * 8) = o;
+                *reinterpret_cast<f16x8 *>(Y0 + r * ldy + ch * 8) = o;
             }
         }
     }
@@ -1095,8 +1116,9 @@ __device__ __forceinline__ void tl_wait_count(unsigned *ctr, unsigned target) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-template <int NB>
+template <int NB, bool WITH_O>
 __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const TlArgs a) {
+    constexpr int L1 = WITH_O ? 1 : 0, L2 = L1 + 1; // the two feed-forward linears
     extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
     f16 *xs = reinterpret_cast<f16 *>(tl_smem);
     const int rp = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3);
@@ -1125,7 +1147,7 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
     // event counters behind the hidden buffers: [p] first linear of phase p
     // done, [TL_FFN_MAX_PHASES + p] second linear of phase p done
     unsigned *const ctr = reinterpret_cast<unsigned *>(hs + 2 * hbuf);
-    const int N1 = a.N[0], N2 = a.N[1], nbr1 = N1 >> 4, nbr2 = N2 >> 4;
+    const int N1 = a.N[L1], N2 = a.N[L2], nbr1 = N1 >> 4, nbr2 = N2 >> 4;
     const int hbr = a.KC >> 4; // hidden block-rows per phase
     const unsigned lane_w = hi * 256 + c16 * 16 + x.khalf8;
 
@@ -1146,9 +1168,9 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
     }
     if (threadIdx.x < 2 * TL_FFN_MAX_PHASES)
         ctr[threadIdx.x] = 0;
-    const int *const cptr1 = a.cptr[0], *const cptr2 = a.cptr[1];
-    const f16 *const data1 = a.data[0], *const data2 = a.data[1];
-    const int *const poff1 = a.row_offset[0], *const poff2 = a.row_offset[1];
+    const int *const cptr1 = a.cptr[L1], *const cptr2 = a.cptr[L2];
+    const f16 *const data1 = a.data[L1], *const data2 = a.data[L2];
+    const int *const poff1 = a.row_offset[L1], *const poff2 = a.row_offset[L2];
     // pair-index boundaries of the wave's block-rows (lane j: start of block-row
     // j, lane NB: end of the last one); block-rows past the phase's range or the
     // matrix are empty
@@ -1169,7 +1191,7 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
 #define TL_FFN_BIAS1(dst_, p_)                                                                    \
     _Pragma("unroll") for (int k = 0; k < NB; k++)                                                \
         dst_[k] = *reinterpret_cast<const f16x4 *>(                                               \
-            a.bias[0] + min((p_) * hbr + wave * NB + k, nbr1 - 1) * 16 + g4 * 4);
+            a.bias[L1] + min((p_) * hbr + wave * NB + k, nbr1 - 1) * 16 + g4 * 4);
     f32x4 acc[NB][2];
     f16x4 b2[NB];
 #pragma unroll
@@ -1178,7 +1200,7 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
         acc[j][1] = f32x4{0.f, 0.f, 0.f, 0.f};
         b2[j] = f16x4{0, 0, 0, 0};
         if (x.bn0 + j < nbr2)
-            b2[j] = *reinterpret_cast<const f16x4 *>(a.bias[1] + (x.bn0 + j) * 16 + g4 * 4);
+            b2[j] = *reinterpret_cast<const f16x4 *>(a.bias[L2] + (x.bn0 + j) * 16 + g4 * 4);
     }
     const char *const xlane1 = reinterpret_cast<const char *>(xs + c16 * ldx + x.khalf8);
     const int xrow1 = 16 * ldx * 2, xrow2 = 16 * ldh * 2;
@@ -1225,8 +1247,46 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
     TL_FFN_BIAS1(b1n, min(1, a.nchunk - 1))
     int bvecS = TL_FFN_BVEC2(0);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's part of the panel has landed
-    TL_FFN_PRELOAD(data1, poff1, bvecF, wA, oA)
-    tl_barrier_lds(); // ... and everyone else's; the counters are zero
+    if constexpr (WITH_O) {
+        // Linear 0 (the attention output projection) with its skip connection
+        // and LayerNorm comes first: the panel just fetched holds the attention
+        // output, and the normalised rows (rounded to half, as the reference
+        // stores them) replace it in LDS as the feed-forward block's input and
+        // as the skip operand of the final LayerNorm.
+        const int NO = a.N[0], nbrO = NO >> 4; // == K
+        const int bvecO = bvec_of((ScalarInts)a.cptr[0], wave * NB, nbrO);
+        f16x4 bO[NB];
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            bO[j] = f16x4{0, 0, 0, 0};
+            if (x.bn0 + j < nbrO)
+                bO[j] = *reinterpret_cast<const f16x4 *>(a.bias[0] + (x.bn0 + j) * 16 + g4 * 4);
+        }
+        TL_FFN_PRELOAD(a.data[0], a.row_offset[0], bvecO, wB, oB)
+        TlLnOperands<NB, NW, NW> lnop1;
+        tl_ln_fetch_at(lnop1, a.M, wave, lane, x.m0, NO, a.skip + (long)x.m0 * NO, (long)NO, a.gamma, a.beta);
+        tl_barrier_lds(); // the whole panel has landed; the counters are zero
+        {
+            const int q0_ = __builtin_amdgcn_readfirstlane(bvecO), qe_ = __builtin_amdgcn_readlane(bvecO, NB);
+            tl_stream<NB>(xlane1, xrow1, a.data[0], a.row_offset[0], lane_w, hi, q0_, qe_, max(qe_ - 1, q0_),
+                          bvecO, wB, oB,
+                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); });
+        }
+        TL_FFN_PRELOAD(data1, poff1, bvecF, wA, oA)
+        // staging tiles in the hidden buffers, which nobody uses yet
+        tl_epilogue_wave<NB, false, false>(a, x, hs + wave * tl_wave_stage_halves<NB>(), nullptr, NO, nbrO, acc,
+                                           bO);
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            acc[j][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+            acc[j][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        tl_barrier_lds(); // every wave's part is staged, and everyone has left the attention panel
+        tl_ln_rows_at(lnop1, a.M, hs, wave, lane, x.m0, NO, xs, (long)ldx);
+    } else {
+        TL_FFN_PRELOAD(data1, poff1, bvecF, wA, oA)
+    }
+    tl_barrier_lds(); // the feed-forward input panel is complete (and the counters are zero)
     if (a.nchunk > 1)
         TL_FFN_PRELOAD(data1, poff1, bvecFn, wB, oB)
     TL_FFN_FIRST(0, bvecF, b1, wA, oA)
@@ -1269,13 +1329,16 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
     // output rows -> staging tiles over the (now unused) panel and hidden
     // buffers, then skip connection + LayerNorm over whole rows
     TlLnOperands<NB, NW, NW> lnop;
-    tl_ln_fetch(lnop, a, wave, lane, x.m0, N2);
+    if constexpr (WITH_O) // the skip operand is the panel in LDS
+        tl_ln_fetch_at(lnop, a.M, wave, lane, x.m0, N2, xs, (long)ldx, a.gamma2, a.beta2);
+    else
+        tl_ln_fetch(lnop, a, wave, lane, x.m0, N2);
     tl_barrier_lds(); // every wave has left the hidden buffers
-    f16 *const stage0 = xs;
-    tl_epilogue_wave<NB, false, false>(a, x, stage0 + wave * tl_wave_stage_halves<NB>(), a.Y[1], N2, nbr2,
+    f16 *const stage0 = WITH_O ? hs : xs;
+    tl_epilogue_wave<NB, false, false>(a, x, stage0 + wave * tl_wave_stage_halves<NB>(), a.Y[L2], N2, nbr2,
                                        acc, b2);
     __syncthreads(); // every wave's part of the rows is staged
-    tl_ln_rows(lnop, a, stage0, wave, lane, x.m0, a.Y[1], N2);
+    tl_ln_rows(lnop, a, stage0, wave, lane, x.m0, a.Y[L2], N2);
 }
 
 // ---------------------------------------------------------------------------
@@ -1451,7 +1514,7 @@ static int launch_chunked_ln_inst(const TlArgs &a, size_t lds, hipStream_t st) {
 }
 
 static int g_tile_ln_chunked = 1;
-static int g_tile_fuse_ffn = 1; // et_tuning_set("tile_fuse_ffn")
+static int g_tile_fuse_ffn = 2; // et_tuning_set("tile_fuse_ffn"): 1 feed-forward block, 2 whole layer tail
 
 // LDS bytes of the fused feed-forward kernel: X panel, two hidden buffers (the
 // output staging tiles reuse their storage)
@@ -1462,13 +1525,16 @@ static size_t ffn_lds_bytes(int K1, int KC2) {
     return std::max(panels, staging);
 }
 
-static int tile_launch_ffn(const TlProblem &p1, const TlProblem &p2, const f16 *X, int M, int K1,
-                           int KC2, int nchunk2, const f16 *skip, const f16 *gamma, const f16 *beta,
-                           hipStream_t st) {
+// pO: the attention output projection in front of the block (the whole layer
+// tail in one launch), or null
+static int tile_launch_ffn(const TlProblem *pO, const TlProblem &p1, const TlProblem &p2, const f16 *X,
+                           int M, int K1, int KC2, int nchunk2, const f16 *skip, const f16 *gamma,
+                           const f16 *beta, const f16 *gamma2, const f16 *beta2, hipStream_t st) {
     TlArgs a;
     memset(&a, 0, sizeof(a));
+    const TlProblem *ps[3] = {pO ? pO : &p1, pO ? &p1 : &p2, &p2};
     for (int i = 0; i < TL_MAX_LIN; i++) {
-        const TlProblem &p = i == 0 ? p1 : p2;
+        const TlProblem &p = *ps[std::min(i, 2)];
         a.Y[i] = p.Y;
         a.cptr[i] = p.cptr;
         a.row_offset[i] = p.row_offset;
@@ -1477,7 +1543,9 @@ static int tile_launch_ffn(const TlProblem &p1, const TlProblem &p2, const f16 *
         a.N[i] = p.N;
     }
     a.X = X;
-    a.nlin = 2;
+    a.nlin = pO ? 3 : 2;
+    a.gamma2 = gamma2;
+    a.beta2 = beta2;
     a.M = M;
     a.K = K1;
     a.KC = KC2;
@@ -1490,10 +1558,17 @@ static int tile_launch_ffn(const TlProblem &p1, const TlProblem &p2, const f16 *
     a.gamma = gamma;
     a.beta = beta;
     const size_t lds = ffn_lds_bytes(K1, KC2);
-    auto k = tile_ffn_fused_kernel<3>;
-    ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_FFN_WAVES * 64), lds, st, a);
+    if (pO) {
+        auto k = tile_ffn_fused_kernel<3, true>;
+        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_FFN_WAVES * 64), lds, st, a);
+    } else {
+        auto k = tile_ffn_fused_kernel<3, false>;
+        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_FFN_WAVES * 64), lds, st, a);
+    }
     return launch_status("fused feed-forward launch");
 }
 
@@ -2016,9 +2091,72 @@ extern "C" int et_tile_plan_run_ffn_ln(const et_tile_plan *p1, const et_tile_pla
     b.bias = p2->d_bias;
     b.N = p2->out_feat;
     b.nbr = p2->out_feat / 16;
-    return tile_launch_ffn(a, b, static_cast<const f16 *>(X), M, p1->in_feat, p2->KC, p2->nchunk,
+    return tile_launch_ffn(nullptr, a, b, static_cast<const f16 *>(X), M, p1->in_feat, p2->KC, p2->nchunk,
                            static_cast<const f16 *>(skip), static_cast<const f16 *>(gamma),
-                           static_cast<const f16 *>(beta), static_cast<hipStream_t>(stream));
+                           static_cast<const f16 *>(beta), nullptr, nullptr,
+                           static_cast<hipStream_t>(stream));
+}
+
+extern "C" int et_tile_plan_tail_fusable(const et_tile_plan *pO, const et_tile_plan *p1,
+                                         const et_tile_plan *p2) {
+    return pO && et_tile_plan_ffn_fusable(p1, p2) && pO->nchunk == 1 && pO->in_feat == pO->out_feat &&
+                   pO->out_feat == p1->in_feat && p2->out_feat == p1->in_feat &&
+                   pO->out_feat / 16 <= et::TL_FFN_WAVES * 3 && et::g_tile_fuse_ffn >= 2
+               ? 1
+               : 0;
+}
+
+extern "C" int et_tile_plan_run_tail(const et_tile_plan *pO, const et_tile_plan *p1,
+                                     const et_tile_plan *p2, void *Y, const void *attn, const void *input,
+                                     void *mid, void *hidden, const void *gamma1, const void *beta1,
+                                     const void *gamma2, const void *beta2, int M, void *stream) {
+    using namespace et;
+    ET_REQUIRE(pO && p1 && p2 && Y && attn && input && gamma1 && beta1 && gamma2 && beta2,
+               ET_ERR_INVALID_ARG, "et_tile_plan_run_tail: null pointer");
+    ET_REQUIRE(M >= 0, ET_ERR_INVALID_ARG, "et_tile_plan_run_tail: M=%d", M);
+    ET_REQUIRE(pO->out_feat == p1->in_feat && p2->in_feat == p1->out_feat && p2->out_feat == p1->in_feat,
+               ET_ERR_INVALID_ARG, "et_tile_plan_run_tail: the three linears do not chain (%d->%d, %d->%d, %d->%d)",
+               pO->in_feat, pO->out_feat, p1->in_feat, p1->out_feat, p2->in_feat, p2->out_feat);
+    ET_REQUIRE(aligned16(Y) && aligned16(attn) && aligned16(input) && aligned16(mid) && aligned16(hidden) &&
+                   aligned16(gamma1) && aligned16(beta1) && aligned16(gamma2) && aligned16(beta2),
+               ET_ERR_ALIGNMENT, "et_tile_plan_run_tail: pointers must be 16-byte aligned");
+    if (M == 0)
+        return ET_OK;
+    if (!et_tile_plan_tail_fusable(pO, p1, p2) || (mid && !ln_fusion_pays(M))) {
+        // step by step through the caller's buffers
+        ET_REQUIRE(mid, ET_ERR_UNSUPPORTED,
+                   "et_tile_plan_run_tail: these shapes need the mid buffer (%d x %d halves)", M, pO->out_feat);
+        const int rc = et_tile_plan_run_ln(pO, mid, attn, input, gamma1, beta1, M, stream);
+        if (rc != ET_OK)
+            return rc;
+        return et_tile_plan_run_ffn_ln(p1, p2, Y, mid, hidden, mid, gamma2, beta2, M, stream);
+    }
+    TlProblem o, a, b;
+    o.Y = nullptr;
+    o.cptr = pO->d_cptr;
+    o.row_offset = pO->d_row_offset;
+    o.data = pO->d_data;
+    o.bias = pO->d_bias;
+    o.N = pO->out_feat;
+    o.nbr = pO->out_feat / 16;
+    a.Y = nullptr;
+    a.cptr = p1->d_cptr;
+    a.row_offset = p1->d_row_offset;
+    a.data = p1->d_data;
+    a.bias = p1->d_bias;
+    a.N = p1->out_feat;
+    a.nbr = p1->out_feat / 16;
+    b.Y = static_cast<f16 *>(Y);
+    b.cptr = p2->d_cptr;
+    b.row_offset = p2->d_row_offset;
+    b.data = p2->d_data;
+    b.bias = p2->d_bias;
+    b.N = p2->out_feat;
+    b.nbr = p2->out_feat / 16;
+    return tile_launch_ffn(&o, a, b, static_cast<const f16 *>(attn), M, p1->in_feat, p2->KC, p2->nchunk,
+                           static_cast<const f16 *>(input), static_cast<const f16 *>(gamma1),
+                           static_cast<const f16 *>(beta1), static_cast<const f16 *>(gamma2),
+                           static_cast<const f16 *>(beta2), static_cast<hipStream_t>(stream));
 }
 
 extern "C" int et_tile_plan_run(const et_tile_plan *plan, void *Y, const void *X, int M, int gelu,

@@ -78,6 +78,23 @@ class Linear_tile:
     def ffn_fusable(first, second):
         return bool(lib().et_linear_tile_ffn_fusable(first._h, second._h))
 
+    @staticmethod
+    def run_tail(out_proj, first, second, attn, inp, gamma1, beta1, gamma2, beta2, out=None, mid=None,
+                 hidden=None, rows=None):
+        """Steps 6-10 of a layer in one launch: out projection + skip + LayerNorm, feed-forward block + skip +
+        LayerNorm.  `mid` / `hidden` are only used where the fused kernel does not apply; mid=None insists on it."""
+        rows = attn.shape[0] if rows is None else rows
+        out = out if out is not None else torch.empty((attn.shape[0], second.out_feat), dtype=torch.float16, device=attn.device)
+        opt = lambda t: _dp(t) if t is not None else None
+        check(lib().et_linear_tile_run_rows_tail(out_proj._h, first._h, second._h, _dp(out), _dp(attn), _dp(inp),
+                                                 opt(mid), opt(hidden), _dp(gamma1), _dp(beta1), _dp(gamma2),
+                                                 _dp(beta2), rows, _stream()))
+        return out
+
+    @staticmethod
+    def tail_fusable(out_proj, first, second):
+        return bool(lib().et_linear_tile_tail_fusable(out_proj._h, first._h, second._h))
+
     def _release(self):  # ownership moved into an encoder
         self._h = None
 

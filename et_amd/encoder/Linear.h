@@ -66,6 +66,22 @@ class Linear_tile {
         return et_tile_plan_ffn_fusable(first.plan, second.plan) != 0;
     }
 
+    // steps 6-10 of a layer (encoder/encoder.cu:33-44) in one launch; `mid`
+    // ([rows x model width]) and `hidden` are used only where the fused kernel
+    // does not apply or does not pay; see et_tile_plan_run_tail
+    static void run_rows_tail(const Linear_tile &out_proj, const Linear_tile &first, const Linear_tile &second,
+                              half *out, half *attn, const half *input, half *mid, half *hidden,
+                              const half *gamma1, const half *beta1, const half *gamma2, const half *beta2,
+                              int rows, void *stream) {
+        etRequire(!out_proj.is_gelu && first.is_gelu && !second.is_gelu,
+                  "Linear_tile::run_rows_tail: only the first feed-forward linear is the GELU variant");
+        etChk(et_tile_plan_run_tail(out_proj.plan, first.plan, second.plan, out, attn, input, mid, hidden,
+                                    gamma1, beta1, gamma2, beta2, rows, stream));
+    }
+    static bool tail_fusable(const Linear_tile &out_proj, const Linear_tile &first, const Linear_tile &second) {
+        return et_tile_plan_tail_fusable(out_proj.plan, first.plan, second.plan) != 0;
+    }
+
     static void run_multi(const Linear_tile *const *lin, half *const *outs, int n, half *in, int rows,
                           void *stream) {
         const et_tile_plan *plans[4];

@@ -99,12 +99,11 @@ class Encoder_base {
     // O projection, skip-LN with the layer input, FFN1+GELU, FFN2, skip-LN.
     void tail(half *out, half *in, half *attn, const Linear_tile &O, const Linear_tile &M1,
               const Linear_tile &M2, int nrows) {
-        // (the projection, its skip connection and LayerNorm are one launch, and
-        // so is the whole feed-forward block; its hidden buffer, units 1..4, is
-        // only touched where the fused kernel does not apply)
-        O.run_rows_ln(buffers[0], attn, in, ln_gamma[0].get(), ln_beta[0].get(), nrows, stream);
-        Linear_tile::run_rows_ffn_ln(M1, M2, out, buffers[0], buffers[1], buffers[0], ln_gamma[1].get(),
-                                     ln_beta[1].get(), nrows, stream);
+        // (all five steps are one launch; unit 0 for the first LayerNorm's rows
+        // and units 1..4 for the hidden activations are only touched where the
+        // fused kernel does not apply)
+        Linear_tile::run_rows_tail(O, M1, M2, out, attn, in, buffers[0], buffers[1], ln_gamma[0].get(),
+                                   ln_beta[0].get(), ln_gamma[1].get(), ln_beta[1].get(), nrows, stream);
     }
 };
 
@@ -284,6 +283,14 @@ class Encoder_length : public Encoder_base {
             Linear_tile::run_multi(qkv, outs, 3, in_p, n, stream);
             etChk(et_OTF_attention_varlen(buffers[3], buffers[0], buffers[1], buffers[2], mask_ptr(),
                                           d_cu.get(), seq_len, d_model, nheads, batch, log2_scale, stream));
+            if (Linear_tile::tail_fusable(O_linear, MLP1_linear, MLP2_linear)) {
+                // steps 6-10 in one launch, straight into unit 0
+                Linear_tile::run_rows_tail(O_linear, MLP1_linear, MLP2_linear, buffers[0], buffers[3], in_p,
+                                           nullptr, nullptr, ln_gamma[0].get(), ln_beta[0].get(),
+                                           ln_gamma[1].get(), ln_beta[1].get(), n, stream);
+                etChk(et_unpack_rows(out, buffers[0], d_cu.get(), batch, seq_len, d_model, stream));
+                return;
+            }
             O_linear.run_rows_ln(buffers[0], buffers[3], in_p, ln_gamma[0].get(), ln_beta[0].get(), n, stream);
             if (Linear_tile::ffn_fusable(MLP1_linear, MLP2_linear) && MLP2_linear.ln_fusable()) {
                 // in place over the skip operand: a workgroup reads its rows of

@@ -192,6 +192,26 @@ int et_tile_plan_run_ffn_ln(const et_tile_plan *first, const et_tile_plan *secon
                             void *Y, const void *X, void *hidden, const void *skip,
                             const void *gamma, const void *beta, int M, void *stream);
 int et_tile_plan_ffn_fusable(const et_tile_plan *first, const et_tile_plan *second);
+/* Steps 6-10 of a layer, encoder/encoder.cu:33-44 (O_linear, skip + LayerNorm
+ * with the layer input, MLP1 with GELU, MLP2, skip + LayerNorm), in ONE launch:
+ *   mid = LayerNorm(half(attn Wo^T + bo) + input) * gamma1 + beta1
+ *   Y   = LayerNorm(half(gelu(mid W1^T + b1) W2^T + b2) + mid) * gamma2 + beta2.
+ * The workgroup that owns a 32-row panel runs the projection first and keeps
+ * its normalised rows (rounded to half, as the reference stores them) in LDS
+ * as the feed-forward input and the second skip operand; mid never reaches
+ * memory.  Needs et_tile_plan_tail_fusable(out, first, second): a square
+ * projection of the model width on top of et_tile_plan_ffn_fusable.  `mid`
+ * (M x model width halves) and `hidden` (M x hidden width) are device buffers
+ * for the cases where the fused kernel does not apply or does not pay; with
+ * mid == NULL the fused kernel is forced (ET_ERR_UNSUPPORTED where it does not
+ * apply).  Y may alias attn or input when the fused kernel runs. */
+int et_tile_plan_run_tail(const et_tile_plan *out, const et_tile_plan *first,
+                          const et_tile_plan *second, void *Y, const void *attn,
+                          const void *input, void *mid, void *hidden,
+                          const void *gamma1, const void *beta1, const void *gamma2,
+                          const void *beta2, int M, void *stream);
+int et_tile_plan_tail_fusable(const et_tile_plan *out, const et_tile_plan *first,
+                              const et_tile_plan *second);
 /* n (<= 4) planned linears with the same in_feat applied to the same X in ONE
  * launch (the Q/K/V projections, encoder/encoder.cu:22-26, which the
  * reference spreads over three streams). */
@@ -307,7 +327,8 @@ int et_device_synchronize(void);
  *   "tile_ln_min_panels" fewest 32-row panels for which et_tile_plan_run_ln
  *                     fuses (default 96; below, two launches are faster)
  *   "tile_fuse_ffn"   0: et_tile_plan_ffn_fusable answers no (the feed-forward
- *                     block runs as separate launches); 1 (default)
+ *                     block runs as separate launches); 1: the block is fused
+ *                     but et_tile_plan_tail_fusable answers no; 2 (default)
  *   "tile_ln_chunked" 0: fused LayerNorm with K > 992 uses the single-buffer
  *                     kernel; 1 (default): the double-buffered one
  *   "ln_rows"         rows per wave of et_skip_layernorm (1, 2, 4)

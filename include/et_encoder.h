@@ -44,6 +44,16 @@ int et_linear_tile_run_rows_ffn_ln(const et_linear_tile *first, const et_linear_
                                    const void *in, void *hidden, const void *skip, const void *gamma,
                                    const void *beta, int rows, void *stream);
 int et_linear_tile_ffn_fusable(const et_linear_tile *first, const et_linear_tile *second);
+/* steps 6-10 of a layer (encoder/encoder.cu:33-44: O_linear, skip + LayerNorm,
+ * MLP1 with GELU, MLP2, skip + LayerNorm) in one launch (et_tile_plan_run_tail);
+ * `mid` ([rows x model width]) and `hidden` ([rows x first.out_feat]) are used
+ * only where the fused kernel does not apply; mid == NULL insists on it */
+int et_linear_tile_run_rows_tail(const et_linear_tile *out_proj, const et_linear_tile *first,
+                                 const et_linear_tile *second, void *out, const void *attn, const void *input,
+                                 void *mid, void *hidden, const void *gamma1, const void *beta1,
+                                 const void *gamma2, const void *beta2, int rows, void *stream);
+int et_linear_tile_tail_fusable(const et_linear_tile *out_proj, const et_linear_tile *first,
+                                const et_linear_tile *second);
 /* n <= 4 linears over one input in one launch (Q/K/V, encoder/encoder.cu:22-26) */
 int et_linear_tile_run_multi(const et_linear_tile *const *hs, void *const *outs, int n,
                              const void *in, int rows, void *stream);

@@ -208,6 +208,57 @@ def test_tile_ffn_fused_gelu_linear_layernorm(K, M, d, F, sp, fused):
         assert np.array_equal(host(xd2), got)
 
 
+TAIL_CASES = [
+    # M, d, hidden, sparsity, fused kernel expected
+    (128, 768, 3072, 0.8, True),   # BERT-base layer tail
+    (77, 768, 3072, 0.5, True),    # ragged M
+    (40, 256, 1024, 0.7, True),    # narrow rows: most waves own nothing in the projections
+    (64, 64, 1536, 0.9, True),     # many empty block-rows
+    (50, 768, 896, 0.8, False),    # hidden chunk too wide: step by step
+]
+
+
+@pytest.mark.parametrize("M,d,F,sp,fused", TAIL_CASES)
+def test_tile_layer_tail_fused(K, M, d, F, sp, fused):
+    """Linear_tile.run_tail == the oracle's O projection, skip+LN, FFN1+GELU, FFN2, skip+LN one after the other"""
+    from et_amd.encoder import Linear_tile
+    r = rng(2300 + M + d)
+    lo = make_tile_linear(r, d, d, sp, seed=3 * M + d, std=0.05, bias_std=0.2)
+    l1 = make_tile_linear(r, F, d, sp, seed=5 * M + F, std=0.05, bias_std=0.2)
+    l2 = make_tile_linear(r, d, F, sp, seed=7 * M + d, std=0.05, bias_std=0.2)
+    attn, inp = randn_h(r, (M, d)), randn_h(r, (M, d))
+    g1, b1 = randn_h(r, (d,), 0.3) + np.float16(1), randn_h(r, (d,), 0.3)
+    g2, b2 = randn_h(r, (d,), 0.3) + np.float16(1), randn_h(r, (d,), 0.3)
+    o = orc.tile_linear(attn, lo["row_ptr"], lo["row_offset"], lo["data"], lo["bias"], d)
+    mid = orc.skip_layernorm(o, inp, g1, b1)
+    h = orc.tile_linear(mid, l1["row_ptr"], l1["row_offset"], l1["data"], l1["bias"], F, gelu=True)
+    y = orc.tile_linear(h, l2["row_ptr"], l2["row_offset"], l2["data"], l2["bias"], d)
+    want = orc.skip_layernorm(y, mid, g2, b2)
+    mk = lambda l, K_, N_, gelu: Linear_tile(K_, N_, M, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], gelu)
+    to, t1, t2 = mk(lo, d, d, False), mk(l1, d, F, True), mk(l2, F, d, False)
+    assert Linear_tile.tail_fusable(to, t1, t2) == fused
+    ln = [dev(t) for t in (g1, b1, g2, b2)]
+    if fused:
+        got = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln))  # no buffers: fused or error
+    else:
+        with pytest.raises(Exception):
+            Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln)
+        midb = torch.empty((M, d), dtype=torch.float16, device="cuda")
+        hid = torch.empty((M, F), dtype=torch.float16, device="cuda")
+        got = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln, mid=midb, hidden=hid))
+    # two LayerNorms amplify half-ulp differences of the first one's output
+    check_close(got, want, max_abs=3e-2, mean_rel=2e-3, what="fused layer tail vs oracle chain")
+    # against this library's separate launches
+    midg = to.run_ln(dev(attn), dev(inp), ln[0], ln[1])
+    sep = host(t2.run_ln(t1.run(midg), midg, ln[2], ln[3]))
+    assert np.abs(got.astype(np.float32) - sep.astype(np.float32)).max() <= 3e-2
+    assert (got != sep).mean() < 0.05
+    if fused:  # the output may overwrite the attention buffer
+        ad = dev(attn)
+        Linear_tile.run_tail(to, t1, t2, ad, dev(inp), *ln, out=ad)
+        assert np.array_equal(host(ad), got)
+
+
 def test_tile_linear_closed_form_reference_smoke_inputs(K):
     """weights = bias = 0.1 (test/gen_linear.cu:8,10): Y = 0.1*sum_{kept k} X + 0.1"""
     r = rng(12)
