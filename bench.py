@@ -230,7 +230,7 @@ def main():
                    "batch": B, "seq_len": S, "d_model": D, "heads": H, "d_ff": DFF, "sparsity": args.sparsity,
                    "softmax_base": 2, "mask": "additive zeros"},
         "layer_GFLOP_surviving": round(layer_flops, 2),
-        "layer_mfma_frac": round(layer_flops / (ms_per_step * 1e3) / 1e3 / MFMA_F16_PEAK_TF, 4),
+        "layer_mfma_frac": round(layer_flops / (ms_per_step * 1e3) * 1e3 / MFMA_F16_PEAK_TF, 4),  # GFLOP/us = PFLOP/s
         "sum_kernel_us": round(total_us, 1),
         "parity_vs_oracle": {"max_abs": round(max_abs, 5), "mean_rel": round(mean_rel, 6), "rows": S},
         "roofline": roof, "kernels": kern, "cpu_baseline": cpu,

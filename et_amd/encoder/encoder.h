@@ -284,9 +284,12 @@ class Encoder_length : public Encoder_base {
             etChk(et_OTF_attention_varlen(buffers[3], buffers[0], buffers[1], buffers[2], mask_ptr(),
                                           d_cu.get(), seq_len, d_model, nheads, batch, log2_scale, stream));
             if (Linear_tile::tail_fusable(O_linear, MLP1_linear, MLP2_linear)) {
-                // steps 6-10 in one launch, straight into unit 0
+                // steps 6-10 in one launch, straight into unit 0.  (With few rows
+                // they run one after the other, in place in unit 0 with the hidden
+                // activations in units 1..4: the attention output and the packed
+                // input are no longer needed by then.)
                 Linear_tile::run_rows_tail(O_linear, MLP1_linear, MLP2_linear, buffers[0], buffers[3], in_p,
-                                           nullptr, nullptr, ln_gamma[0].get(), ln_beta[0].get(),
+                                           buffers[0], buffers[1], ln_gamma[0].get(), ln_beta[0].get(),
                                            ln_gamma[1].get(), ln_beta[1].get(), n, stream);
                 etChk(et_unpack_rows(out, buffers[0], d_cu.get(), batch, seq_len, d_model, stream));
                 return;
