@@ -246,20 +246,22 @@ __device__ __forceinline__ void tl_static_for(F &&f) {
 // One pair's operands: 16 bytes of W per lane and the lane's X offset.  The
 // pair's address is wave-uniform (scalar registers) and the lane's part a
 // 32-bit offset, so the loads need no vector address arithmetic.
-__device__ __forceinline__ void tl_load_pair_at(const char *wq, const char *oq, unsigned lane_w,
-                                                unsigned hi, f16x8 &w, int &o) {
-    // (the empty asm keeps the compiler from folding the lane offsets into
-    // loop-invariant 64-bit vector addresses, which costs two 64-bit vector
-    // adds per pair instead of none)
-    unsigned lo = hi * 4u, lw = lane_w * 2u;
+// lo / lw: the lane's byte offsets into a pair's two ints and its 1 KB of W
+__device__ __forceinline__ void tl_load_pair_at(const char *wq, const char *oq, unsigned &lo,
+                                                unsigned &lw, f16x8 &w, int &o) {
+    // (the empty asm, in place on variables that live across the whole stream,
+    // makes the lane offsets look freshly computed: otherwise the compiler folds
+    // them into loop-invariant 64-bit vector addresses and pays two 64-bit
+    // vector adds per pair instead of using scalar base + 32-bit lane offset)
     asm("" : "+v"(lo), "+v"(lw));
     o = *reinterpret_cast<const int *>(oq + lo);
     w = *reinterpret_cast<const f16x8 *>(wq + lw);
 }
 __device__ __forceinline__ void tl_load_pair(const f16 *data, const int *poff, int q, unsigned lane_w,
                                              unsigned hi, f16x8 &w, int &o) {
+    unsigned lo = hi * 4u, lw = lane_w * 2u;
     tl_load_pair_at(reinterpret_cast<const char *>(data) + (size_t)q * 1024,
-                    reinterpret_cast<const char *>(poff) + (size_t)q * 8, lane_w, hi, w, o);
+                    reinterpret_cast<const char *>(poff) + (size_t)q * 8, lo, lw, w, o);
 }
 
 __device__ __forceinline__ void tl_preload(const f16 *data, const int *poff, unsigned lane_w, unsigned hi,
@@ -269,15 +271,45 @@ __device__ __forceinline__ void tl_preload(const f16 *data, const int *poff, uns
         tl_load_pair(data, poff, min(q0 + i, qlast), lane_w, hi, w[i], o[i]);
 }
 
+#ifdef TL_STAGETRACE
+// profiling builds only: lane 0 of a traced wave stamps (cycle counter << 8 |
+// code) into an LDS buffer at every stage
+struct TlTracer {
+    unsigned long long *buf;
+    int n, cap;
+};
+__device__ unsigned long long *g_stage_trace = nullptr;
+__device__ __forceinline__ void tl_stamp(TlTracer &t, unsigned lane_w, unsigned code) {
+    if (t.buf && t.n < t.cap) {
+        if (lane_w == 0)
+            t.buf[t.n] = ((unsigned long long)__builtin_readcyclecounter() << 8) | code;
+        t.n++;
+    }
+}
+#define TL_STAMP(code_) tl_stamp(*trc_, lane_w, code_)
+#else
+#define TL_STAMP(code_)
+#endif
+
 // bvec: lane j holds the first pair of block-row j, lane NB the end of the
 // last one (read back with v_readlane)
 template <int NB, class Flush>
 __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f16 *data,
                                           const int *poff, unsigned lane_w, unsigned hi, int q0,
                                           int qend, int qlast, int bvec, f16x8 (&w)[TL_DEPTH],
-                                          int (&o)[TL_DEPTH], Flush &&flush) {
+                                          int (&o)[TL_DEPTH], Flush &&flush
+#ifdef TL_STAGETRACE
+                                          , TlTracer *trc_ = nullptr
+#endif
+) {
+#ifdef TL_STAGETRACE
+    TlTracer dummy_{nullptr, 0, 0};
+    if (!trc_)
+        trc_ = &dummy_;
+#endif
     if (q0 >= qend)
         return;
+    TL_STAMP(3);
     f32x4 cur0 = f32x4{0.f, 0.f, 0.f, 0.f}, cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
     int j = 0;
     int bend = __builtin_amdgcn_readlane(bvec, 1);
@@ -295,6 +327,7 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
     // constant, which goes into the load's immediate offset
     const char *wp = reinterpret_cast<const char *>(data) + (size_t)(q0 + TL_DEPTH) * 1024;
     const char *op = reinterpret_cast<const char *>(poff) + (size_t)(q0 + TL_DEPTH) * 8;
+    unsigned lane_lo = hi * 4u, lane_lw = lane_w * 2u;
     auto stage = [&](auto ic, auto always) {
         constexpr int I = decltype(ic)::value;
         constexpr int S = I % TL_DEPTH, SN = (I + 1) % TL_DEPTH, P = I & 1;
@@ -303,14 +336,16 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
         // keep the reads above the MFMAs: left alone, the scheduler sinks them
         // to the end of the stage and every stage then waits out the LDS latency
         __builtin_amdgcn_sched_barrier(0);
+        TL_STAMP(1);
         cur0 = mfma16x16x32(w[S], xa[P], cur0);
         cur1 = mfma16x16x32(w[S], xb[P], cur1);
         // pair q + I + TL_DEPTH; the last stages of a stream request nothing:
         // a request still in flight when the stream ends would make the next
         // use of these registers wait out a full memory latency
         if (decltype(always)::value || q + I + TL_DEPTH < qend)
-            tl_load_pair_at(wp + I * 1024, op + I * 8, lane_w, hi, w[S], o[S]);
+            tl_load_pair_at(wp + I * 1024, op + I * 8, lane_lo, lane_lw, w[S], o[S]);
         if (q + I + 1 == bend) { // block-row j is complete
+            TL_STAMP(2);
             flush(j, cur0, cur1);
             cur0 = f32x4{0.f, 0.f, 0.f, 0.f};
             cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -1147,6 +1182,15 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
     // event counters behind the hidden buffers: [p] first linear of phase p
     // done, [TL_FFN_MAX_PHASES + p] second linear of phase p done
     unsigned *const ctr = reinterpret_cast<unsigned *>(hs + 2 * hbuf);
+#ifdef TL_STAGETRACE
+    TlTracer trc{nullptr, 0, 192};
+    if (rp == 0 && x.wave < 8)
+        trc.buf = reinterpret_cast<unsigned long long *>(ctr + 2 * TL_FFN_MAX_PHASES) + x.wave * 192;
+    TlTracer *const trc_ = &trc;
+#define TL_TRC_ARG , &trc
+#else
+#define TL_TRC_ARG
+#endif
     const int N1 = a.N[L1], N2 = a.N[L2], nbr1 = N1 >> 4, nbr2 = N2 >> 4;
     const int hbr = a.KC >> 4; // hidden block-rows per phase
     const unsigned lane_w = hi * 256 + c16 * 16 + x.khalf8;
@@ -1216,8 +1260,8 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
                           f16x4 bj = f16x4{0, 0, 0, 0};                                           \
                           _Pragma("unroll") for (int k = 0; k < NB; k++)                          \
                               bj += b1_[k] * ((j == k) ? (f16)1 : (f16)0);                        \
-                          tl_stage_tile<true>(hlane + j * 16, ldh, c0, c1, bj);                   \
-                      });                                                                         \
+                          tl_stage_tile<true>(hlane + j * 16, ldh, c0, c1, bj);                          \
+                      } TL_TRC_ARG);                                                              \
         /* block-rows of this phase without any tile: bias only */                                \
         const int lim1 = min(((p_) + 1) * hbr, nbr1);                                             \
         _Pragma("unroll") for (int k = 0; k < NB; k++)                                            \
@@ -1270,7 +1314,7 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
             const int q0_ = __builtin_amdgcn_readfirstlane(bvecO), qe_ = __builtin_amdgcn_readlane(bvecO, NB);
             tl_stream<NB>(xlane1, xrow1, a.data[0], a.row_offset[0], lane_w, hi, q0_, qe_, max(qe_ - 1, q0_),
                           bvecO, wB, oB,
-                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); });
+                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); } TL_TRC_ARG);
         }
         TL_FFN_PRELOAD(data1, poff1, bvecF, wA, oA)
         // staging tiles in the hidden buffers, which nobody uses yet
@@ -1299,19 +1343,23 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
         TL_FFN_BIAS1(b1n2, min(p + 2, a.nchunk - 1))
         TL_FFN_PRELOAD(data2, poff2, bvecS, wA, oA) // S(p), a stream ahead
         if (p + 1 < a.nchunk) {
+            TL_STAMP(5);
             if (p >= 1) // F(p+1) overwrites the buffer that S(p-1) read
                 tl_wait_count(ctr + TL_FFN_MAX_PHASES + p - 1, NW);
+            TL_STAMP(6);
             TL_FFN_FIRST(p + 1, bvecFn, b1n, wB, oB)
         }
         if (p + 2 < a.nchunk)
             TL_FFN_PRELOAD(data1, poff1, bvecF2, wB, oB) // F(p+2), a stream ahead
+        TL_STAMP(7);
         tl_wait_count(ctr + p, NW); // hidden buffer p & 1 is complete
+        TL_STAMP(8);
         {
             const char *const xlane2 =
                 reinterpret_cast<const char *>(hs + (p & 1) * hbuf + c16 * ldh + x.khalf8);
             const int q0_ = __builtin_amdgcn_readfirstlane(bvecS), qe_ = __builtin_amdgcn_readlane(bvecS, NB);
             tl_stream<NB>(xlane2, xrow2, data2, poff2, lane_w, hi, q0_, qe_, max(qe_ - 1, q0_), bvecS, wA, oA,
-                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); });
+                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); } TL_TRC_ARG);
             tl_signal(ctr + TL_FFN_MAX_PHASES + p, lane);
         }
         bvecS = bvecSn;
@@ -1339,6 +1387,14 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
                                        acc, b2);
     __syncthreads(); // every wave's part of the rows is staged
     tl_ln_rows(lnop, a, stage0, wave, lane, x.m0, a.Y[L2], N2);
+#ifdef TL_STAGETRACE
+    TL_STAMP(9);
+    __syncthreads();
+    if (rp == 0 && g_stage_trace)
+        for (int i = threadIdx.x; i < 8 * 192; i += blockDim.x)
+            g_stage_trace[i] = reinterpret_cast<unsigned long long *>(ctr + 2 * TL_FFN_MAX_PHASES)[i];
+#endif
+#undef TL_TRC_ARG
 }
 
 // ---------------------------------------------------------------------------
@@ -1520,7 +1576,10 @@ static int g_tile_fuse_ffn = 2; // et_tuning_set("tile_fuse_ffn"): 1 feed-forwar
 // output staging tiles reuse their storage)
 static size_t ffn_lds_bytes(int K1, int KC2) {
     const size_t ldx = K1 + ((K1 & 31) ? 0 : TL_PAD), ldh = KC2 + ((KC2 & 31) ? 0 : TL_PAD);
-    const size_t panels = (size_t)TL_BM * (ldx + 2 * ldh) * sizeof(f16) + 2 * TL_FFN_MAX_PHASES * sizeof(unsigned);
+    size_t panels = (size_t)TL_BM * (ldx + 2 * ldh) * sizeof(f16) + 2 * TL_FFN_MAX_PHASES * sizeof(unsigned);
+#ifdef TL_STAGETRACE
+    panels += 8 * 192 * 8;
+#endif
     const size_t staging = (size_t)TL_FFN_WAVES * TL_BM * (16 * 3 + 8) * sizeof(f16);
     return std::max(panels, staging);
 }
@@ -2179,6 +2238,11 @@ extern "C" int et_tile_plan_run(const et_tile_plan *plan, void *Y, const void *X
                        plan->nchunk, gelu != 0, TL_PLAN, static_cast<hipStream_t>(stream));
 }
 
+#ifdef TL_STAGETRACE
+extern "C" int et_debug_stage_trace(void *buf) {
+    return hipMemcpyToSymbol(HIP_SYMBOL(et::g_stage_trace), &buf, sizeof(buf)) == hipSuccess ? 0 : -1;
+}
+#endif
 #ifdef TL_TRACE
 // profiling builds only: per-wave phase tick counters are written to `buf`
 // (8 x u64 per wave, indexed by hardware workgroup id)
