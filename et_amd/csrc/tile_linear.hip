@@ -1237,14 +1237,10 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
         dst_[k] = *reinterpret_cast<const f16x4 *>(                                               \
             a.bias[L1] + min((p_) * hbr + wave * NB + k, nbr1 - 1) * 16 + g4 * 4);
     f32x4 acc[NB][2];
-    f16x4 b2[NB];
 #pragma unroll
     for (int j = 0; j < NB; j++) {
         acc[j][0] = f32x4{0.f, 0.f, 0.f, 0.f};
         acc[j][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-        b2[j] = f16x4{0, 0, 0, 0};
-        if (x.bn0 + j < nbr2)
-            b2[j] = *reinterpret_cast<const f16x4 *>(a.bias[L2] + (x.bn0 + j) * 16 + g4 * 4);
     }
     const char *const xlane1 = reinterpret_cast<const char *>(xs + c16 * ldx + x.khalf8);
     const int xrow1 = 16 * ldx * 2, xrow2 = 16 * ldh * 2;
@@ -1260,7 +1256,7 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
                           f16x4 bj = f16x4{0, 0, 0, 0};                                           \
                           _Pragma("unroll") for (int k = 0; k < NB; k++)                          \
                               bj += b1_[k] * ((j == k) ? (f16)1 : (f16)0);                        \
-                          tl_stage_tile<true>(hlane + j * 16, ldh, c0, c1, bj);                          \
+                          tl_stage_tile<true>(hlane + j * 16, ldh, c0, c1, bj);                   \
                       } TL_TRC_ARG);                                                              \
         /* block-rows of this phase without any tile: bias only */                                \
         const int lim1 = min(((p_) + 1) * hbr, nbr1);                                             \
@@ -1307,8 +1303,6 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
                 bO[j] = *reinterpret_cast<const f16x4 *>(a.bias[0] + (x.bn0 + j) * 16 + g4 * 4);
         }
         TL_FFN_PRELOAD(a.data[0], a.row_offset[0], bvecO, wB, oB)
-        TlLnOperands<NB, NW, NW> lnop1;
-        tl_ln_fetch_at(lnop1, a.M, wave, lane, x.m0, NO, a.skip + (long)x.m0 * NO, (long)NO, a.gamma, a.beta);
         tl_barrier_lds(); // the whole panel has landed; the counters are zero
         {
             const int q0_ = __builtin_amdgcn_readfirstlane(bvecO), qe_ = __builtin_amdgcn_readlane(bvecO, NB);
@@ -1317,6 +1311,8 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
                           [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); } TL_TRC_ARG);
         }
         TL_FFN_PRELOAD(data1, poff1, bvecF, wA, oA)
+        TlLnOperands<NB, NW, NW> lnop1; // (requested here: their latency runs under the wait for the other waves)
+        tl_ln_fetch_at(lnop1, a.M, wave, lane, x.m0, NO, a.skip + (long)x.m0 * NO, (long)NO, a.gamma, a.beta);
         // staging tiles in the hidden buffers, which nobody uses yet
         tl_epilogue_wave<NB, false, false>(a, x, hs + wave * tl_wave_stage_halves<NB>(), nullptr, NO, nbrO, acc,
                                            bO);
@@ -1339,8 +1335,6 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
         // operands of the streams after the next two
         const int bvecSn = TL_FFN_BVEC2(min(p + 1, a.nchunk - 1));
         const int bvecF2 = TL_FFN_BVEC1(min(p + 2, a.nchunk - 1));
-        f16x4 b1n2[NB];
-        TL_FFN_BIAS1(b1n2, min(p + 2, a.nchunk - 1))
         TL_FFN_PRELOAD(data2, poff2, bvecS, wA, oA) // S(p), a stream ahead
         if (p + 1 < a.nchunk) {
             TL_STAMP(5);
@@ -1349,8 +1343,10 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
             TL_STAMP(6);
             TL_FFN_FIRST(p + 1, bvecFn, b1n, wB, oB)
         }
-        if (p + 2 < a.nchunk)
+        if (p + 2 < a.nchunk) {
             TL_FFN_PRELOAD(data1, poff1, bvecF2, wB, oB) // F(p+2), a stream ahead
+            TL_FFN_BIAS1(b1n, p + 2)
+        }
         TL_STAMP(7);
         tl_wait_count(ctr + p, NW); // hidden buffer p & 1 is complete
         TL_STAMP(8);
@@ -1364,9 +1360,6 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
         }
         bvecS = bvecSn;
         bvecFn = bvecF2;
-#pragma unroll
-        for (int k = 0; k < NB; k++)
-            b1n[k] = b1n2[k];
     }
 #undef TL_FFN_BVEC1
 #undef TL_FFN_BVEC2
@@ -1381,6 +1374,13 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
         tl_ln_fetch_at(lnop, a.M, wave, lane, x.m0, N2, xs, (long)ldx, a.gamma2, a.beta2);
     else
         tl_ln_fetch(lnop, a, wave, lane, x.m0, N2);
+    f16x4 b2[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        b2[j] = f16x4{0, 0, 0, 0};
+        if (x.bn0 + j < nbr2)
+            b2[j] = *reinterpret_cast<const f16x4 *>(a.bias[L2] + (x.bn0 + j) * 16 + g4 * 4);
+    }
     tl_barrier_lds(); // every wave has left the hidden buffers
     f16 *const stage0 = WITH_O ? hs : xs;
     tl_epilogue_wave<NB, false, false>(a, x, stage0 + wave * tl_wave_stage_halves<NB>(), a.Y[L2], N2, nbr2,
