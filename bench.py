@@ -37,11 +37,9 @@ D, H, DFF = 768, 12, 3072
 # default workload and scaled by the 64 MiB copy kernel launched below; commands and raw figures are in
 # profiles/encoder_layer_b16_s512_hbm_traffic.txt.  Only valid for batch 16 x seq 512 at 80 % sparsity.
 MEASURED_TRAFFIC_MIB = {
-    "tile_linear qkv (3 x 768->768, one launch)": 17.91 + 36.00,
-    "attention (on-the-fly)": 36.17 + 12.00,
-    "tile_linear o (768->768) + skip + LayerNorm": 26.09 + 12.00,
-    "tile_linear ffn1+gelu (768->3072)": 19.96 + 48.13,
-    "tile_linear ffn2 (3072->768) + skip + LayerNorm": 67.92 + 12.00,
+    "tile_linear qkv (3 x 768->768, one launch)": 17.91 + 36.01,
+    "attention (on-the-fly)": 36.16 + 12.00,
+    "layer tail: o + skip + LayerNorm + feed-forward (gelu) + skip + LayerNorm, fused": 43.44 + 14.00,
 }
 
 
