@@ -1115,7 +1115,7 @@ __global__ void __launch_bounds__(TL_CTHREADS) tile_linear_chunked_ln_kernel(con
 
 // ---------------------------------------------------------------------------
 // Fused feed-forward block: Y = LayerNorm(skip + W2 * gelu(W1 * X + b1) + b2)
-// in ONE launch (encoder/encoder.cu:33-41 runs it as MLP1, MLP2 and
+// in ONE launch (encoder/encoder.cu:36-44 runs it as MLP1, MLP2 and
 // skip_layernorm with the [rows x ffn] intermediate written to and read back
 // from memory).  One workgroup of 16 waves per 32-row panel keeps the panel of
 // X in LDS and walks the hidden dimension in chunks of the second plan's
@@ -1123,14 +1123,19 @@ __global__ void __launch_bounds__(TL_CTHREADS) tile_linear_chunked_ln_kernel(con
 // linear (bias, GELU, rounded to half exactly like the stored intermediate)
 // into one of two LDS buffers, then multiplies that buffer with chunk p of the
 // second linear into register accumulators that live across all phases.  The
-// hidden activations never leave the CU.  With two hidden buffers a single
-// barrier per phase is enough: phase p+1's first linear overwrites the buffer
-// that phase p-1's second linear read, and every wave has passed barrier p
-// since.  Each wave owns NB block-rows of either linear per phase; the first
-// pairs of a stream are requested one whole stream ahead (two register sets).
-// arguments: linear 0 = first (N[0] = hidden width), linear 1 = second
-// (N[1] = output width, Y[1] = output), K = input width, KC / nchunk = the
-// second plan's chunking.
+// hidden activations never leave the CU.  Each wave owns NB block-rows of
+// either linear per phase.  The first linear runs one phase ahead of the
+// second, and the hand-overs ("hidden buffer p is complete", "everyone has
+// finished reading it") are event counters in LDS rather than barriers, so a
+// wave only ever waits when it is a whole stream ahead of the slowest wave.
+// WITH_O: the attention output projection with its skip connection and
+// LayerNorm (encoder/encoder.cu:33-35) runs first on the same panel, and its
+// normalised rows replace the panel in LDS - steps 6-10 of a layer in one
+// launch.
+// arguments: [linear 0 = projection (WITH_O),] then the first feed-forward
+// linear (N = hidden width) and the second (N = output width, Y = output);
+// K = input width, KC / nchunk = the second plan's chunking; skip / gamma /
+// beta belong to the first LayerNorm that runs, gamma2 / beta2 to the second.
 // ---------------------------------------------------------------------------
 constexpr int TL_FFN_WAVES = 16;
 constexpr int TL_FFN_MAX_PHASES = 16;
