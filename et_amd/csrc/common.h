@@ -73,11 +73,24 @@ __device__ __forceinline__ void load_lds16(const void *gsrc, void *lds_base) {
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
 
 // ---- wave64 reductions (all lanes receive the result) -----------------------
+// Data-parallel-primitive moves inside a row of 16 lanes (no LDS round trip as
+// with __shfl): quad_perm [1,0,3,2] and [2,3,0,1], row_half_mirror, row_mirror.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m > 0; m >>= 1)
-        v += __shfl_xor(v, m, WAVE);
-    return v;
+    v += dpp_move<0xB1>(v);  // pairs
+    v += dpp_move<0x4E>(v);  // quads
+    v += dpp_move<0x141>(v); // 8 lanes
+    v += dpp_move<0x140>(v); // the row of 16: every lane holds its row's sum
+    // the four rows through scalar registers
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return (r0 + r1) + (r2 + r3);
 }
 
 __device__ __forceinline__ float f16_bits_to_float(uint16_t b) {

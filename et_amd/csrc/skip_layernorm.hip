@@ -26,6 +26,7 @@ skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip
     if (row0 >= num)
         return;
     const int nchunk = size >> 3;
+    const float inv_n = 1.0f / (float)size;
     const f16x8 *g = reinterpret_cast<const f16x8 *>(gamma);
     const f16x8 *b = reinterpret_cast<const f16x8 *>(beta);
     const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
@@ -51,9 +52,12 @@ skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             x[i] = an[i] + sn[i]; // half add, one rounding (kernels/skip_layernorm.cu:20)
+            // pairs of halves summed in fp32 by the dot-product unit (chunks
+            // beyond the row are zero)
+            typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-                sum += (float)x[i][j]; // chunks beyond the row are zero
+            for (int j = 0; j < 8; j += 2)
+                sum = __builtin_amdgcn_fdot2(h2{x[i][j], x[i][j + 1]}, h2{(f16)1, (f16)1}, sum, false);
         }
         if (r + 1 < ROWS && row + 1 < num) {
 #pragma unroll
@@ -65,7 +69,7 @@ skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip
                 }
             }
         }
-        const float mean = wave_sum(sum) / (float)size;
+        const float mean = wave_sum(sum) * inv_n;
         float var = 0.f;
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
@@ -78,7 +82,8 @@ skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip
                 }
             }
         }
-        const float rstd = rsqrtf(wave_sum(var) / (float)size + 1e-6f);
+        const float rstd = rsqrtf(wave_sum(var) * inv_n + 1e-6f);
+        const float shift = -mean * rstd;
         f16x8 *a = reinterpret_cast<f16x8 *>(in_out + row * size);
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
@@ -87,8 +92,8 @@ skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip
                 const f16x8 gg = g[c], bb = b[c];
                 f16x8 y;
 #pragma unroll
-                for (int j = 0; j < 8; j++)
-                    y[j] = (f16)(((float)x[i][j] - mean) * rstd * (float)gg[j] + (float)bb[j]);
+                for (int j = 0; j < 8; j++) // ((x - mean) * rstd) * gamma + beta, the first step as one fma
+                    y[j] = (f16)(__builtin_fmaf((float)x[i][j], rstd, shift) * (float)gg[j] + (float)bb[j]);
                 a[c] = y;
             }
         }

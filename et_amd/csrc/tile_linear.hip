@@ -448,6 +448,7 @@ __device__ __forceinline__ void tl_ln_rows_at(const TlLnOperands<NB, NW, NLW> &o
     constexpr int NCH = TlLnOperands<NB, NW, NLW>::NCH;
     constexpr int ROWS = TlLnOperands<NB, NW, NLW>::ROWS;
     const int npiece = N >> 3;
+    const float inv_n = 1.0f / (float)N;
     const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int k = 0; k < ROWS; k++) {
@@ -466,11 +467,13 @@ __device__ __forceinline__ void tl_ln_rows_at(const TlLnOperands<NB, NW, NLW> &o
                     stage0 + tile * tl_wave_stage_halves<NB>() + r * lds + c * 8);
                 xv[i] = y + op.skip[k][i]; // half add, one rounding (kernels/skip_layernorm.cu:20)
             }
+            // (pairs of halves summed in fp32 by the dot-product unit: no conversions)
+            typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-                sum += (float)xv[i][j];
+            for (int j = 0; j < 8; j += 2)
+                sum = __builtin_amdgcn_fdot2(h2{xv[i][j], xv[i][j + 1]}, h2{(f16)1, (f16)1}, sum, false);
         }
-        const float mean = wave_sum(sum) / (float)N;
+        const float mean = wave_sum(sum) * inv_n;
         float var = 0.f;
 #pragma unroll
         for (int i = 0; i < NCH; i++)
@@ -481,15 +484,16 @@ __device__ __forceinline__ void tl_ln_rows_at(const TlLnOperands<NB, NW, NLW> &o
                     var += d * d;
                 }
             }
-        const float rstd = rsqrtf(wave_sum(var) / (float)N + 1e-6f);
+        const float rstd = rsqrtf(wave_sum(var) * inv_n + 1e-6f);
+        const float shift = -mean * rstd;
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const int ch = lane + 64 * i;
             if (ch < npiece) {
                 f16x8 o;
 #pragma unroll
-                for (int j = 0; j < 8; j++)
-                    o[j] = (f16)(((float)xv[i][j] - mean) * rstd * (float)op.gamma[i][j] +
+                for (int j = 0; j < 8; j++) // ((x - mean) * rstd) * gamma + beta, the first step as one fma
+                    o[j] = (f16)(__builtin_fmaf((float)xv[i][j], rstd, shift) * (float)op.gamma[i][j] +
                                  (float)op.beta[i][j]);
                 *reinterpret_cast<f16x8 *>(Y0 + r * ldy + ch * 8) = o;
             }
