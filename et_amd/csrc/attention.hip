@@ -57,10 +57,23 @@ __device__ __forceinline__ f16x8 load8_guard(const f16 *p, int d0, int n) {
     return v;
 }
 
+// Maximum over the four lanes l, l^16, l^32, l^48 (a query's four key groups),
+// result in all four.  gfx950's row-swap instructions exchange whole rows of 16
+// lanes between two registers in the vector ALU, so no LDS round trip as with
+// __shfl_xor.  (The empty asm statements keep the optimiser from reasoning
+// about the swapped copies: it otherwise folds max(a, b) of the pair away.)
 __device__ __forceinline__ float xor_max_16_32(float v) {
-    v = fmaxf(v, __shfl_xor(v, 16, WAVE));
-    v = fmaxf(v, __shfl_xor(v, 32, WAVE));
-    return v;
+    unsigned a = __builtin_bit_cast(unsigned, v), b = a;
+    asm("" : "+v"(b));
+    auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false); // a: lanes 0-31 twice, b: lanes 32-63 twice
+    unsigned x0 = r[0], x1 = r[1];
+    asm("v_max_f32 %0, %0, %1" : "+v"(x0) : "v"(x1));
+    unsigned y1 = x0;
+    asm("" : "+v"(y1));
+    auto q = __builtin_amdgcn_permlane16_swap(x0, y1, false, false); // even rows twice, odd rows twice
+    unsigned z0 = q[0], z1 = q[1];
+    asm("v_max_f32 %0, %0, %1" : "+v"(z0) : "v"(z1));
+    return __builtin_bit_cast(float, z0);
 }
 
 template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK>
