@@ -169,11 +169,12 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
         }
 
         f32x4 ot[DV][QS];
-        float m_run[QS], l_run[QS];
+        float m_run[QS];
+        f32x4 l_acc[QS]; // row sums of P, accumulated by the matrix unit (all 16 rows of the tile equal)
 #pragma unroll
         for (int qs = 0; qs < QS; qs++) {
             m_run[qs] = -INFINITY;
-            l_run[qs] = 0.f;
+            l_acc[qs] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int d = 0; d < DV; d++)
                 ot[d][qs] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -474,13 +475,12 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                     const float m_fin = (m_new == -INFINITY) ? 0.f : m_new;
                     const float alpha = __builtin_amdgcn_exp2f((m_run[qs] - m_fin) * ls); // 1 where unchanged
                     m_run[qs] = m_new;
-                    l_run[qs] *= alpha;
+                    l_acc[qs] *= alpha;
 #pragma unroll
                     for (int d = 0; d < DV; d++)
                         ot[d][qs] *= alpha;
                 }
                 const float msc = ((m_run[qs] == -INFINITY) ? 0.f : m_run[qs]) * ls;
-                float psum = 0.f;
                 f16x2 ph[8];
 #pragma unroll
                 for (int ksub = 0; ksub < 4; ksub++)
@@ -490,11 +490,9 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                         float p1 = __builtin_fmaf(st[ksub][qs][2 * r2 + 1], ls, -msc);
                         p0 = __builtin_amdgcn_exp2f(p0);
                         p1 = __builtin_amdgcn_exp2f(p1);
-                        psum += p0 + p1;
                         typedef float f32x2 __attribute__((ext_vector_type(2)));
                         ph[ksub * 2 + r2] = __builtin_convertvector(f32x2{p0, p1}, f16x2);
                     }
-                l_run[qs] += psum;
 #pragma unroll
                 for (int kk = 0; kk < 2; kk++)
                     pf[qs][kk] = f16x8{ph[kk * 4 + 0][0], ph[kk * 4 + 0][1], ph[kk * 4 + 1][0], ph[kk * 4 + 1][1],
@@ -539,6 +537,15 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                         for (int qs = 0; qs < QS; qs++)
                             ot[d][qs] = mfma16x16x32(vfr[d & 1][kk], pf[qs][kk], ot[d][qs]);
                 }
+                // the softmax denominators: ones^T P^T sums a query's 64
+                // probabilities (as rounded to half for the product above)
+                // without any vector adds or cross-lane steps
+                const f16x8 ones8 = f16x8{1, 1, 1, 1, 1, 1, 1, 1};
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                    for (int qs = 0; qs < QS; qs++)
+                        l_acc[qs] = mfma16x16x32(ones8, pf[qs][kk], l_acc[qs]);
             }
         };
 
@@ -590,9 +597,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
         }
 #pragma unroll
         for (int qs = 0; qs < QS; qs++) {
-            float l = l_run[qs];
-            l += __shfl_xor(l, 16, WAVE);
-            l += __shfl_xor(l, 32, WAVE);
+            const float l = l_acc[qs][0];
             const float inv = l > 0.f ? 1.0f / l : 0.f;
             const int ql = (wave * QS + qs) * 16 + c16;
 #pragma unroll
