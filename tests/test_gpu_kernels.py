@@ -167,6 +167,8 @@ FFN_CASES = [
     (33, 512, 768, 0.7, True),      # hidden width in ONE chunk
     (40, 768, 1536 + 256, 0.8, True),  # last hidden chunk partial (256 of 768 columns)
     (64, 64, 3072, 0.9, True),      # tiny model width, many empty block-rows
+    (45, 80, 400, 0.5, True),       # widths that are multiples of 16 but not of 32 (unpadded LDS rows)
+    (32, 768, 768 * 17, 0.95, False),  # more hidden chunks than the kernel's event counters: step by step
     (50, 768, 896, 0.8, False),     # one hidden chunk of 896 columns: too wide for the fused kernel
     (36, 1024, 2048, 0.8, False),   # model width beyond one LDS panel
 ]
@@ -214,6 +216,8 @@ TAIL_CASES = [
     (77, 768, 3072, 0.5, True),    # ragged M
     (40, 256, 1024, 0.7, True),    # narrow rows: most waves own nothing in the projections
     (64, 64, 1536, 0.9, True),     # many empty block-rows
+    (45, 80, 400, 0.5, True),      # widths that are multiples of 16 but not of 32 (unpadded LDS rows)
+    (1, 768, 3072, 0.8, True),     # a single row
     (50, 768, 896, 0.8, False),    # hidden chunk too wide: step by step
 ]
 
