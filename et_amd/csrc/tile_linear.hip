@@ -1282,9 +1282,13 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
         tl_preload(data_, poff_, lane_w, hi, q0_, max(qe_ - 1, q0_), w_, o_);                     \
     }
 
-    // The streams run in the order F(0), F(1), S(0), F(2), S(1), ..., S(last)
-    // (F = first linear, S = second): the first linear stays one phase ahead,
-    // so what a wave waits for was finished by most waves a stream ago.
+    // Stream order (F = first linear, S = second).  Half of the waves run
+    // F(0) F(1) S(0) F(2) S(1) ... S(last), the first linear one phase ahead;
+    // the other half F(0) S(0) F(1) S(1) ...  Both orders respect "S(p) after
+    // every wave's F(p)" and "F(p+2) after every wave's S(p)" (the hidden buffer
+    // it overwrites), what a wave waits for was usually finished a stream ago,
+    // and at most times the two halves of a SIMD's waves are in different kinds
+    // of stream: F streams load the vector ALU (GELU), S streams hardly do.
     // Register set A serves F(0) and every S, set B every later F.
     f16x8 wA[TL_DEPTH], wB[TL_DEPTH];
     int oA[TL_DEPTH], oB[TL_DEPTH];
@@ -1340,21 +1344,22 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
         TL_FFN_PRELOAD(data1, poff1, bvecFn, wB, oB)
     TL_FFN_FIRST(0, bvecF, b1, wA, oA)
 
+    const int behind = (wave >> 2) & 1; // (a SIMD's waves are w, w+4, w+8, w+12)
     for (int p = 0; p < a.nchunk; p++) {
-        // operands of the streams after the next two
         const int bvecSn = TL_FFN_BVEC2(min(p + 1, a.nchunk - 1));
-        const int bvecF2 = TL_FFN_BVEC1(min(p + 2, a.nchunk - 1));
-        TL_FFN_PRELOAD(data2, poff2, bvecS, wA, oA) // S(p), a stream ahead
-        if (p + 1 < a.nchunk) {
+        TL_FFN_PRELOAD(data2, poff2, bvecS, wA, oA) // S(p), a stream ahead (unless no F runs in between)
+        const int fq = p + 1 - behind; // the first-linear phase this wave runs before S(p)
+        if (fq >= 1 && fq < a.nchunk) {
             TL_STAMP(5);
-            if (p >= 1) // F(p+1) overwrites the buffer that S(p-1) read
-                tl_wait_count(ctr + TL_FFN_MAX_PHASES + p - 1, NW);
+            if (fq >= 2) // F(fq) overwrites the buffer that S(fq-2) read
+                tl_wait_count(ctr + TL_FFN_MAX_PHASES + fq - 2, NW);
             TL_STAMP(6);
-            TL_FFN_FIRST(p + 1, bvecFn, b1n, wB, oB)
-        }
-        if (p + 2 < a.nchunk) {
-            TL_FFN_PRELOAD(data1, poff1, bvecF2, wB, oB) // F(p+2), a stream ahead
-            TL_FFN_BIAS1(b1n, p + 2)
+            TL_FFN_FIRST(fq, bvecFn, b1n, wB, oB)
+            if (fq + 1 < a.nchunk) { // F(fq+1), a stream (or two) ahead
+                bvecFn = TL_FFN_BVEC1(fq + 1);
+                TL_FFN_PRELOAD(data1, poff1, bvecFn, wB, oB)
+                TL_FFN_BIAS1(b1n, fq + 1)
+            }
         }
         TL_STAMP(7);
         tl_wait_count(ctr + p, NW); // hidden buffer p & 1 is complete
@@ -1368,7 +1373,6 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
             tl_signal(ctr + TL_FFN_MAX_PHASES + p, lane);
         }
         bvecS = bvecSn;
-        bvecFn = bvecF2;
     }
 #undef TL_FFN_BVEC1
 #undef TL_FFN_BVEC2
