@@ -62,6 +62,71 @@ def test_encoder_tile_layer(S, B, sp, ls, use_mask):
     assert np.array_equal(got2, got)
 
 
+@pytest.mark.parametrize("S,B", [(128, 2), (200, 3)])
+def test_encoder_tile_layer_fused_tail_forced(S, B):
+    """the one-launch layer tail (normally used from 96 row panels up) inside Encoder_tile, forced on small shapes"""
+    from et_amd import lib
+    from et_amd.encoder import Encoder_tile
+    r = rng(620 + S)
+    d, H, dff = 768, 12, 3072
+    lins, ln = make_layer(r, d, dff, 0.8, seed=940)
+    x = randn_h(r, (B * S, d))
+    mask = randn_h(r, (S, S), 0.5)
+    want = orc.encoder_tile_layer(x, lins, ln, mask, S, H, B, None, 1.0)
+    enc = Encoder_tile(d, S, H, workspace(Encoder_tile, d, S, H, B), *build_linears(lins, B * S), *ln, mask, B)
+    xd = dev(x)
+    stepwise = host(enc.run(torch.empty_like(xd), xd))
+    try:
+        lib().et_tuning_set(b"tile_ln_min_panels", 1)
+        fused = host(enc.run(torch.empty_like(xd), xd))
+        inplace = host(enc.run(xd, xd))
+    finally:
+        lib().et_tuning_set(b"tile_ln_min_panels", 0)
+    check_close(fused, want, what="Encoder_tile, fused tail")
+    check_close(stepwise, want, what="Encoder_tile, step by step")
+    assert np.abs(fused.astype(np.float32) - stepwise.astype(np.float32)).max() <= 2e-2
+    assert np.array_equal(inplace, fused)
+
+
+def test_encoder_tile_layer_vs_torch_fp32_layer():
+    """Independent of the oracle: a textbook post-LN transformer layer written with torch ops in fp32 on the CPU
+    (dense weights with the pruned tiles zeroed, softmax base e, tanh GELU, LayerNorm eps 1e-6)."""
+    import torch.nn.functional as F
+    from et_amd.encoder import Encoder_tile
+    r = rng(77)
+    d, H, dff, S, B = 768, 12, 3072, 128, 2
+    hd = d // H
+    lins, ln = make_layer(r, d, dff, 0.8, seed=960, std=0.03, bias_std=0.05)
+    x = randn_h(r, (B * S, d))
+    mask = randn_h(r, (S, S), 0.5)
+
+    def dense(l):
+        W = np.zeros((l["N"], l["K"]), np.float32)
+        rp, ro, data = l["row_ptr"], l["row_offset"], l["data"].reshape(-1, 16, 16)
+        for bn in range(l["N"] // 16):
+            for i in range(rp[bn], rp[bn + 1]):
+                W[bn * 16:(bn + 1) * 16, ro[i]:ro[i] + 16] = data[i]
+        return torch.from_numpy(W), torch.from_numpy(l["bias"].astype(np.float32))
+
+    (Wq, bq), (Wk, bk), (Wv, bv), (Wo, bo), (W1, b1), (W2, b2) = [dense(l) for l in lins]
+    g1, be1, g2, be2 = [torch.from_numpy(t.astype(np.float32)) for t in ln]
+    xt = torch.from_numpy(x.astype(np.float32))
+    q, k, v = F.linear(xt, Wq, bq), F.linear(xt, Wk, bk), F.linear(xt, Wv, bv)
+    heads = lambda t: t.view(B, S, H, hd).transpose(1, 2)
+    # the reference scales by half(sqrt(1/head_dim)) (kernels/attention.cu:126)
+    scale = float(np.float16(math.sqrt(1.0 / hd)))
+    p = torch.softmax(heads(q) @ heads(k).transpose(-1, -2) * scale + torch.from_numpy(mask.astype(np.float32)), -1)
+    attn = (p @ heads(v)).transpose(1, 2).reshape(B * S, d)
+    mid = F.layer_norm(F.linear(attn, Wo, bo) + xt, (d,), g1, be1, eps=1e-6)
+    y = F.layer_norm(F.linear(F.gelu(F.linear(mid, W1, b1), approximate="tanh"), W2, b2) + mid, (d,), g2, be2, eps=1e-6)
+    enc = Encoder_tile(d, S, H, workspace(Encoder_tile, d, S, H, B), *build_linears(lins, B * S), *ln, mask, B)
+    enc.set_log2_scale(LOG2E)  # textbook softmax instead of the reference's base 2
+    xd = dev(x)
+    got = host(enc.run(torch.empty_like(xd), xd))
+    # half storage between the steps against fp32 throughout
+    check_close(got, y.numpy(), max_abs=3e-2, mean_rel=3e-3, what="Encoder_tile vs torch fp32 layer")
+
+
 def test_encoder_prune_layer():
     from et_amd.encoder import Encoder_prune, Linear_row
     r = rng(600)
