@@ -1350,13 +1350,14 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
         TL_FFN_PRELOAD(data2, poff2, bvecS, wA, oA) // S(p), a stream ahead (unless no F runs in between)
         const int fq = p + 1 - behind; // the first-linear phase this wave runs before S(p)
         if (fq >= 1 && fq < a.nchunk) {
+            const int bvecF2 = TL_FFN_BVEC1(min(fq + 1, a.nchunk - 1)); // (scalar loads, used after the stream)
             TL_STAMP(5);
             if (fq >= 2) // F(fq) overwrites the buffer that S(fq-2) read
                 tl_wait_count(ctr + TL_FFN_MAX_PHASES + fq - 2, NW);
             TL_STAMP(6);
             TL_FFN_FIRST(fq, bvecFn, b1n, wB, oB)
+            bvecFn = bvecF2;
             if (fq + 1 < a.nchunk) { // F(fq+1), a stream (or two) ahead
-                bvecFn = TL_FFN_BVEC1(fq + 1);
                 TL_FFN_PRELOAD(data1, poff1, bvecFn, wB, oB)
                 TL_FFN_BIAS1(b1n, fq + 1)
             }
