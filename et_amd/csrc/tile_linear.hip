@@ -2204,6 +2204,30 @@ extern "C" int et_tile_plan_run_tail(const et_tile_plan *pO, const et_tile_plan 
             return rc;
         return et_tile_plan_run_ffn_ln(p1, p2, Y, mid, hidden, mid, gamma2, beta2, M, stream);
     }
+    // The fused kernel runs one workgroup per CU and 32-row panel, in rounds of
+    // as many panels as there are CUs.  A last round that would leave most CUs
+    // idle costs as much as a full one: with the caller's buffers at hand those
+    // rows run step by step instead (after the fused launch on the same stream;
+    // rows are independent).
+    if (mid && hidden) {
+        const int cus = std::max(et_device_cu_count(), 1);
+        const int panels = (M + TL_BM - 1) / TL_BM, full = panels / cus * cus, rem = panels - full;
+        if (full > 0 && rem > 0 && rem < g_tile_ln_min_panels) {
+            const int M1 = full * TL_BM;
+            int rc = et_tile_plan_run_tail(pO, p1, p2, Y, attn, input, nullptr, nullptr, gamma1, beta1, gamma2,
+                                           beta2, M1, stream);
+            if (rc != ET_OK)
+                return rc;
+            const size_t off = (size_t)M1 * pO->out_feat; // all of Y, attn, input, mid are [rows x model width]
+            f16 *midr = static_cast<f16 *>(mid) + off;
+            rc = et_tile_plan_run_ln(pO, midr, static_cast<const f16 *>(attn) + off,
+                                     static_cast<const f16 *>(input) + off, gamma1, beta1, M - M1, stream);
+            if (rc != ET_OK)
+                return rc;
+            return et_tile_plan_run_ffn_ln(p1, p2, static_cast<f16 *>(Y) + off, midr, hidden, midr, gamma2, beta2,
+                                           M - M1, stream);
+        }
+    }
     TlProblem o, a, b;
     o.Y = nullptr;
     o.cptr = pO->d_cptr;

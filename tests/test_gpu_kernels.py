@@ -263,6 +263,43 @@ def test_tile_layer_tail_fused(K, M, d, F, sp, fused):
         assert np.array_equal(host(ad), got)
 
 
+def test_tile_layer_tail_splits_off_a_small_last_round(K):
+    """one workgroup per CU and 32-row panel: a last round of few panels runs step by step behind the fused launch"""
+    from et_amd import lib
+    from et_amd.encoder import Linear_tile
+    cus = lib().et_device_cu_count()
+    assert cus > 0
+    d, F, sp = 256, 1024, 0.7
+    M = cus * 32 + 1607
+    r = rng(2900)
+    lo = make_tile_linear(r, d, d, sp, seed=11, std=0.05, bias_std=0.2)
+    l1 = make_tile_linear(r, F, d, sp, seed=12, std=0.05, bias_std=0.2)
+    l2 = make_tile_linear(r, d, F, sp, seed=13, std=0.05, bias_std=0.2)
+    attn, inp = randn_h(r, (M, d)), randn_h(r, (M, d))
+    g1, b1 = randn_h(r, (d,), 0.3) + np.float16(1), randn_h(r, (d,), 0.3)
+    g2, b2 = randn_h(r, (d,), 0.3) + np.float16(1), randn_h(r, (d,), 0.3)
+    mk = lambda l, K_, N_, gelu: Linear_tile(K_, N_, M, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], gelu)
+    to, t1, t2 = mk(lo, d, d, False), mk(l1, d, F, True), mk(l2, F, d, False)
+    ln = [dev(t) for t in (g1, b1, g2, b2)]
+    mid = torch.full((M, d), float("nan"), dtype=torch.float16, device="cuda")
+    hid = torch.empty((M, F), dtype=torch.float16, device="cuda")
+    got = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln, mid=mid, hidden=hid))
+    # the fused launch never writes mid; the rows of the last round go through it
+    midh = host(mid)
+    assert np.isnan(midh[:cus * 32].astype(np.float32)).all() and np.isfinite(midh[cus * 32:].astype(np.float32)).all()
+    rows = np.r_[0:64, cus * 32 - 64:cus * 32 + 64, M - 64:M]
+    o = orc.tile_linear(attn[rows], lo["row_ptr"], lo["row_offset"], lo["data"], lo["bias"], d)
+    m = orc.skip_layernorm(o, inp[rows], g1, b1)
+    h = orc.tile_linear(m, l1["row_ptr"], l1["row_offset"], l1["data"], l1["bias"], F, gelu=True)
+    y = orc.tile_linear(h, l2["row_ptr"], l2["row_offset"], l2["data"], l2["bias"], d)
+    want = orc.skip_layernorm(y, m, g2, b2)
+    check_close(got[rows], want, max_abs=3e-2, mean_rel=2e-3, what="layer tail with a split-off last round")
+    # all rows: equal to the fused kernel forced on everything, up to fp32 summation order in the last round
+    allf = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln))
+    assert np.array_equal(allf[:cus * 32], got[:cus * 32])
+    assert np.abs(allf.astype(np.float32) - got.astype(np.float32)).max() <= 3e-2
+
+
 def test_tile_linear_closed_form_reference_smoke_inputs(K):
     """weights = bias = 0.1 (test/gen_linear.cu:8,10): Y = 0.1*sum_{kept k} X + 0.1"""
     r = rng(12)
