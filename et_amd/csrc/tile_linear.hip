@@ -369,6 +369,90 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
     });
 }
 
+// The same stream over a 64-row panel: every W pair is used for four 16-row
+// subtiles (four MFMAs per kilobyte of W instead of two: the stream is bound by
+// delivering W, so this is what raises its throughput).  flush(j, c0..c3).
+template <int NB, class Flush>
+__device__ __forceinline__ void tl_stream64(const char *xlane, int xrow16, const f16 *data,
+                                          const int *poff, unsigned lane_w, unsigned hi, int q0,
+                                          int qend, int qlast, int bvec, f16x8 (&w)[TL_DEPTH],
+                                          int (&o)[TL_DEPTH], Flush &&flush
+#ifdef TL_STAGETRACE
+                                          , TlTracer *trc_ = nullptr
+#endif
+) {
+#ifdef TL_STAGETRACE
+    TlTracer dummy_{nullptr, 0, 0};
+    if (!trc_)
+        trc_ = &dummy_;
+#endif
+    if (q0 >= qend)
+        return;
+    TL_STAMP(3);
+    f32x4 cur0 = f32x4{0.f, 0.f, 0.f, 0.f}, cur1 = cur0, cur2 = cur0, cur3 = cur0;
+    int j = 0;
+    int bend = __builtin_amdgcn_readlane(bvec, 1);
+#pragma unroll
+    for (int t = 0; t < NB - 1; t++) { // leading empty block-rows
+        j += (bend == q0 && j + 1 < NB) ? 1 : 0;
+        bend = __builtin_amdgcn_readlane(bvec, j + 1);
+    }
+    f16x8 xa[2], xb[2], xc[2], xd[2];
+    xa[0] = *reinterpret_cast<const f16x8 *>(xlane + o[0]);
+    xb[0] = *reinterpret_cast<const f16x8 *>(xlane + o[0] + xrow16);
+    xc[0] = *reinterpret_cast<const f16x8 *>(xlane + o[0] + 2 * xrow16);
+    xd[0] = *reinterpret_cast<const f16x8 *>(xlane + o[0] + 3 * xrow16);
+    xa[1] = xb[1] = xc[1] = xd[1] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    int q = q0;
+    // running (wave-uniform) addresses of pair q + TL_DEPTH: a stage adds a
+    // constant, which goes into the load's immediate offset
+    const char *wp = reinterpret_cast<const char *>(data) + (size_t)(q0 + TL_DEPTH) * 1024;
+    const char *op = reinterpret_cast<const char *>(poff) + (size_t)(q0 + TL_DEPTH) * 8;
+    unsigned lane_lo = hi * 4u, lane_lw = lane_w * 2u;
+    auto stage = [&](auto ic, auto always) {
+        constexpr int I = decltype(ic)::value;
+        constexpr int S = I % TL_DEPTH, SN = (I + 1) % TL_DEPTH, P = I & 1;
+        xa[P ^ 1] = *reinterpret_cast<const f16x8 *>(xlane + o[SN]);
+        xb[P ^ 1] = *reinterpret_cast<const f16x8 *>(xlane + o[SN] + xrow16);
+        xc[P ^ 1] = *reinterpret_cast<const f16x8 *>(xlane + o[SN] + 2 * xrow16);
+        xd[P ^ 1] = *reinterpret_cast<const f16x8 *>(xlane + o[SN] + 3 * xrow16);
+        // keep the reads above the MFMAs: left alone, the scheduler sinks them
+        // to the end of the stage and every stage then waits out the LDS latency
+        __builtin_amdgcn_sched_barrier(0);
+        TL_STAMP(1);
+        cur0 = mfma16x16x32(w[S], xa[P], cur0);
+        cur1 = mfma16x16x32(w[S], xb[P], cur1);
+        cur2 = mfma16x16x32(w[S], xc[P], cur2);
+        cur3 = mfma16x16x32(w[S], xd[P], cur3);
+        // pair q + I + TL_DEPTH; the last stages of a stream request nothing:
+        // a request still in flight when the stream ends would make the next
+        // use of these registers wait out a full memory latency
+        if (decltype(always)::value || q + I + TL_DEPTH < qend)
+            tl_load_pair_at(wp + I * 1024, op + I * 8, lane_lo, lane_lw, w[S], o[S]);
+        if (q + I + 1 == bend) { // block-row j is complete
+            TL_STAMP(2);
+            flush(j, cur0, cur1, cur2, cur3);
+            cur0 = cur1 = cur2 = cur3 = f32x4{0.f, 0.f, 0.f, 0.f};
+            j++;
+            bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));
+#pragma unroll
+            for (int t = 0; t < NB - 2; t++) { // skip empty block-rows
+                j += (bend == q + I + 1 && j + 1 < NB) ? 1 : 0;
+                bend = __builtin_amdgcn_readlane(bvec, min(j + 1, NB));
+            }
+        }
+    };
+    for (; q + 2 * TL_DEPTH <= qend; q += TL_DEPTH) { // straight-line body: counted waits
+        tl_static_for<0, TL_DEPTH>([&](auto ic) { stage(ic, std::true_type()); });
+        wp += TL_DEPTH * 1024;
+        op += TL_DEPTH * 8;
+    }
+    tl_static_for<0, 2 * TL_DEPTH - 1>([&](auto ic) {
+        if (q + decltype(ic)::value < qend)
+            stage(ic, std::false_type());
+    });
+}
+
 // flush for kernels that keep NB static accumulators: acc[j] += cur with a
 // 0/1 mask per accumulator (branch-free; a branch per j makes the compiler
 // keep a copy of every accumulator per pipeline stage)
@@ -946,6 +1030,228 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
 #undef TL_PANEL
 #undef TL_BIAS
 #ifdef TL_TRACE
+    if (g_trace && lane == 0) {
+        unsigned hwid, xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        unsigned long long *t = g_trace + ((size_t)blockIdx.x * NW + wave) * 8;
+        t[0] = tt0; t[1] = tpanel; t[2] = tcomp; t[3] = tepi; t[4] = TL_TICK(); t[5] = hwid; t[6] = xcc; t[7] = tgap;
+    }
+#endif
+#undef TL_BVEC
+#undef TL_KARG
+}
+
+// The resident-panel kernel on 64-row panels (tl_stream64): one workgroup of 8
+// waves per CU (the panel and eight 64-row staging tiles fill the LDS), items
+// of 64 rows.  Used where there are enough 64-row items to fill the chip.
+constexpr int TL_BM64 = 64;
+template <int NB, bool GELU>
+__global__ void __launch_bounds__(TL_WAVES * 64) tile_linear_resident64_kernel(const TlArgs a) {
+    constexpr int NW = TL_WAVES;
+    constexpr bool LN = false;
+    extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
+    f16 *xs = reinterpret_cast<f16 *>(tl_smem);
+    const int vid = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3); // see tile_linear_plan_kernel
+    const int it0 = vid * a.ipw;
+    const int it1 = min(it0 + a.ipw, a.total);
+    if (it0 >= it1)
+        return;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int c16 = lane & 15, g4 = lane >> 4, khalf8 = (g4 & 1) * 8, hi = lane >> 5;
+    const int ldx = a.KC + ((a.KC & 31) ? 0 : TL_PAD);
+    const char *xlane = reinterpret_cast<const char *>(xs + c16 * ldx + khalf8);
+    const int xrow16 = 16 * ldx * 2; // bytes between the two 16-row subtiles
+    constexpr int lds = 16 * NB + 8; // halves per staged row
+    f16 *const stage0 = xs + TL_BM64 * ldx;
+    f16 *const stage = stage0 + wave * (TL_BM64 * (16 * NB + 8));
+    f16 *const stage_lane = stage + c16 * lds + g4 * 4;
+    const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    const int lane_w = hi * 256 + c16 * 16 + khalf8; // lane's halves inside a 1 KB tile pair
+
+    // pair-index boundaries of a wave's block-rows: lane j holds the start of
+    // block-row j, lane NB the end of the last one (read back with v_readlane)
+#define TL_BVEC(t_) ((t_).cptr[min((t_).bn0 + min(lane, NB), (t_).nbr)] >> 1)
+    // (block-rows beyond the matrix read the last block-row's bias; their
+    // output is never stored)
+#define TL_BIAS(dst_, t_)                                                                         \
+    _Pragma("unroll") for (int k = 0; k < NB; k++)                                                \
+        dst_[k] = *reinterpret_cast<const f16x4 *>(                                               \
+            (t_).bias + min((t_).bn0 + k, (t_).nbr - 1) * 16 + g4 * 4);
+    // wave w fills panel rows 8w..8w+7
+#define TL_PANEL(rp_)                                                                             \
+    {                                                                                             \
+        const int pcpr = a.K >> 3;                                                                \
+        _Pragma("unroll") for (int rr = 0; rr < TL_BM64 / NW; rr++) {                             \
+            const int row = (rp_) * TL_BM64 + wave * (TL_BM64 / NW) + rr;                         \
+            if (row < a.M) {                                                                      \
+                const f16 *src = a.X + (size_t)row * a.K;                                         \
+                f16 *dstrow = xs + (wave * (TL_BM64 / NW) + rr) * ldx;                            \
+                if (lane < pcpr)                                                                  \
+                    load_lds16(src + lane * 8, dstrow);                                           \
+                if (64 + lane < pcpr)                                                             \
+                    load_lds16(src + (64 + lane) * 8, dstrow + 512);                              \
+            }                                                                                     \
+        }                                                                                         \
+        __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): this wave's part has landed */           \
+        __syncthreads();                    /* ... and everyone else's */                         \
+    }
+    // the first pairs of an item's stream
+#define TL_PRELOAD(t_, bvec_)                                                                     \
+    {                                                                                             \
+        q0 = __builtin_amdgcn_readfirstlane(bvec_);                                               \
+        qend = __builtin_amdgcn_readlane(bvec_, NB);                                              \
+        qlast = max(qend - 1, q0);                                                                \
+        wdata = (t_).data;                                                                        \
+        wpoff = (t_).poff;                                                                        \
+        tl_preload(wdata, wpoff, lane_w, hi, q0, qlast, w, o);                                    \
+    }
+
+    // Per-linear arguments are read from the kernel-argument segment with a
+    // run-time index (scalar loads).  Indexing the by-value struct itself would
+    // make the compiler copy it to scratch memory, and chains of selects over
+    // its constant-indexed elements compile to long branch ladders.
+    typedef const __attribute__((address_space(4))) char *KArg;
+    const KArg ka = (KArg)__builtin_amdgcn_kernarg_segment_ptr(); // TlArgs is the only argument
+#define TL_KARG(type_, field_, lin_)                                                              \
+    (*(const __attribute__((address_space(4))) type_ *)(ka + offsetof(TlArgs, field_) +           \
+                                                         (lin_) * sizeof(type_)))
+    auto tl_item = [&](int rp, int lin, int cg) {
+        TlItem t;
+        t.rp = rp;
+        t.lin = lin;
+        t.cg = cg;
+        t.bn0 = (cg * NW + wave) * NB;
+        typedef f16 *YPtr;
+        typedef const int *IPtr;
+        typedef const f16 *HPtr;
+        t.Y = TL_KARG(YPtr, Y, lin);
+        t.cptr = TL_KARG(IPtr, cptr, lin);
+        t.poff = TL_KARG(IPtr, row_offset, lin);
+        t.data = TL_KARG(HPtr, data, lin);
+        t.bias = TL_KARG(HPtr, bias, lin);
+        t.N = TL_KARG(int, N, lin);
+        t.nbr = t.N >> 4;
+        return t;
+    };
+    // the item after t in (row panel, linear, column group) order
+    auto tl_next = [&](const TlItem &t) {
+        const bool cw = t.cg + 1 == a.ncg;
+        const bool lw = cw && t.lin + 1 == a.nlin;
+        return tl_item(t.rp + (lw ? 1 : 0), lw ? 0 : t.lin + (cw ? 1 : 0), cw ? 0 : t.cg + 1);
+    };
+#if 0
+    const unsigned long long tt0 = TL_TICK();
+    unsigned long long tpanel = 0, tcomp = 0, tepi = 0, tgap = 0, tlast = tt0;
+#endif
+    const int per_rp = a.ncg * a.nlin;
+    const int rp0 = it0 / per_rp, rest0 = it0 - rp0 * per_rp;
+    TlItem cur = tl_item(rp0, rest0 / a.ncg, rest0 % a.ncg);
+
+    int bvec = TL_BVEC(cur);
+    f16x4 b4[NB];
+    TL_BIAS(b4, cur)
+    TL_PANEL(cur.rp)
+    int q0, qend, qlast;
+    const f16 *wdata;
+    const int *wpoff;
+    f16x8 w[TL_DEPTH];
+    int o[TL_DEPTH];
+    TL_PRELOAD(cur, bvec)
+#if 0
+    tlast = TL_TICK();
+    tpanel = tlast - tt0;
+#endif
+
+    for (int it = it0;; it++) {
+        const bool has_next = it + 1 < it1;
+        const TlItem nxt = tl_next(cur); // (past the last item: a valid linear, never run)
+        const int bvec_n = TL_BVEC(nxt);
+        f16x4 b4n[NB];
+        TL_BIAS(b4n, nxt)
+
+#if 0
+        const unsigned long long ta = TL_TICK();
+        tgap += ta - tlast;
+#endif
+        // a finished block-row goes straight to the wave's staging tile
+        tl_stream64<NB>(xlane, xrow16, wdata, wpoff, lane_w, hi, q0, qend, qlast, bvec, w, o,
+                      [&](int j, f32x4 c0, f32x4 c1, f32x4 c2, f32x4 c3) {
+                          // bias of block-row j as a 0/1-masked sum (exact); a chain
+                          // of selects over b4[] would be turned into an indexed
+                          // load and put the array into scratch memory
+                          f16x4 bj = f16x4{0, 0, 0, 0};
+#pragma unroll
+                          for (int k = 0; k < NB; k++)
+                              bj += b4[k] * ((j == k) ? (f16)1 : (f16)0);
+                          tl_stage_tile<GELU>(stage_lane + j * 16, lds, c0, c1, bj);
+                          tl_stage_tile<GELU>(stage_lane + 32 * lds + j * 16, lds, c2, c3, bj);
+                      });
+#if 0
+        const unsigned long long tb = TL_TICK();
+        tcomp += tb - ta;
+#endif
+        // block-rows without any tile: bias only
+#pragma unroll
+        for (int k = 0; k < NB; k++)
+            if (__builtin_amdgcn_readlane(bvec, k) == __builtin_amdgcn_readlane(bvec, k + 1))
+            {
+                tl_stage_tile<GELU>(stage_lane + k * 16, lds, f32x4{0.f, 0.f, 0.f, 0.f},
+                                    f32x4{0.f, 0.f, 0.f, 0.f}, b4[k]);
+                tl_stage_tile<GELU>(stage_lane + 32 * lds + k * 16, lds, f32x4{0.f, 0.f, 0.f, 0.f},
+                                    f32x4{0.f, 0.f, 0.f, 0.f}, b4[k]);
+            }
+
+        const bool same_panel = has_next && nxt.rp == cur.rp;
+        if (same_panel)
+            TL_PRELOAD(nxt, bvec_n)
+
+        if constexpr (LN) {
+            // the workgroup holds whole rows: skip connection + LayerNorm here
+            TlLnOperands<NB, NW, NW> lnop;
+            tl_ln_fetch(lnop, a, wave, lane, cur.rp * TL_BM64, cur.N);
+            __syncthreads(); // every wave's part of the rows is staged
+            tl_ln_rows(lnop, a, stage0, wave, lane, cur.rp * TL_BM64, cur.Y, cur.N);
+            if (has_next && same_panel)
+                __syncthreads(); // the staging tiles are free again
+        } else {
+            // staging tile -> Y: 16-byte stores of 32*NB contiguous bytes per row
+            const int nvalid = min(NB, cur.nbr - cur.bn0); // the last column group may be partial
+            const int cpr = 2 * nvalid;                    // 16-byte chunks per row
+            const int m0 = cur.rp * TL_BM64;
+            f16 *ybase = cur.Y + (size_t)m0 * cur.N + cur.bn0 * 16;
+#pragma unroll
+            for (int t = 0; t < 2 * NB; t++) {
+                const int i = lane + 64 * t;
+                const int r = i / (2 * NB), c = i - r * (2 * NB);
+                if (c < cpr && m0 + r < a.M) {
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + r * lds + c * 8);
+                    *reinterpret_cast<u32x4 *>(ybase + (size_t)r * cur.N + c * 8) = v;
+                }
+            }
+        }
+#if 0
+        tlast = TL_TICK();
+        tepi += tlast - tb;
+#endif
+        if (!has_next)
+            break;
+        if (!same_panel) {
+            __syncthreads(); // every wave is done with the previous panel
+            TL_PANEL(nxt.rp)
+            TL_PRELOAD(nxt, bvec_n)
+        }
+        cur = nxt;
+        bvec = bvec_n;
+#pragma unroll
+        for (int k = 0; k < NB; k++)
+            b4[k] = b4n[k];
+    }
+#undef TL_PRELOAD
+#undef TL_PANEL
+#undef TL_BIAS
+#if 0
     if (g_trace && lane == 0) {
         unsigned hwid, xcc;
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
@@ -1720,6 +2026,17 @@ static int choose_nb(int nrp, int nbr_max, int nlin) {
     return 1;
 }
 
+static int g_tile_bm64 = 1; // et_tuning_set("tile_bm64")
+
+template <bool GELU>
+static int launch_resident64(const TlArgs &a, size_t lds, hipStream_t st) {
+    auto k = tile_linear_resident64_kernel<3, GELU>;
+    ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_THREADS), lds, st, a);
+    return launch_status("tile_linear (64-row panels) launch");
+}
+
 static int tile_launch(const TlProblem *probs, int nlin, const f16 *X, int M, int K,
                        int KC, int nchunk, bool gelu, int mode, hipStream_t st) {
     TlArgs a;
@@ -1742,6 +2059,38 @@ static int tile_launch(const TlProblem *probs, int nlin, const f16 *X, int M, in
     a.K = K;
     a.KC = KC;
     a.nchunk = nchunk;
+    if (mode == TL_PLAN && nchunk == 1 && g_tile_bm64 && g_tile_nb == 0) {
+        // 64-row panels, one workgroup per CU: twice the rows per kilobyte of W
+        // streamed.  Needs the panel and eight 64-row staging tiles in LDS and
+        // at least two items per CU.
+        const int cus = std::max(et_device_cu_count(), 1);
+        const size_t lds64 = (size_t)TL_BM64 * (KC + ((KC & 31) ? 0 : TL_PAD)) * sizeof(f16) +
+                             (size_t)TL_WAVES * TL_BM64 * (16 * 3 + 8) * sizeof(f16);
+        const int nrp64 = (M + TL_BM64 - 1) / TL_BM64;
+        const int ncg64 = (nbr_max + TL_WAVES * 3 - 1) / (TL_WAVES * 3);
+        const long items = (long)nrp64 * ncg64 * nlin;
+        if (lds64 <= 160 * 1024 && items >= 2L * cus) {
+            a.ncg = ncg64;
+            a.total = (int)items;
+            const int per_rp = ncg64 * nlin;
+            double best = 0.0;
+            a.ipw = 1;
+            for (int d = 1; d <= per_rp; d++) { // as below, with one workgroup slot per CU
+                if (per_rp % d)
+                    continue;
+                const long nwg = items / d, rounds = (nwg + cus - 1) / cus;
+                const double cost = (double)rounds * (2.0 / 3.0 + d);
+                if (d == 1 || cost < best * 0.999) {
+                    best = cost;
+                    a.ipw = d;
+                }
+            }
+            if (g_tile_ipw > 0)
+                a.ipw = g_tile_ipw;
+            a.per_xcd = ((a.total + a.ipw - 1) / a.ipw + 7) / 8;
+            return gelu ? launch_resident64<true>(a, lds64, st) : launch_resident64<false>(a, lds64, st);
+        }
+    }
     const int nrp = (M + TL_BM - 1) / TL_BM;
     const int nb = choose_nb(nrp, nbr_max, nlin);
     a.ncg = (nbr_max + TL_WAVES * nb - 1) / (TL_WAVES * nb);
@@ -1839,6 +2188,10 @@ extern "C" int et_tuning_set(const char *key, int value) {
     }
     if (key && !strcmp(key, "tile_ipw")) {
         et::g_tile_ipw = value;
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "tile_bm64")) {
+        et::g_tile_bm64 = value;
         return ET_OK;
     }
     if (key && !strcmp(key, "tile_fuse_ffn")) {
