@@ -326,6 +326,8 @@ int et_device_synchronize(void);
  *                     as two launches; 1 (default): fused where the rows fit
  *   "tile_ln_min_panels" fewest 32-row panels for which et_tile_plan_run_ln
  *                     fuses (default 96; below, two launches are faster)
+ *   "tile_bm64"       0: planned linears always use 32-row panels; 1 (default):
+ *                     64-row panels where two such items per CU exist
  *   "tile_fuse_ffn"   0: et_tile_plan_ffn_fusable answers no (the feed-forward
  *                     block runs as separate launches); 1: the block is fused
  *                     but et_tile_plan_tail_fusable answers no; 2 (default)
