@@ -831,8 +831,12 @@ __device__ __forceinline__ void tl_stage_tile(f16 *dst, int lds, f32x4 c0, f32x4
     *reinterpret_cast<f16x4 *>(dst + 16 * lds) = o1;
 }
 
-template <int NB, bool GELU, int NW, bool LN>
+template <int NB, bool GELU, int NW, bool LN, int BM = TL_BM>
 __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlArgs a) {
+    // BM = 64: 64-row panels and items (tl_stream64: four MFMAs per streamed W
+    // pair), one workgroup per CU - the panel and the 64-row staging tiles fill
+    // the LDS.  Chosen by the launcher where enough 64-row items exist.
+    static_assert(BM == TL_BM || (BM == 2 * TL_BM && !LN), "64-row panels: without the LayerNorm epilogue");
     extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
     f16 *xs = reinterpret_cast<f16 *>(tl_smem);
     const int vid = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3); // see tile_linear_plan_kernel
@@ -847,8 +851,8 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
     const char *xlane = reinterpret_cast<const char *>(xs + c16 * ldx + khalf8);
     const int xrow16 = 16 * ldx * 2; // bytes between the two 16-row subtiles
     constexpr int lds = 16 * NB + 8; // halves per staged row
-    f16 *const stage0 = xs + TL_BM * ldx;
-    f16 *const stage = stage0 + wave * tl_wave_stage_halves<NB>();
+    f16 *const stage0 = xs + BM * ldx;
+    f16 *const stage = stage0 + wave * (BM * (16 * NB + 8));
     f16 *const stage_lane = stage + c16 * lds + g4 * 4;
     const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     const int lane_w = hi * 256 + c16 * 16 + khalf8; // lane's halves inside a 1 KB tile pair
@@ -862,15 +866,15 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
     _Pragma("unroll") for (int k = 0; k < NB; k++)                                                \
         dst_[k] = *reinterpret_cast<const f16x4 *>(                                               \
             (t_).bias + min((t_).bn0 + k, (t_).nbr - 1) * 16 + g4 * 4);
-    // wave w fills panel rows 4w..4w+3 (see tile_linear_plan_kernel)
+    // wave w fills panel rows (BM/NW)w ... (see tile_linear_plan_kernel)
 #define TL_PANEL(rp_)                                                                             \
     {                                                                                             \
         const int pcpr = a.K >> 3;                                                                \
-        _Pragma("unroll") for (int rr = 0; rr < TL_BM / NW; rr++) {                               \
-            const int row = (rp_) * TL_BM + wave * (TL_BM / NW) + rr;                             \
+        _Pragma("unroll") for (int rr = 0; rr < BM / NW; rr++) {                               \
+            const int row = (rp_) * BM + wave * (BM / NW) + rr;                             \
             if (row < a.M) {                                                                      \
                 const f16 *src = a.X + (size_t)row * a.K;                                         \
-                f16 *dstrow = xs + (wave * (TL_BM / NW) + rr) * ldx;                                       \
+                f16 *dstrow = xs + (wave * (BM / NW) + rr) * ldx;                                       \
                 if (lane < pcpr)                                                                  \
                     load_lds16(src + lane * 8, dstrow);                                           \
                 if (64 + lane < pcpr)                                                             \
@@ -959,17 +963,29 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
         tgap += ta - tlast;
 #endif
         // a finished block-row goes straight to the wave's staging tile
-        tl_stream<NB>(xlane, xrow16, wdata, wpoff, lane_w, hi, q0, qend, qlast, bvec, w, o,
-                      [&](int j, f32x4 c0, f32x4 c1) {
-                          // bias of block-row j as a 0/1-masked sum (exact); a chain
-                          // of selects over b4[] would be turned into an indexed
-                          // load and put the array into scratch memory
-                          f16x4 bj = f16x4{0, 0, 0, 0};
+        // bias of block-row j as a 0/1-masked sum (exact); a chain of selects
+        // over b4[] would be turned into an indexed load and put the array into
+        // scratch memory
+        auto bias_of = [&](int j) {
+            f16x4 bj = f16x4{0, 0, 0, 0};
 #pragma unroll
-                          for (int k = 0; k < NB; k++)
-                              bj += b4[k] * ((j == k) ? (f16)1 : (f16)0);
-                          tl_stage_tile<GELU>(stage_lane + j * 16, lds, c0, c1, bj);
-                      });
+            for (int k = 0; k < NB; k++)
+                bj += b4[k] * ((j == k) ? (f16)1 : (f16)0);
+            return bj;
+        };
+        if constexpr (BM == TL_BM) {
+            tl_stream<NB>(xlane, xrow16, wdata, wpoff, lane_w, hi, q0, qend, qlast, bvec, w, o,
+                          [&](int j, f32x4 c0, f32x4 c1) {
+                              tl_stage_tile<GELU>(stage_lane + j * 16, lds, c0, c1, bias_of(j));
+                          });
+        } else {
+            tl_stream64<NB>(xlane, xrow16, wdata, wpoff, lane_w, hi, q0, qend, qlast, bvec, w, o,
+                            [&](int j, f32x4 c0, f32x4 c1, f32x4 c2, f32x4 c3) {
+                                const f16x4 bj = bias_of(j);
+                                tl_stage_tile<GELU>(stage_lane + j * 16, lds, c0, c1, bj);
+                                tl_stage_tile<GELU>(stage_lane + 32 * lds + j * 16, lds, c2, c3, bj);
+                            });
+        }
 #ifdef TL_TRACE
         const unsigned long long tb = TL_TICK();
         tcomp += tb - ta;
@@ -977,9 +993,12 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
         // block-rows without any tile: bias only
 #pragma unroll
         for (int k = 0; k < NB; k++)
-            if (__builtin_amdgcn_readlane(bvec, k) == __builtin_amdgcn_readlane(bvec, k + 1))
-                tl_stage_tile<GELU>(stage_lane + k * 16, lds, f32x4{0.f, 0.f, 0.f, 0.f},
-                                    f32x4{0.f, 0.f, 0.f, 0.f}, b4[k]);
+            if (__builtin_amdgcn_readlane(bvec, k) == __builtin_amdgcn_readlane(bvec, k + 1)) {
+#pragma unroll
+                for (int h = 0; h < BM / TL_BM; h++)
+                    tl_stage_tile<GELU>(stage_lane + h * 32 * lds + k * 16, lds, f32x4{0.f, 0.f, 0.f, 0.f},
+                                        f32x4{0.f, 0.f, 0.f, 0.f}, b4[k]);
+            }
 
         const bool same_panel = has_next && nxt.rp == cur.rp;
         if (same_panel)
@@ -988,19 +1007,19 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
         if constexpr (LN) {
             // the workgroup holds whole rows: skip connection + LayerNorm here
             TlLnOperands<NB, NW, NW> lnop;
-            tl_ln_fetch(lnop, a, wave, lane, cur.rp * TL_BM, cur.N);
+            tl_ln_fetch(lnop, a, wave, lane, cur.rp * BM, cur.N);
             __syncthreads(); // every wave's part of the rows is staged
-            tl_ln_rows(lnop, a, stage0, wave, lane, cur.rp * TL_BM, cur.Y, cur.N);
+            tl_ln_rows(lnop, a, stage0, wave, lane, cur.rp * BM, cur.Y, cur.N);
             if (has_next && same_panel)
                 __syncthreads(); // the staging tiles are free again
         } else {
             // staging tile -> Y: 16-byte stores of 32*NB contiguous bytes per row
             const int nvalid = min(NB, cur.nbr - cur.bn0); // the last column group may be partial
             const int cpr = 2 * nvalid;                    // 16-byte chunks per row
-            const int m0 = cur.rp * TL_BM;
+            const int m0 = cur.rp * BM;
             f16 *ybase = cur.Y + (size_t)m0 * cur.N + cur.bn0 * 16;
 #pragma unroll
-            for (int t = 0; t < NB; t++) {
+            for (int t = 0; t < NB * (BM / TL_BM); t++) {
                 const int i = lane + 64 * t;
                 const int r = i / (2 * NB), c = i - r * (2 * NB);
                 if (c < cpr && m0 + r < a.M) {
@@ -1030,228 +1049,6 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
 #undef TL_PANEL
 #undef TL_BIAS
 #ifdef TL_TRACE
-    if (g_trace && lane == 0) {
-        unsigned hwid, xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        unsigned long long *t = g_trace + ((size_t)blockIdx.x * NW + wave) * 8;
-        t[0] = tt0; t[1] = tpanel; t[2] = tcomp; t[3] = tepi; t[4] = TL_TICK(); t[5] = hwid; t[6] = xcc; t[7] = tgap;
-    }
-#endif
-#undef TL_BVEC
-#undef TL_KARG
-}
-
-// The resident-panel kernel on 64-row panels (tl_stream64): one workgroup of 8
-// waves per CU (the panel and eight 64-row staging tiles fill the LDS), items
-// of 64 rows.  Used where there are enough 64-row items to fill the chip.
-constexpr int TL_BM64 = 64;
-template <int NB, bool GELU>
-__global__ void __launch_bounds__(TL_WAVES * 64) tile_linear_resident64_kernel(const TlArgs a) {
-    constexpr int NW = TL_WAVES;
-    constexpr bool LN = false;
-    extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
-    f16 *xs = reinterpret_cast<f16 *>(tl_smem);
-    const int vid = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3); // see tile_linear_plan_kernel
-    const int it0 = vid * a.ipw;
-    const int it1 = min(it0 + a.ipw, a.total);
-    if (it0 >= it1)
-        return;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
-    const int c16 = lane & 15, g4 = lane >> 4, khalf8 = (g4 & 1) * 8, hi = lane >> 5;
-    const int ldx = a.KC + ((a.KC & 31) ? 0 : TL_PAD);
-    const char *xlane = reinterpret_cast<const char *>(xs + c16 * ldx + khalf8);
-    const int xrow16 = 16 * ldx * 2; // bytes between the two 16-row subtiles
-    constexpr int lds = 16 * NB + 8; // halves per staged row
-    f16 *const stage0 = xs + TL_BM64 * ldx;
-    f16 *const stage = stage0 + wave * (TL_BM64 * (16 * NB + 8));
-    f16 *const stage_lane = stage + c16 * lds + g4 * 4;
-    const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-    const int lane_w = hi * 256 + c16 * 16 + khalf8; // lane's halves inside a 1 KB tile pair
-
-    // pair-index boundaries of a wave's block-rows: lane j holds the start of
-    // block-row j, lane NB the end of the last one (read back with v_readlane)
-#define TL_BVEC(t_) ((t_).cptr[min((t_).bn0 + min(lane, NB), (t_).nbr)] >> 1)
-    // (block-rows beyond the matrix read the last block-row's bias; their
-    // output is never stored)
-#define TL_BIAS(dst_, t_)                                                                         \
-    _Pragma("unroll") for (int k = 0; k < NB; k++)                                                \
-        dst_[k] = *reinterpret_cast<const f16x4 *>(                                               \
-            (t_).bias + min((t_).bn0 + k, (t_).nbr - 1) * 16 + g4 * 4);
-    // wave w fills panel rows 8w..8w+7
-#define TL_PANEL(rp_)                                                                             \
-    {                                                                                             \
-        const int pcpr = a.K >> 3;                                                                \
-        _Pragma("unroll") for (int rr = 0; rr < TL_BM64 / NW; rr++) {                             \
-            const int row = (rp_) * TL_BM64 + wave * (TL_BM64 / NW) + rr;                         \
-            if (row < a.M) {                                                                      \
-                const f16 *src = a.X + (size_t)row * a.K;                                         \
-                f16 *dstrow = xs + (wave * (TL_BM64 / NW) + rr) * ldx;                            \
-                if (lane < pcpr)                                                                  \
-                    load_lds16(src + lane * 8, dstrow);                                           \
-                if (64 + lane < pcpr)                                                             \
-                    load_lds16(src + (64 + lane) * 8, dstrow + 512);                              \
-            }                                                                                     \
-        }                                                                                         \
-        __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): this wave's part has landed */           \
-        __syncthreads();                    /* ... and everyone else's */                         \
-    }
-    // the first pairs of an item's stream
-#define TL_PRELOAD(t_, bvec_)                                                                     \
-    {                                                                                             \
-        q0 = __builtin_amdgcn_readfirstlane(bvec_);                                               \
-        qend = __builtin_amdgcn_readlane(bvec_, NB);                                              \
-        qlast = max(qend - 1, q0);                                                                \
-        wdata = (t_).data;                                                                        \
-        wpoff = (t_).poff;                                                                        \
-        tl_preload(wdata, wpoff, lane_w, hi, q0, qlast, w, o);                                    \
-    }
-
-    // Per-linear arguments are read from the kernel-argument segment with a
-    // run-time index (scalar loads).  Indexing the by-value struct itself would
-    // make the compiler copy it to scratch memory, and chains of selects over
-    // its constant-indexed elements compile to long branch ladders.
-    typedef const __attribute__((address_space(4))) char *KArg;
-    const KArg ka = (KArg)__builtin_amdgcn_kernarg_segment_ptr(); // TlArgs is the only argument
-#define TL_KARG(type_, field_, lin_)                                                              \
-    (*(const __attribute__((address_space(4))) type_ *)(ka + offsetof(TlArgs, field_) +           \
-                                                         (lin_) * sizeof(type_)))
-    auto tl_item = [&](int rp, int lin, int cg) {
-        TlItem t;
-        t.rp = rp;
-        t.lin = lin;
-        t.cg = cg;
-        t.bn0 = (cg * NW + wave) * NB;
-        typedef f16 *YPtr;
-        typedef const int *IPtr;
-        typedef const f16 *HPtr;
-        t.Y = TL_KARG(YPtr, Y, lin);
-        t.cptr = TL_KARG(IPtr, cptr, lin);
-        t.poff = TL_KARG(IPtr, row_offset, lin);
-        t.data = TL_KARG(HPtr, data, lin);
-        t.bias = TL_KARG(HPtr, bias, lin);
-        t.N = TL_KARG(int, N, lin);
-        t.nbr = t.N >> 4;
-        return t;
-    };
-    // the item after t in (row panel, linear, column group) order
-    auto tl_next = [&](const TlItem &t) {
-        const bool cw = t.cg + 1 == a.ncg;
-        const bool lw = cw && t.lin + 1 == a.nlin;
-        return tl_item(t.rp + (lw ? 1 : 0), lw ? 0 : t.lin + (cw ? 1 : 0), cw ? 0 : t.cg + 1);
-    };
-#if 0
-    const unsigned long long tt0 = TL_TICK();
-    unsigned long long tpanel = 0, tcomp = 0, tepi = 0, tgap = 0, tlast = tt0;
-#endif
-    const int per_rp = a.ncg * a.nlin;
-    const int rp0 = it0 / per_rp, rest0 = it0 - rp0 * per_rp;
-    TlItem cur = tl_item(rp0, rest0 / a.ncg, rest0 % a.ncg);
-
-    int bvec = TL_BVEC(cur);
-    f16x4 b4[NB];
-    TL_BIAS(b4, cur)
-    TL_PANEL(cur.rp)
-    int q0, qend, qlast;
-    const f16 *wdata;
-    const int *wpoff;
-    f16x8 w[TL_DEPTH];
-    int o[TL_DEPTH];
-    TL_PRELOAD(cur, bvec)
-#if 0
-    tlast = TL_TICK();
-    tpanel = tlast - tt0;
-#endif
-
-    for (int it = it0;; it++) {
-        const bool has_next = it + 1 < it1;
-        const TlItem nxt = tl_next(cur); // (past the last item: a valid linear, never run)
-        const int bvec_n = TL_BVEC(nxt);
-        f16x4 b4n[NB];
-        TL_BIAS(b4n, nxt)
-
-#if 0
-        const unsigned long long ta = TL_TICK();
-        tgap += ta - tlast;
-#endif
-        // a finished block-row goes straight to the wave's staging tile
-        tl_stream64<NB>(xlane, xrow16, wdata, wpoff, lane_w, hi, q0, qend, qlast, bvec, w, o,
-                      [&](int j, f32x4 c0, f32x4 c1, f32x4 c2, f32x4 c3) {
-                          // bias of block-row j as a 0/1-masked sum (exact); a chain
-                          // of selects over b4[] would be turned into an indexed
-                          // load and put the array into scratch memory
-                          f16x4 bj = f16x4{0, 0, 0, 0};
-#pragma unroll
-                          for (int k = 0; k < NB; k++)
-                              bj += b4[k] * ((j == k) ? (f16)1 : (f16)0);
-                          tl_stage_tile<GELU>(stage_lane + j * 16, lds, c0, c1, bj);
-                          tl_stage_tile<GELU>(stage_lane + 32 * lds + j * 16, lds, c2, c3, bj);
-                      });
-#if 0
-        const unsigned long long tb = TL_TICK();
-        tcomp += tb - ta;
-#endif
-        // block-rows without any tile: bias only
-#pragma unroll
-        for (int k = 0; k < NB; k++)
-            if (__builtin_amdgcn_readlane(bvec, k) == __builtin_amdgcn_readlane(bvec, k + 1))
-            {
-                tl_stage_tile<GELU>(stage_lane + k * 16, lds, f32x4{0.f, 0.f, 0.f, 0.f},
-                                    f32x4{0.f, 0.f, 0.f, 0.f}, b4[k]);
-                tl_stage_tile<GELU>(stage_lane + 32 * lds + k * 16, lds, f32x4{0.f, 0.f, 0.f, 0.f},
-                                    f32x4{0.f, 0.f, 0.f, 0.f}, b4[k]);
-            }
-
-        const bool same_panel = has_next && nxt.rp == cur.rp;
-        if (same_panel)
-            TL_PRELOAD(nxt, bvec_n)
-
-        if constexpr (LN) {
-            // the workgroup holds whole rows: skip connection + LayerNorm here
-            TlLnOperands<NB, NW, NW> lnop;
-            tl_ln_fetch(lnop, a, wave, lane, cur.rp * TL_BM64, cur.N);
-            __syncthreads(); // every wave's part of the rows is staged
-            tl_ln_rows(lnop, a, stage0, wave, lane, cur.rp * TL_BM64, cur.Y, cur.N);
-            if (has_next && same_panel)
-                __syncthreads(); // the staging tiles are free again
-        } else {
-            // staging tile -> Y: 16-byte stores of 32*NB contiguous bytes per row
-            const int nvalid = min(NB, cur.nbr - cur.bn0); // the last column group may be partial
-            const int cpr = 2 * nvalid;                    // 16-byte chunks per row
-            const int m0 = cur.rp * TL_BM64;
-            f16 *ybase = cur.Y + (size_t)m0 * cur.N + cur.bn0 * 16;
-#pragma unroll
-            for (int t = 0; t < 2 * NB; t++) {
-                const int i = lane + 64 * t;
-                const int r = i / (2 * NB), c = i - r * (2 * NB);
-                if (c < cpr && m0 + r < a.M) {
-                    const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + r * lds + c * 8);
-                    *reinterpret_cast<u32x4 *>(ybase + (size_t)r * cur.N + c * 8) = v;
-                }
-            }
-        }
-#if 0
-        tlast = TL_TICK();
-        tepi += tlast - tb;
-#endif
-        if (!has_next)
-            break;
-        if (!same_panel) {
-            __syncthreads(); // every wave is done with the previous panel
-            TL_PANEL(nxt.rp)
-            TL_PRELOAD(nxt, bvec_n)
-        }
-        cur = nxt;
-        bvec = bvec_n;
-#pragma unroll
-        for (int k = 0; k < NB; k++)
-            b4[k] = b4n[k];
-    }
-#undef TL_PRELOAD
-#undef TL_PANEL
-#undef TL_BIAS
-#if 0
     if (g_trace && lane == 0) {
         unsigned hwid, xcc;
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
@@ -2026,11 +1823,12 @@ static int choose_nb(int nrp, int nbr_max, int nlin) {
     return 1;
 }
 
+constexpr int TL_BM64 = 2 * TL_BM;
 static int g_tile_bm64 = 1; // et_tuning_set("tile_bm64")
 
 template <bool GELU>
 static int launch_resident64(const TlArgs &a, size_t lds, hipStream_t st) {
-    auto k = tile_linear_resident64_kernel<3, GELU>;
+    auto k = tile_linear_resident_kernel<3, GELU, TL_WAVES, false, TL_BM64>;
     ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_THREADS), lds, st, a);
