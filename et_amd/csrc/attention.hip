@@ -374,9 +374,12 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
         // valid and the vector paths apply, so the body has no per-lane
         // predicates at all.
         bool has_mask_next = false;
-        auto tile_body = [&](int kb, const f16 *ks, const f16 *vt, auto fast_c, auto masked_c) {
-            constexpr bool FAST = decltype(fast_c)::value;
-            constexpr bool MASKED = decltype(masked_c)::value; // this tile's mask values are in mk
+        // (FAST and MASKED are wave-uniform run-time flags, not template
+        // parameters: four inlined copies of this body made the register
+        // allocator keep a second copy of every accumulator - 223 VGPRs against
+        // 122 for one copy - which halved the waves per SIMD)
+        auto tile_body = [&](int kb, const f16 *ks, const f16 *vt, const bool FAST, const bool MASKED) {
+            // MASKED: this tile's mask values are in mk
             // ---- scores, transposed: st[ksub][qs][r] = S[q = c16][key = 16 ksub + 4 g4 + r]
             f32x4 st[4][QS];
             if (!SHAREDQK) {
@@ -566,17 +569,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 else
                     load_tile(kb + AT_KT, no_t{});
             }
-            if (has_mask_cur) {
-                if (fast_tile(kb))
-                    tile_body(kb, ks, vt, yes_t{}, yes_t{});
-                else
-                    tile_body(kb, ks, vt, no_t{}, yes_t{});
-            } else {
-                if (fast_tile(kb))
-                    tile_body(kb, ks, vt, yes_t{}, no_t{});
-                else
-                    tile_body(kb, ks, vt, no_t{}, no_t{});
-            }
+            tile_body(kb, ks, vt, fast_tile(kb), has_mask_cur);
             has_mask_cur = has_mask_next;
             if (more) {
                 if (DMA)
