@@ -76,8 +76,12 @@ __device__ __forceinline__ float xor_max_16_32(float v) {
     return __builtin_bit_cast(float, z0);
 }
 
-template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK>
+// PLAIN: the launcher has established that there is no mask (or an all-zero
+// one), every sequence has full length and seq_len is a multiple of the
+// workgroup's query rows - no guards, no mask bookkeeping.
+template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK, bool PLAIN = false>
 __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attention_kernel(const AttnArgs a) {
+    static_assert(!PLAIN || (!PRUNED && !SHAREDQK), "the plain form exists for the on-the-fly kernel only");
     constexpr int AT_THREADS = NW * 64; // NW waves, each owning 16*QS query rows
     constexpr int AT_WAVES = NW;
     constexpr int DK = HD / 32;    // k-steps of Q K^T
@@ -362,7 +366,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
         };
         const bool vec_ok = (!a.mask || mask_vec) && (!SHAREDQK || qk_vec);
         auto fast_tile = [&](int kb) { return kb + AT_KT <= len && wave_rows_ok && vec_ok; };
-        bool has_mask_cur = a.mask && tile_has_mask(0);
+        bool has_mask_cur = !PLAIN && a.mask && tile_has_mask(0);
         if (has_mask_cur) {
             if (fast_tile(0))
                 load_mask(0, yes_t{});
@@ -446,7 +450,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                         for (int r = 0; r < 4; r++)
                             st[ksub][qs][r] += (float)mk[qs][ksub][r];
             }
-            if (a.mask) { // next tile's mask
+            if (!PLAIN && a.mask) { // next tile's mask
                 has_mask_next = kb + AT_KT < len && tile_has_mask((kb + AT_KT) / AT_KT);
                 if (has_mask_next) {
                     if (fast_tile(kb + AT_KT))
@@ -569,7 +573,10 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 else
                     load_tile(kb + AT_KT, no_t{});
             }
-            tile_body(kb, ks, vt, fast_tile(kb), has_mask_cur);
+            if constexpr (PLAIN)
+                tile_body(kb, ks, vt, true, false);
+            else
+                tile_body(kb, ks, vt, fast_tile(kb), has_mask_cur);
             has_mask_cur = has_mask_next;
             if (more) {
                 if (DMA)
@@ -689,10 +696,10 @@ template <int HD, int QS, int NW, bool PRUNED> constexpr size_t attn_lds_bytes()
     return sizeof(f16) * (size_t)(KV > O ? KV : O);
 }
 
-template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK>
+template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK, bool PLAIN = false>
 static void attn_launch_one(const AttnArgs &a, hipStream_t st) {
     constexpr size_t lds = attn_lds_bytes<HD, QS, NW, PRUNED>();
-    auto kern = attention_kernel<HD, QS, NW, PRUNED, SHAREDQK>;
+    auto kern = attention_kernel<HD, QS, NW, PRUNED, SHAREDQK, PLAIN>;
     if (lds > 64 * 1024) { // above the default dynamic-LDS limit: opt in once per kernel
         static bool done = false;
         if (!done) {
@@ -706,7 +713,18 @@ static void attn_launch_one(const AttnArgs &a, hipStream_t st) {
 
 // variant 0: 4 waves x 32 query rows; 1: 8 waves x 16 rows; 2: 4 waves x 16 rows
 template <int HD, bool PRUNED, bool SHAREDQK>
-static void attn_launch_variant(int variant, const AttnArgs &a, hipStream_t st) {
+static void attn_launch_variant(int variant, bool plain, const AttnArgs &a, hipStream_t st) {
+    if constexpr (!PRUNED && !SHAREDQK) {
+        if (plain) {
+            if (variant == 0)
+                attn_launch_one<HD, 2, 4, false, false, true>(a, st);
+            else if (variant == 1)
+                attn_launch_one<HD, 1, 8, false, false, true>(a, st);
+            else
+                attn_launch_one<HD, 1, 4, false, false, true>(a, st);
+            return;
+        }
+    }
     if (variant == 0)
         attn_launch_one<HD, 2, 4, PRUNED, SHAREDQK>(a, st);
     else if (variant == 1)
@@ -757,22 +775,25 @@ struct MaskSummaryEntry {
     const void *mask;
     const unsigned *summary;
     int seq_len;
+    bool all_zero; // no bit set: the mask adds nothing anywhere
 };
 static std::mutex g_msum_mutex;
 static std::vector<MaskSummaryEntry> g_msum;
 
-static void attach_mask_summary(AttnArgs &a) {
+// returns whether the mask is known to be zero everywhere
+static bool attach_mask_summary(AttnArgs &a) {
     a.msum = nullptr;
     a.msum_words = 0;
     if (!a.mask)
-        return;
+        return true;
     std::lock_guard<std::mutex> lock(g_msum_mutex);
     for (const MaskSummaryEntry &e : g_msum)
         if (e.mask == a.mask && e.seq_len == a.seq_len) {
             a.msum = e.summary;
             a.msum_words = mask_summary_words(a.seq_len);
-            return;
+            return e.all_zero;
         }
+    return false;
 }
 
 static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedqk,
@@ -793,7 +814,7 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
     }
     a.ldo = d_model;
     a.scale = head_scale(hd);
-    attach_mask_summary(a);
+    const bool no_mask = attach_mask_summary(a);
     // 128 query rows per workgroup when that still fills the chip, else 64
     int variant = 0;
     {
@@ -806,14 +827,15 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
             variant = g_attn_variant;
     }
     const int QB = variant == 2 ? 64 : 128;
+    const bool plain = no_mask && !a.seq_lens && !a.cu_seqlens && a.seq_len % QB == 0;
     a.nqb = (a.seq_len + QB - 1) / QB;
     a.total = a.nqb * a.nhead * a.batch;
     a.per_xcd = (a.total + 7) / 8;
 #define ET_ATTN_CASE(HDV)                                                                         \
     if (hd == HDV) {                                                                              \
-        if (sharedqk) attn_launch_variant<HDV, false, true>(variant, a, st);                                \
-        else if (pruned) attn_launch_variant<HDV, true, false>(variant, a, st);                             \
-        else attn_launch_variant<HDV, false, false>(variant, a, st);                                        \
+        if (sharedqk) attn_launch_variant<HDV, false, true>(variant, false, a, st);                     \
+        else if (pruned) attn_launch_variant<HDV, true, false>(variant, false, a, st);                  \
+        else attn_launch_variant<HDV, false, false>(variant, plain, a, st);                             \
     }
     ET_ATTN_CASE(32)
     ET_ATTN_CASE(64)
@@ -967,7 +989,17 @@ extern "C" int et_attention_mask_summary_attach(const void *mask, int seq_len, c
             g_msum.erase(g_msum.begin() + i);
             break;
         }
-    if (summary)
-        g_msum.push_back({mask, static_cast<const unsigned *>(summary), seq_len});
+    if (summary) {
+        // read the summary back once: an all-zero mask selects the kernels
+        // without any mask handling
+        const size_t words = (size_t)((seq_len + 15) / 16) * mask_summary_words(seq_len);
+        std::vector<unsigned> h(words);
+        ET_HIP(hipDeviceSynchronize());
+        ET_HIP(hipMemcpy(h.data(), summary, words * sizeof(unsigned), hipMemcpyDeviceToHost));
+        bool all_zero = true;
+        for (unsigned w : h)
+            all_zero = all_zero && w == 0;
+        g_msum.push_back({mask, static_cast<const unsigned *>(summary), seq_len, all_zero});
+    }
     return ET_OK;
 }
