@@ -442,13 +442,20 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
             // so after the first tiles the accumulator rescale is skipped.
             f16x8 pf[QS][2];
             if (MASKED) {
+                // (the multiplier is exactly 1.0 but opaque to the optimiser,
+                // which would otherwise turn the fused form back into a
+                // conversion and an add)
+                float one = 1.0f;
+                asm("" : "+s"(one));
 #pragma unroll
                 for (int qs = 0; qs < QS; qs++)
 #pragma unroll
                     for (int ksub = 0; ksub < 4; ksub++)
 #pragma unroll
                         for (int r = 0; r < 4; r++)
-                            st[ksub][qs][r] += (float)mk[qs][ksub][r];
+                            // (as a fused multiply-add by one: the mixed-precision
+                            // form takes the half operand directly, no conversion)
+                            st[ksub][qs][r] = __builtin_fmaf((float)mk[qs][ksub][r], one, st[ksub][qs][r]);
             }
             if (!PLAIN && a.mask) { // next tile's mask
                 has_mask_next = kb + AT_KT < len && tile_has_mask((kb + AT_KT) / AT_KT);
