@@ -16,13 +16,20 @@
 // subtiles; the X operand is gathered from LDS at the tile's column offset.
 // The product is formed transposed (D = W_tile * X^T) so that a lane ends up
 // with four consecutive output features of one row, which makes the
-// half-precision staging write 8 bytes wide.  Results are staged in LDS (the
-// X panel's storage is reused) and written with 16-byte row-contiguous
-// stores, because at >= 80 % sparsity this op is bound by the Y write.
+// half-precision staging write 8 bytes wide.  Results are staged in LDS and
+// written with 16-byte row-contiguous stores, because at >= 80 % sparsity a
+// linear on its own is bound by the Y write.
 // K larger than the LDS panel is walked in chunks of KC columns; plans sort
 // each block-row's tiles by column and carry a per-chunk CSR so a chunk only
-// touches its own tiles (TL_CSR); raw unsorted input with K > one panel falls
+// touches its own tiles (TL_PLAN); raw unsorted input with K > one panel falls
 // back to filtering the whole list per chunk (TL_FILTER).
+//
+// Kernels in this file: tile_linear_resident_kernel (K in one panel: persistent
+// workgroups, 32- or 64-row panels, optional LayerNorm epilogue),
+// tile_linear_plan_kernel (K in chunks), tile_linear_chunked_ln_kernel (K in
+// chunks + LayerNorm, double-buffered panels with a fetching wave),
+// tile_ffn_fused_kernel (feed-forward block / whole layer tail in one launch,
+// hidden activations in LDS), tile_linear_generic_kernel (raw and dense input).
 #include "common.h"
 
 #include <algorithm>
@@ -218,9 +225,10 @@ __device__ __forceinline__ void tl_epilogue_wave(const TlArgs &a, const TlCtx &x
 // contiguous run of tile pairs [q0, qend): 1 KB of W per pair at an address
 // linear in the pair index, plus one int per half-wave giving the LDS byte
 // offset of that tile's X columns.  The run is consumed through a TL_DEPTH-stage
-// register pipeline (stage = pair index mod TL_DEPTH), every load unconditional
-// with a clamped address, so TL_DEPTH pairs are always in flight per wave and
-// the waits are counted, not drained.  X operands are read from LDS one stage
+// register pipeline (stage = pair index mod TL_DEPTH) with unconditional loads
+// in the main loop, so TL_DEPTH pairs are always in flight per wave and the
+// waits are counted, not drained; only the last stages of a run test whether
+// there is still a pair to request.  X operands are read from LDS one stage
 // ahead.  Products accumulate into one running 32x16 accumulator; when the
 // stream crosses a block-row boundary (a scalar compare per pair) flush(j,
 // cur0, cur1) receives block-row j's finished sums.  All control flow in here
@@ -601,9 +609,9 @@ __device__ __forceinline__ void tl_ln_rows_at(const TlLnOperands<NB, NW, NLW> &o
 // a chunk is ONE contiguous stream of tile pairs: 1 KB of W per pair at an
 // address that is linear in the pair index, plus one int per half-wave giving
 // the LDS byte offset of that tile's X columns.  The stream is consumed
-// through a fixed 4-stage register pipeline (stage = pair index mod 4), every
-// load unconditional with a clamped address, so four pairs are always in
-// flight per wave and the waits are counted, not drained.  Products accumulate
+// through a fixed 4-stage register pipeline (stage = pair index mod 4, see
+// tl_stream), so four pairs are always in flight per wave and the waits are
+// counted, not drained.  Products accumulate
 // into one running 32x16 accumulator; when the stream crosses a block-row
 // boundary (a scalar compare per pair) it is added into that block-row's
 // static accumulator.
