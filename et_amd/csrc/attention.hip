@@ -108,11 +108,15 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
     f16 *smem = reinterpret_cast<f16 *>(at_smem);
     static_assert(SM * 2 <= 160 * 1024, "LDS budget");
 
-    const int pid = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3);
-    if (pid >= a.total)
+    // Workgroup ids go round-robin over the 8 XCDs.  XCD x works on the
+    // (batch, head) pairs x, x+8, x+16, ... in that order, all query blocks of a
+    // pair together (they share its K and V in that XCD's L2): with sequences of
+    // different lengths every XCD gets an even mix, and pairs keep their order.
+    const int xcd = blockIdx.x & 7, rest = blockIdx.x >> 3; // rest < per_xcd = ceil(pairs / 8) * nqb
+    const int qb = rest % a.nqb;
+    const int bh = (rest / a.nqb) * 8 + xcd;
+    if (bh >= a.nhead * a.batch)
         return;
-    const int qb = pid % a.nqb;
-    const int bh = pid / a.nqb;
     const int h = bh % a.nhead;
     const int b = bh / a.nhead;
 
@@ -837,7 +841,7 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
     const bool plain = no_mask && !a.seq_lens && !a.cu_seqlens && a.seq_len % QB == 0;
     a.nqb = (a.seq_len + QB - 1) / QB;
     a.total = a.nqb * a.nhead * a.batch;
-    a.per_xcd = (a.total + 7) / 8;
+    a.per_xcd = (a.nhead * a.batch + 7) / 8 * a.nqb;
 #define ET_ATTN_CASE(HDV)                                                                         \
     if (hd == HDV) {                                                                              \
         if (sharedqk) attn_launch_variant<HDV, false, true>(variant, false, a, st);                     \
