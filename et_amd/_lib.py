@@ -58,6 +58,8 @@ PROTOTYPES = {
     "et_head_ptr": (_i, [_ip, _i, _i, _i, _ip]),
     "et_pack_rows": (_i, [_vp, _vp, _ip, _i, _i, _i, _vp]),
     "et_unpack_rows": (_i, [_vp, _vp, _ip, _i, _i, _i, _vp]),
+    "et_pack_rows_ordered": (_i, [_vp, _vp, _ip, _ip, _i, _i, _i, _vp]),
+    "et_unpack_rows_ordered": (_i, [_vp, _vp, _ip, _ip, _i, _i, _i, _vp]),
     "et_scatter_cols": (_i, [_vp, _vp, _ip, _i, _i, _i, _i, _vp]),
     # include/et_encoder.h
     "et_linear_tile_create": (_i, [C.POINTER(_vp), _i, _i, _i, _i, _vp, _ip, _ip, _vp, _i]),

@@ -25,9 +25,11 @@ int hip_fail(hipError_t e, const char *what) {
 // one workgroup per (sequence, position), 16-byte copies
 __global__ void __launch_bounds__(128)
 pack_rows_kernel(f16 *__restrict__ packed, const f16 *__restrict__ padded,
-                 const int *__restrict__ cu, int seq_len, int width) {
-    const int b = blockIdx.y, t = blockIdx.x;
-    const int start = cu[b], len = cu[b + 1] - start;
+                 const int *__restrict__ cu, const int *__restrict__ order, int seq_len, int width) {
+    // packed sequence i is padded sequence order[i] (order == null: i itself)
+    const int i = blockIdx.y, t = blockIdx.x;
+    const int b = order ? order[i] : i;
+    const int start = cu[i], len = cu[i + 1] - start;
     if (t >= len)
         return;
     const int nch = width >> 3;
@@ -39,9 +41,10 @@ pack_rows_kernel(f16 *__restrict__ packed, const f16 *__restrict__ padded,
 
 __global__ void __launch_bounds__(128)
 unpack_rows_kernel(f16 *__restrict__ padded, const f16 *__restrict__ packed,
-                   const int *__restrict__ cu, int seq_len, int width) {
-    const int b = blockIdx.y, t = blockIdx.x;
-    const int start = cu[b], len = cu[b + 1] - start;
+                   const int *__restrict__ cu, const int *__restrict__ order, int seq_len, int width) {
+    const int i = blockIdx.y, t = blockIdx.x;
+    const int b = order ? order[i] : i;
+    const int start = cu[i], len = cu[i + 1] - start;
     const int nch = width >> 3;
     u32x4 *dst = reinterpret_cast<u32x4 *>(padded + ((size_t)b * seq_len + t) * width);
     const u32x4 *src = reinterpret_cast<const u32x4 *>(packed + (size_t)(start + t) * width);
@@ -195,25 +198,35 @@ static int pack_check(const void *packed, const void *padded, const int *cu, int
 
 int et_pack_rows(void *packed, const void *padded, const int *cu_seqlens, int batch, int seq_len,
                  int width, void *stream) {
+    return et_pack_rows_ordered(packed, padded, cu_seqlens, nullptr, batch, seq_len, width, stream);
+}
+
+int et_unpack_rows(void *padded, const void *packed, const int *cu_seqlens, int batch, int seq_len,
+                   int width, void *stream) {
+    return et_unpack_rows_ordered(padded, packed, cu_seqlens, nullptr, batch, seq_len, width, stream);
+}
+
+int et_pack_rows_ordered(void *packed, const void *padded, const int *cu_seqlens, const int *order,
+                         int batch, int seq_len, int width, void *stream) {
     using namespace et;
     const int rc = pack_check(packed, padded, cu_seqlens, batch, seq_len, width, "et_pack_rows");
     if (rc != ET_OK)
         return rc;
     hipLaunchKernelGGL(pack_rows_kernel, dim3(seq_len, batch), dim3(128), 0,
                        static_cast<hipStream_t>(stream), static_cast<f16 *>(packed),
-                       static_cast<const f16 *>(padded), cu_seqlens, seq_len, width);
+                       static_cast<const f16 *>(padded), cu_seqlens, order, seq_len, width);
     return launch_status("et_pack_rows");
 }
 
-int et_unpack_rows(void *padded, const void *packed, const int *cu_seqlens, int batch, int seq_len,
-                   int width, void *stream) {
+int et_unpack_rows_ordered(void *padded, const void *packed, const int *cu_seqlens, const int *order,
+                           int batch, int seq_len, int width, void *stream) {
     using namespace et;
     const int rc = pack_check(packed, padded, cu_seqlens, batch, seq_len, width, "et_unpack_rows");
     if (rc != ET_OK)
         return rc;
     hipLaunchKernelGGL(unpack_rows_kernel, dim3(seq_len, batch), dim3(128), 0,
                        static_cast<hipStream_t>(stream), static_cast<f16 *>(padded),
-                       static_cast<const f16 *>(packed), cu_seqlens, seq_len, width);
+                       static_cast<const f16 *>(packed), cu_seqlens, order, seq_len, width);
     return launch_status("et_unpack_rows");
 }
 

@@ -32,7 +32,8 @@ class Encoder_base {
     // per-sequence lengths (optional)
     std::vector<int> lens;
     Weight<int> d_lens;
-    Weight<int> d_cu;
+    Weight<int> d_cu;    // row offsets of the packed sequences
+    Weight<int> d_order; // packed position -> batch index
     int total_rows; // sum of lengths when set, else batch*seq_len
 
     int rows() const { return batch * seq_len; }
@@ -81,15 +82,25 @@ class Encoder_base {
         if (!host_lens)
             return;
         lens.assign(host_lens, host_lens + batch);
-        std::vector<int> cu(batch + 1, 0);
+        // packed layout: longest sequence first (ties in batch order), so the
+        // attention kernel, which starts workgroups in packed order, ends with
+        // the short ones
+        std::vector<int> order(batch);
         for (int b = 0; b < batch; b++)
-            cu[b + 1] = cu[b] + lens[b];
+            order[b] = b;
+        std::stable_sort(order.begin(), order.end(), [this](int x, int y) { return lens[x] > lens[y]; });
+        std::vector<int> cu(batch + 1, 0);
+        for (int i = 0; i < batch; i++)
+            cu[i + 1] = cu[i] + lens[order[i]];
         total_rows = cu[batch];
         d_lens = Weight<int>(lens.data(), batch);
         d_cu = Weight<int>(cu.data(), batch + 1);
+        d_order = Weight<int>(order.data(), batch);
     }
     int valid_rows() const { return total_rows; }
+    // packed sequence i is rows cu[i]..cu[i+1]-1 and is batch entry order[i]
     const int *device_cu_seqlens() const { return lens.empty() ? nullptr : d_cu.get(); }
+    const int *device_pack_order() const { return lens.empty() ? nullptr : d_order.get(); }
 
   protected:
     half *mask_ptr() const { return has_mask ? mask.get() : nullptr; }
@@ -258,7 +269,8 @@ class Encoder_length : public Encoder_base {
     }
 
     // One layer on packed rows: in_p/out_p are [valid_rows() x d_model] with
-    // sequence b at rows cu[b]..cu[b+1]-1; out_p may alias in_p.
+    // packed sequence i (batch entry device_pack_order()[i]) at rows
+    // cu[i]..cu[i+1]-1; out_p may alias in_p.
     void run_packed(half *out_p, half *in_p) {
         const int n = total_rows;
         const Linear_tile *qkv[3] = {&Q_linear, &K_linear, &V_linear};
@@ -277,7 +289,7 @@ class Encoder_length : public Encoder_base {
             // unit 0, from where it is expanded into `out`.
             const int n = total_rows;
             half *in_p = buffers[4];
-            etChk(et_pack_rows(in_p, in, d_cu.get(), batch, seq_len, d_model, stream));
+            etChk(et_pack_rows_ordered(in_p, in, d_cu.get(), d_order.get(), batch, seq_len, d_model, stream));
             const Linear_tile *qkv[3] = {&Q_linear, &K_linear, &V_linear};
             half *outs[3] = {buffers[0], buffers[1], buffers[2]};
             Linear_tile::run_multi(qkv, outs, 3, in_p, n, stream);
@@ -291,7 +303,7 @@ class Encoder_length : public Encoder_base {
                 Linear_tile::run_rows_tail(O_linear, MLP1_linear, MLP2_linear, buffers[0], buffers[3], in_p,
                                            buffers[0], buffers[1], ln_gamma[0].get(), ln_beta[0].get(),
                                            ln_gamma[1].get(), ln_beta[1].get(), n, stream);
-                etChk(et_unpack_rows(out, buffers[0], d_cu.get(), batch, seq_len, d_model, stream));
+                etChk(et_unpack_rows_ordered(out, buffers[0], d_cu.get(), d_order.get(), batch, seq_len, d_model, stream));
                 return;
             }
             O_linear.run_rows_ln(buffers[0], buffers[3], in_p, ln_gamma[0].get(), ln_beta[0].get(), n, stream);
@@ -309,7 +321,7 @@ class Encoder_length : public Encoder_base {
                 MLP2_linear.run_rows(out, buffers[1], n, stream);
                 etChk(et_skip_layernorm(buffers[0], out, ln_gamma[1].get(), ln_beta[1].get(), n, d_model, stream));
             }
-            etChk(et_unpack_rows(out, buffers[0], d_cu.get(), batch, seq_len, d_model, stream));
+            etChk(et_unpack_rows_ordered(out, buffers[0], d_cu.get(), d_order.get(), batch, seq_len, d_model, stream));
             return;
         }
         const Linear_tile *qkv[3] = {&Q_linear, &K_linear, &V_linear};
@@ -353,9 +365,10 @@ class Encoder_stack {
             }
             return;
         }
-        etChk(et_pack_rows(act, in, cu, batch, seq_len, d_model, stream));
+        const int *order = layers[0]->device_pack_order();
+        etChk(et_pack_rows_ordered(act, in, cu, order, batch, seq_len, d_model, stream));
         for (Encoder_length *l : layers)
             l->run_packed(act, act);
-        etChk(et_unpack_rows(out, act, cu, batch, seq_len, d_model, stream));
+        etChk(et_unpack_rows_ordered(out, act, cu, order, batch, seq_len, d_model, stream));
     }
 };

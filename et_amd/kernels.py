@@ -104,19 +104,22 @@ def sharedQK_attention(QK, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2
     return Z
 
 
-def pack_rows(padded, cu_seqlens, seq_len, total_rows):
+def pack_rows(padded, cu_seqlens, seq_len, total_rows, order=None):
+    """order (int32 device tensor, optional): packed sequence i is padded sequence order[i]."""
     width = padded.shape[1]
     batch = cu_seqlens.numel() - 1
     packed = torch.empty((total_rows, width), dtype=torch.float16, device=padded.device)
-    check(lib().et_pack_rows(_h(packed), _h(padded), _i32(cu_seqlens), batch, seq_len, width, _stream()))
+    check(lib().et_pack_rows_ordered(_h(packed), _h(padded), _i32(cu_seqlens), _i32(order), batch, seq_len,
+                                     width, _stream()))
     return packed
 
 
-def unpack_rows(packed, cu_seqlens, seq_len):
+def unpack_rows(packed, cu_seqlens, seq_len, order=None):
     width = packed.shape[1]
     batch = cu_seqlens.numel() - 1
     padded = torch.empty((batch * seq_len, width), dtype=torch.float16, device=packed.device)
-    check(lib().et_unpack_rows(_h(padded), _h(packed), _i32(cu_seqlens), batch, seq_len, width, _stream()))
+    check(lib().et_unpack_rows_ordered(_h(padded), _h(packed), _i32(cu_seqlens), _i32(order), batch, seq_len,
+                                       width, _stream()))
     return padded
 
 

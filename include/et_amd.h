@@ -291,6 +291,17 @@ int et_pack_rows(void *packed, const void *padded, const int *cu_seqlens,
 /* inverse; padding rows of `padded` are written as zero */
 int et_unpack_rows(void *padded, const void *packed, const int *cu_seqlens,
                    int batch, int seq_len, int width, void *stream);
+/* The same with the packed sequences in another order: packed sequence i
+ * (rows cu_seqlens[i] .. cu_seqlens[i+1]) is padded sequence order[i]; order
+ * is a device array holding a permutation of 0..batch-1, NULL = identity.
+ * Packing longest first makes the attention kernel, which dispatches packed
+ * sequences in index order, start the longest ones first. */
+int et_pack_rows_ordered(void *packed, const void *padded,
+                         const int *cu_seqlens, const int *order, int batch,
+                         int seq_len, int width, void *stream);
+int et_unpack_rows_ordered(void *padded, const void *packed,
+                           const int *cu_seqlens, const int *order, int batch,
+                           int seq_len, int width, void *stream);
 /* out[r][col_id[j]] = in[r][j] for j < n, every other column of out[rows x
  * width] zero: expands a row_mat linear's compact output
  * (kernels/linear.cu:30-32) back to model width. */

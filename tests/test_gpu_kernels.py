@@ -522,6 +522,14 @@ def test_pack_unpack_scatter(K):
     want = np.zeros_like(x)
     want[sel] = x[sel]
     assert np.array_equal(back, want)
+    # longest first: packed sequence i is padded sequence order[i]
+    order = np.argsort(-lens, kind="stable").astype(np.int32)
+    cu_o = np.concatenate([[0], np.cumsum(lens[order])]).astype(np.int32)
+    sel_o = np.concatenate([np.arange(b * S, b * S + lens[b]) for b in order]).astype(np.int64)
+    packed_o = host(K.pack_rows(dev(x), dev(cu_o), S, int(cu_o[-1]), order=dev(order)))
+    assert np.array_equal(packed_o, x[sel_o])
+    back_o = host(K.unpack_rows(dev(packed_o), dev(cu_o), S, order=dev(order)))
+    assert np.array_equal(back_o, want)
     ids = np.sort(r.choice(d, 230, replace=False)).astype(np.int32)
     comp = randn_h(r, (50, 240))
     sc = host(K.scatter_cols(dev(comp), dev(ids), d))
