@@ -265,6 +265,19 @@ def run_extras(torch, orc, K, dev):
         torch.cuda.synchronize()
         return a.elapsed_time(b) / reps * 1e3  # us
 
+    def timeit_graph(fn, reps=100, warm=3):
+        """the same calls captured once in a HIP graph and replayed (no per-kernel launch work on the host)"""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            fn()
+        return timeit(graph.replay, reps=reps, warm=warm)
+
     # config 2: tile linear 4096x768 -> 3072 at 0/50/80/90 %
     r = rng(7)
     M, N, Kd = 4096, 3072, 768
@@ -292,7 +305,9 @@ def run_extras(torch, orc, K, dev):
     enc = Encoder_tile(D, S, H, ws, *L, *ln, np.zeros((S, S), np.float16), B)
     o = torch.empty_like(x)
     us = timeit(lambda: enc.run(o, x))
-    out["config1_dense_layer_b1_s128"] = {"us": round(us, 2), "seqs_per_s": round(1e6 / us, 1)}
+    us_g = timeit_graph(lambda: enc.run(o, x))
+    out["config1_dense_layer_b1_s128"] = {"us": round(us, 2), "seqs_per_s": round(1e6 / us, 1),
+                                          "us_as_hip_graph": round(us_g, 2)}
 
     # config 4: attention-aware pruned layer, batch 32 x seq 256 (Q/K keep 32 of 64 columns per head,
     # O/FFN1/FFN2 row-pruned at 70 %)
@@ -341,6 +356,8 @@ def run_extras(torch, orc, K, dev):
             l.set_seq_lens(ll)
         us = timeit(lambda: stack.run(o, x), reps=10, warm=3)
         res5[name] = {"us_12_layers": round(us, 1), "seqs_per_s": round(B * 1e6 / us, 1)}
+        if ll is not None:
+            res5[name]["us_12_layers_as_hip_graph"] = round(timeit_graph(lambda: stack.run(o, x), reps=10), 1)
     res5["padding_skip_speedup"] = round(res5["padded"]["us_12_layers"] / res5["length_aware"]["us_12_layers"], 3)
     out["config5_length_aware_12_layer_stack_b64"] = res5
     return out

@@ -277,3 +277,44 @@ def test_encoder_stack_variable_length():
     for lins, ln in params:
         cur = orc.encoder_tile_layer(cur, lins, ln, None, S, H, B, None, 1.0)
     check_close(got_full, cur, what="stack full length")
+
+
+def test_encoder_runs_inside_a_captured_hip_graph():
+    """run() allocates nothing, never synchronises and issues only kernel launches on the caller's
+    stream, so a caller can capture it in a HIP graph: every replay equals the eager result."""
+    from et_amd.encoder import Encoder_length, Encoder_stack, Encoder_tile
+    r = rng(810)
+    d, H, dff, S, B, NL = 256, 4, 1024, 128, 4, 2
+    lens = np.array([128, 9, 77, 50], np.int32)
+    layers = []
+    for i in range(NL):
+        lins, ln = make_layer(r, d, dff, 0.5, seed=960 + 10 * i, std=0.05)
+        layers.append(Encoder_length(d, S, H, workspace(Encoder_length, d, S, H, B), *build_linears(lins, B * S), *ln, None, B))
+    stack = Encoder_stack(layers, d, S, B)
+    stack.set_seq_lens(lens)
+    lins, ln = make_layer(r, d, dff, 0.8, seed=990, std=0.05)
+    mask = randn_h(r, (S, S), 0.5)
+    tile = Encoder_tile(d, S, H, workspace(Encoder_tile, d, S, H, B), *build_linears(lins, B * S), *ln, mask, B)
+    inputs = [dev(randn_h(r, (B * S, d))) for _ in range(3)]
+    for name, run in (("stack, packed rows", stack.run), ("Encoder_tile", tile.run)):
+        eager = [host(run(torch.empty_like(x), x)) for x in inputs]
+        x_static, out_static = torch.empty_like(inputs[0]), torch.empty_like(inputs[0])
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):   # warm-up on the capture stream
+            x_static.copy_(inputs[0])
+            run(out_static, x_static)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            run(out_static, x_static)
+        for k in (1, 2, 0, 2):          # eager work and synchronisations between the replays
+            x_static.copy_(inputs[k])
+            out_static.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert np.array_equal(host(out_static), eager[k]), f"{name}: replay with input {k}"
+            again = host(run(torch.empty_like(inputs[k]), inputs[k]))
+            assert np.array_equal(again, eager[k])
+        del graph
