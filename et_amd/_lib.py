@@ -61,6 +61,7 @@ PROTOTYPES = {
     "et_pack_rows_ordered": (_i, [_vp, _vp, _ip, _ip, _i, _i, _i, _vp]),
     "et_unpack_rows_ordered": (_i, [_vp, _vp, _ip, _ip, _i, _i, _i, _vp]),
     "et_scatter_cols": (_i, [_vp, _vp, _ip, _i, _i, _i, _i, _vp]),
+    "et_scatter_skip_layernorm": (_i, [_vp, _vp, _ip, _i, _i, _vp, _vp, _vp, _i, _i, _vp]),
     # include/et_encoder.h
     "et_linear_tile_create": (_i, [C.POINTER(_vp), _i, _i, _i, _i, _vp, _ip, _ip, _vp, _i]),
     "et_linear_tile_destroy": (None, [_vp]),

@@ -116,6 +116,102 @@ skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip
     }
 }
 
+// The same for a compact operand: a[r][col_id[j]] = compact[r][j] for j < n,
+// every other column of a zero (the output of a row-pruned linear,
+// kernels/linear.cu:30-32, expanded to model width), out = LayerNorm(a + skip).
+// One wave per row: the wave builds the expanded row in its own LDS strip
+// (zero fill, then 2-byte scattered writes), reads it back in the chunk layout
+// of the kernel above and goes on with the same arithmetic.
+template <int NCH>
+__global__ void __launch_bounds__(256)
+scatter_skip_layernorm_kernel(f16 *__restrict__ out, const f16 *__restrict__ compact,
+                              const int *__restrict__ col_id, int n, int ld_in,
+                              const f16 *skip, const f16 *__restrict__ gamma,
+                              const f16 *__restrict__ beta, int num, int size, float inv_n) {
+    typedef f16x8 vec;
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    extern __shared__ __attribute__((aligned(16))) unsigned char ln_smem[];
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const long row = (long)blockIdx.x * 4 + wave;
+    if (row >= num)
+        return;
+    f16 *strip = reinterpret_cast<f16 *>(ln_smem) + wave * size;
+    const int nchunk = size >> 3;
+    const bool last_ok = lane + (NCH - 1) * 64 < nchunk;
+    int ci[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; i++)
+        ci[i] = i == NCH - 1 ? min(lane + i * 64, nchunk - 1) : lane + i * 64;
+    const vec zero = vec{0, 0, 0, 0, 0, 0, 0, 0};
+    float one = 1.0f;
+    asm("" : "+s"(one));
+
+    vec sn[NCH], gg[NCH], bb[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; i++)
+        sn[i] = reinterpret_cast<const vec *>(skip + row * size)[ci[i]];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        gg[i] = reinterpret_cast<const vec *>(gamma)[ci[i]];
+        bb[i] = reinterpret_cast<const vec *>(beta)[ci[i]];
+    }
+#pragma unroll
+    for (int i = 0; i < NCH; i++)
+        if (i < NCH - 1 || last_ok)
+            reinterpret_cast<vec *>(strip)[ci[i]] = zero;
+    // (LDS operations of one wave execute in order; the fences keep the compiler
+    // from reordering the strip's writes and reads, which touch other lanes' data)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    for (int j0 = lane * 8; j0 < n; j0 += 64 * 8) { // eight compact values per lane and step
+        const vec v = *reinterpret_cast<const vec *>(compact + row * ld_in + j0);
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int c = col_id[min(j0 + k, n - 1)];
+            if (j0 + k < n)
+                strip[c] = v[k];
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+
+    vec x[NCH];
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        x[i] = reinterpret_cast<const vec *>(strip)[ci[i]] + sn[i]; // half add, one rounding
+        if (i == NCH - 1)
+            x[i] = last_ok ? x[i] : zero;
+#pragma unroll
+        for (int j = 0; j < 8; j += 2)
+            sum = __builtin_amdgcn_fdot2(h2{x[i][j], x[i][j + 1]}, h2{(f16)1, (f16)1}, sum, false);
+    }
+    const float mean = wave_sum(sum) * inv_n;
+    const float neg_mean = -mean;
+    float var = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        if (i < NCH - 1 || last_ok) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float d = __builtin_fmaf((float)x[i][j], one, neg_mean);
+                var += d * d;
+            }
+        }
+    }
+    const float rstd = rsqrtf(wave_sum(var) * inv_n + 1e-6f);
+    const float shift = -mean * rstd;
+    vec *a = reinterpret_cast<vec *>(out + row * size);
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        vec y;
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            y[j] = (f16)(__builtin_fmaf((float)x[i][j], rstd, shift) * (float)gg[i][j] + (float)bb[i][j]);
+        if (i < NCH - 1 || last_ok)
+            a[ci[i]] = y;
+    }
+}
+
 // Any size, any alignment: one wave per row, three passes over memory.
 __global__ void __launch_bounds__(256)
 skip_layernorm_generic_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip,
@@ -199,4 +295,47 @@ extern "C" int et_skip_layernorm(void *in_out, const void *skip, const void *gam
 #undef ET_LN_CASE
     }
     return launch_status("et_skip_layernorm launch");
+}
+
+extern "C" int et_scatter_skip_layernorm(void *out, const void *compact, const int *col_id, int n,
+                                         int ld_in, const void *skip, const void *gamma,
+                                         const void *beta, int num, int size, void *stream) {
+    using namespace et;
+    ET_REQUIRE(out && compact && col_id && skip && gamma && beta, ET_ERR_INVALID_ARG,
+               "et_scatter_skip_layernorm: null pointer");
+    ET_REQUIRE(num >= 0 && size > 0 && n >= 0 && n <= ld_in && n <= size, ET_ERR_INVALID_ARG,
+               "et_scatter_skip_layernorm: num=%d size=%d n=%d ld_in=%d", num, size, n, ld_in);
+    ET_REQUIRE(out != compact, ET_ERR_INVALID_ARG, "et_scatter_skip_layernorm: out must not alias compact");
+    if (num == 0)
+        return ET_OK;
+    const bool vec = size % 8 == 0 && size <= 4096 && ld_in % 8 == 0 && n > 0 && aligned16(out) &&
+                     aligned16(compact) && aligned16(skip) && aligned16(gamma) && aligned16(beta);
+    if (!vec) { // the two steps, one after the other
+        ET_REQUIRE(out != skip, ET_ERR_INVALID_ARG,
+                   "et_scatter_skip_layernorm: out must not alias skip for these sizes");
+        const int rc = et_scatter_cols(out, compact, col_id, num, n, ld_in, size, stream);
+        return rc != ET_OK ? rc : et_skip_layernorm(out, skip, gamma, beta, num, size, stream);
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid((num + 3) / 4), block(256);
+    const size_t lds = (size_t)4 * size * sizeof(f16);
+    const float inv_n = 1.0f / (float)size;
+#define ET_SLN_CASE(NCH_)                                                                         \
+    hipLaunchKernelGGL((scatter_skip_layernorm_kernel<NCH_>), grid, block, lds, st,               \
+                       static_cast<f16 *>(out), static_cast<const f16 *>(compact), col_id, n, ld_in, \
+                       static_cast<const f16 *>(skip), static_cast<const f16 *>(gamma),           \
+                       static_cast<const f16 *>(beta), num, size, inv_n);                         \
+    break;
+    switch ((size / 8 + 63) / 64) {
+    case 1: ET_SLN_CASE(1)
+    case 2: ET_SLN_CASE(2)
+    case 3: ET_SLN_CASE(3)
+    case 4: ET_SLN_CASE(4)
+    case 5: ET_SLN_CASE(5)
+    case 6: ET_SLN_CASE(6)
+    case 7: ET_SLN_CASE(7)
+    default: ET_SLN_CASE(8)
+    }
+#undef ET_SLN_CASE
+    return launch_status("et_scatter_skip_layernorm launch");
 }

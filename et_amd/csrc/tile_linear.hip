@@ -1875,7 +1875,7 @@ static int tile_launch(const TlProblem *probs, int nlin, const f16 *X, int M, in
         const int nrp64 = (M + TL_BM64 - 1) / TL_BM64;
         const int ncg64 = (nbr_max + TL_WAVES * 3 - 1) / (TL_WAVES * 3);
         const long items = (long)nrp64 * ncg64 * nlin;
-        if (lds64 <= 160 * 1024 && items >= 2L * cus) {
+        if (lds64 <= 160 * 1024 && items >= (g_tile_bm64 >= 2 ? 1L : 2L * cus)) {
             a.ncg = ncg64;
             a.total = (int)items;
             const int per_rp = ncg64 * nlin;

@@ -92,6 +92,7 @@ class Linear_tile {
         }
         etChk(et_tile_plan_run_multi(plans, ys, n, in, rows, stream));
     }
+    const et_tile_plan *tile_plan() const { return plan; } // for et_tile_plan_run_multi with other plans
     int rows() const { return size; }
     int in_features() const { return in_feat; }
     int out_features() const { return out_feat; }
@@ -174,5 +175,11 @@ class Linear_row {
     // out[rows x out_feat] = the compact result expanded to model width, pruned columns zero
     void scatter(half *out, const half *compact, int rows, void *stream) const {
         etChk(et_scatter_cols(out, compact, row_id.get(), rows, row_id_size, nrow, out_feat, stream));
+    }
+    // out = LayerNorm(scatter(compact) + skip) in one launch; out may alias skip
+    void scatter_skip_layernorm(half *out, const half *compact, const half *skip, const half *gamma,
+                                const half *beta, int rows, void *stream) const {
+        etChk(et_scatter_skip_layernorm(out, compact, row_id.get(), row_id_size, nrow, skip, gamma, beta, rows,
+                                        out_feat, stream));
     }
 };

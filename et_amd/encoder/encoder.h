@@ -6,6 +6,7 @@
 // run() (the reference blocks the host three times per layer,
 // encoder/encoder.cu:27-29), Q/K/V projected by one launch.
 #pragma once
+#include <algorithm>
 #include <vector>
 
 #include "Linear.h"
@@ -218,19 +219,27 @@ class Encoder_attnaware : public Encoder_base {
     }
     void run(half *out, half *in) override {
         const int n = rows();
-        Q_linear.run_rows(buffers[0], in, n, stream); // compact [n x nrow]
-        K_linear.run_rows(buffers[1], in, n, stream);
-        V_linear.run_rows(buffers[2], in, n, stream);
+        if (Q_linear.plan && K_linear.plan && Q_linear.in_feat == V_linear.in_features() &&
+            K_linear.in_feat == V_linear.in_features()) {
+            // one launch for the three projections (Q and K compact [n x nrow])
+            const et_tile_plan *plans[3] = {Q_linear.plan, K_linear.plan, V_linear.tile_plan()};
+            void *ys[3] = {buffers[0], buffers[1], buffers[2]};
+            etChk(et_tile_plan_run_multi(plans, ys, 3, in, n, stream));
+        } else {
+            Q_linear.run_rows(buffers[0], in, n, stream); // compact [n x nrow]
+            K_linear.run_rows(buffers[1], in, n, stream);
+            V_linear.run_rows(buffers[2], in, n, stream);
+        }
         etChk(et_Prune_attention(buffers[3], buffers[0], buffers[1], buffers[2], Q_linear.head_ptr.get(),
                                  Q_linear.nrow, nullptr, nullptr, d_model, mask_ptr(), seq_len, d_model,
                                  nheads, batch, lens_ptr(), log2_scale, stream));
         O_linear.run_rows(buffers[0], buffers[3], n, stream);
-        O_linear.scatter(buffers[1], buffers[0], n, stream);
-        etChk(et_skip_layernorm(buffers[1], in, ln_gamma[0].get(), ln_beta[0].get(), n, d_model, stream));
+        // expansion to model width, skip connection and LayerNorm in one launch
+        O_linear.scatter_skip_layernorm(buffers[1], buffers[0], in, ln_gamma[0].get(), ln_beta[0].get(), n, stream);
         MLP1_linear.run_rows(buffers[2], buffers[1], n, stream); // compact hidden, spans units 2..4
         MLP2_linear.run_rows(buffers[0], buffers[2], n, stream);
-        MLP2_linear.scatter(out, buffers[0], n, stream);
-        etChk(et_skip_layernorm(out, buffers[1], ln_gamma[1].get(), ln_beta[1].get(), n, d_model, stream));
+        MLP2_linear.scatter_skip_layernorm(out, buffers[0], buffers[1], ln_gamma[1].get(), ln_beta[1].get(), n,
+                                           stream);
     }
 };
 

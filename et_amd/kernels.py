@@ -130,6 +130,16 @@ def scatter_cols(x, col_id, width):
     return out
 
 
+def scatter_skip_layernorm(compact, col_id, skip, gamma, beta, out=None):
+    """LayerNorm(expand(compact) + skip): compact[rows x ld] holds columns col_id of a [rows x width] matrix"""
+    rows, ld = compact.shape
+    width = skip.shape[1]
+    out = torch.empty_like(skip) if out is None else out
+    check(lib().et_scatter_skip_layernorm(_h(out), _h(compact), _i32(col_id), col_id.numel(), ld, _h(skip),
+                                          _h(gamma), _h(beta), rows, width, _stream()))
+    return out
+
+
 def attention_mask_summary(mask, seq_len):
     """Per-(16 rows x 64 keys) non-zero bits of an additive mask; attach() lets the
     attention launchers skip the all-zero tiles of that mask tensor."""

@@ -307,6 +307,14 @@ int et_unpack_rows_ordered(void *padded, const void *packed,
  * (kernels/linear.cu:30-32) back to model width. */
 int et_scatter_cols(void *out, const void *in, const int *col_id, int rows,
                     int n, int ld_in, int width, void *stream);
+/* et_scatter_cols followed by et_skip_layernorm (kernels/kernels.h:3-5) in
+ * one launch: out[num x size] = LayerNorm(expand(compact) + skip), the
+ * expanded rows never written to memory.  out may alias skip, not compact. */
+int et_scatter_skip_layernorm(void *out, const void *compact,
+                              const int *col_id, int n, int ld_in,
+                              const void *skip, const void *gamma,
+                              const void *beta, int num, int size,
+                              void *stream);
 
 /* ------------------------------------------------------------------------
  * Device memory / stream plumbing so that host code above this ABI needs no

@@ -329,6 +329,26 @@ def test_tile_linear_multi_qkv_one_launch(K):
         check_close(host(o), want, max_abs=2e-3, mean_rel=5e-4, what="qkv multi")
 
 
+@pytest.mark.parametrize("M", [200, 5700])
+def test_tile_linear_multi_unequal_widths(K, M):
+    """Q and K narrower than V (attention-aware pruning): linears of different widths in one launch,
+    with column groups that exist for the widest one only (M = 5700 takes the 64-row kernel)"""
+    from et_amd.encoder import Linear_tile, run_multi
+    r = rng(33 + M)
+    d = 768
+    widths = (384, 384, 768)
+    lins = [make_tile_linear(r, n, d, sp, seed=60 + j, std=0.05, bias_std=0.1) for j, (n, sp) in enumerate(zip(widths, (0.0, 0.5, 0.5)))]
+    X = randn_h(r, (M, d))
+    lts = [Linear_tile(d, l["N"], M, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"]) for l in lins]
+    outs = [host(o) for o in run_multi(lts, dev(X))]
+    rows = np.unique(np.concatenate([np.arange(0, 70), r.integers(0, M, 130), np.arange(M - 70, M)]))
+    for l, lt, o in zip(lins, lts, outs):
+        assert o.shape == (M, l["N"])
+        want = orc.tile_linear(X[rows], l["row_ptr"], l["row_offset"], l["data"], l["bias"], l["N"], f64=True)
+        check_close(o[rows], want, max_abs=2e-3, mean_rel=5e-4, what="multi, unequal widths")
+        assert np.array_equal(o, host(lt.run(dev(X))))   # the same linear launched alone
+
+
 def test_tile_linear_full_size_config2_rows_sample(K):
     """config-2 shape (4096x768 -> 3072, 80 %): rows are independent, so a row sample pins the full-size launch"""
     r = rng(32)
@@ -536,3 +556,24 @@ def test_pack_unpack_scatter(K):
     want = np.zeros((50, d), np.float16)
     want[:, ids] = comp[:, :230]
     assert np.array_equal(sc, want)
+
+
+@pytest.mark.parametrize("rows,d,n,ld", [(50, 768, 230, 240), (131, 768, 768, 768), (7, 256, 1, 16),
+                                          (33, 1536, 921, 928), (20, 1000, 300, 304), (9, 772, 100, 100)])
+def test_scatter_skip_layernorm_one_launch(K, rows, d, n, ld):
+    """LayerNorm(expand(compact) + skip) == et_scatter_cols then et_skip_layernorm, bit for bit, and the oracle"""
+    r = rng(46 + d + n)
+    ids = np.sort(r.choice(d, n, replace=False)).astype(np.int32)
+    comp, skip = randn_h(r, (rows, ld)), randn_h(r, (rows, d))
+    g, b = randn_h(r, (d,), 0.3) + np.float16(1), randn_h(r, (d,), 0.3)
+    expanded = np.zeros((rows, d), np.float16)
+    expanded[:, ids] = comp[:, :n]
+    got = host(K.scatter_skip_layernorm(dev(comp), dev(ids), dev(skip), dev(g), dev(b)))
+    check_close(got, orc.skip_layernorm(expanded, skip, g, b, f64=True), what="scatter + skip + LayerNorm")
+    two = K.scatter_cols(dev(comp), dev(ids), d)
+    K.skip_layernorm(two, dev(skip), dev(g), dev(b))
+    assert np.array_equal(got, host(two))
+    if d % 8 == 0 and ld % 8 == 0:   # the one-launch form may overwrite the skip operand
+        sk = dev(skip)
+        K.scatter_skip_layernorm(dev(comp), dev(ids), sk, dev(g), dev(b), out=sk)
+        assert np.array_equal(host(sk), got)
