@@ -28,6 +28,7 @@ PROTOTYPES = {
     "et_attention_mask_summary": (_i, [_vp, _i, _vp, _vp]),
     "et_attention_mask_summary_attach": (_i, [_vp, _i, _vp]),
     "et_OTF_attention_varlen": (_i, [_vp, _vp, _vp, _vp, _vp, _ip, _i, _i, _i, _i, _f, _vp]),
+    "et_OTF_attention_qk_width": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _ip, _f, _vp]),
     "et_Prune_attention": (_i, [_vp, _vp, _vp, _vp, _ip, _i, _ip, _ip, _i, _vp, _i, _i, _i, _i, _ip, _f, _vp]),
     "et_sharedQK_attention": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _ip, _f, _vp]),
     "et_qk_scores": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),

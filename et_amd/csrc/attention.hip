@@ -79,17 +79,22 @@ __device__ __forceinline__ float xor_max_16_32(float v) {
 // PLAIN: the launcher has established that there is no mask (or an all-zero
 // one), every sequence has full length and seq_len is a multiple of the
 // workgroup's query rows - no guards, no mask bookkeeping.
-template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK, bool PLAIN = false>
+// HDK: width of a head in Q and K.  HDK < HD is attention-aware pruning with
+// the same number of kept columns in every head: Q and K are compact
+// [rows x nhead*HDK], head h at columns h*HDK, and the scores contract over
+// HDK; V and the output keep HD columns per head.
+template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK, bool PLAIN = false, int HDK = HD>
 __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attention_kernel(const AttnArgs a) {
     static_assert(!PLAIN || (!PRUNED && !SHAREDQK), "the plain form exists for the on-the-fly kernel only");
+    static_assert(HDK == HD || (!PRUNED && !SHAREDQK && HDK % 32 == 0), "narrow Q/K heads: on-the-fly kernel only");
     constexpr int AT_THREADS = NW * 64; // NW waves, each owning 16*QS query rows
     constexpr int AT_WAVES = NW;
-    constexpr int DK = HD / 32;    // k-steps of Q K^T
+    constexpr int DK = HDK / 32;   // k-steps of Q K^T
     constexpr int DV = HD / 16;    // 16-wide column subtiles of the output
     // LDS row strides.  K rows are read with ds_read_b128 by 16 lanes at a
     // time: a stride of 32 (mod 64) bytes is conflict-free (measured); V^T rows
     // are read with ds_read_b64, for which an odd multiple of 16 bytes is.
-    constexpr int LDK = HD + 16;
+    constexpr int LDK = HDK + 16;
     constexpr int LDV = AT_KT + 8;
     constexpr int QB = AT_WAVES * 16 * QS; // queries per workgroup
     constexpr int LDO = HD + 8;
@@ -135,7 +140,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
     if (q0 >= rows_alloc)
         return;
 
-    int qc0 = h * HD, nqk = HD, vc0 = h * HD, nv = HD;
+    int qc0 = h * HDK, nqk = HD, vc0 = h * HD, nv = HD;
     if (PRUNED) {
         if (a.qk_head_ptr) {
             qc0 = a.qk_head_ptr[h];
@@ -274,10 +279,11 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
         // row's first bytes.  Rows at or beyond len re-read the last valid row
         // (their scores are masked to -inf / their P is 0).
         auto dma_tile = [&](int kb, int buf) {
-            constexpr int ROWB = LDK * 2;                // LDS bytes per row, K and V alike
-            constexpr int NINST = AT_KT * ROWB / 1024;   // per operand
-            static_assert(AT_KT * ROWB % 1024 == 0, "tile is a whole number of DMA instructions");
-            constexpr int NTOT = (SHAREDQK ? 1 : 2) * NINST;
+            constexpr int ROWBK = LDK * 2, ROWBV = LDVN * 2; // LDS bytes per row
+            constexpr int NINSTK = SHAREDQK ? 0 : AT_KT * ROWBK / 1024, NINSTV = AT_KT * ROWBV / 1024;
+            static_assert(AT_KT * ROWBK % 1024 == 0 && AT_KT * ROWBV % 1024 == 0,
+                          "a tile is a whole number of DMA instructions");
+            constexpr int NTOT = NINSTK + NINSTV;
             f16 *ks = smem + buf * (KBUF + VBUF);
             f16 *vs = ks + KBUF;
 #pragma unroll
@@ -285,12 +291,13 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 const int i = i0 + wave;
                 if (NTOT % AT_WAVES != 0 && i >= NTOT)
                     break;
-                const bool isv = SHAREDQK || i >= NINST;
-                const int ii = (!SHAREDQK && isv) ? i - NINST : i;
+                const bool isv = i >= NINSTK;
+                const int ii = isv ? i - NINSTK : i;
                 const int p = ii * 1024 + lane * 16;
-                const int row = p / ROWB, cb = p - row * ROWB;
+                const int rowb = isv ? ROWBV : ROWBK;
+                const int row = p / rowb, cb = p - row * rowb;
                 const int rr = min(kb + row, len - 1);
-                const int col = cb < HD * 2 ? (cb >> 1) : 0;
+                const int col = cb < (isv ? HD : HDK) * 2 ? (cb >> 1) : 0;
                 const f16 *src = isv ? a.V + (size_t)(row0 + rr) * a.ldv + vc0 + col
                                      : a.K + (size_t)(row0 + rr) * a.ldq + qc0 + col;
                 load_lds16(src, (isv ? vs : ks) + ii * 512);
@@ -700,17 +707,17 @@ qk_scores_kernel(f16 *__restrict__ QK, const f16 *__restrict__ Q, const f16 *__r
 }
 
 // LDS bytes of one workgroup (mirrors the constants inside the kernel)
-template <int HD, int QS, int NW, bool PRUNED> constexpr size_t attn_lds_bytes() {
+template <int HD, int QS, int NW, bool PRUNED, int HDK = HD> constexpr size_t attn_lds_bytes() {
     // (must agree with the kernel's KBUF / VBUF)
-    constexpr int KV = 2 * (AT_KT * (HD + 16) + (PRUNED ? HD * (AT_KT + 8) : AT_KT * (HD + 16)));
+    constexpr int KV = 2 * (AT_KT * (HDK + 16) + (PRUNED ? HD * (AT_KT + 8) : AT_KT * (HD + 16)));
     constexpr int O = NW * 16 * QS * (HD + 8);
     return sizeof(f16) * (size_t)(KV > O ? KV : O);
 }
 
-template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK, bool PLAIN = false>
+template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK, bool PLAIN = false, int HDK = HD>
 static void attn_launch_one(const AttnArgs &a, hipStream_t st) {
-    constexpr size_t lds = attn_lds_bytes<HD, QS, NW, PRUNED>();
-    auto kern = attention_kernel<HD, QS, NW, PRUNED, SHAREDQK, PLAIN>;
+    constexpr size_t lds = attn_lds_bytes<HD, QS, NW, PRUNED, HDK>();
+    auto kern = attention_kernel<HD, QS, NW, PRUNED, SHAREDQK, PLAIN, HDK>;
     if (lds > 64 * 1024) { // above the default dynamic-LDS limit: opt in once per kernel
         static bool done = false;
         if (!done) {
@@ -723,25 +730,25 @@ static void attn_launch_one(const AttnArgs &a, hipStream_t st) {
 }
 
 // variant 0: 4 waves x 32 query rows; 1: 8 waves x 16 rows; 2: 4 waves x 16 rows
-template <int HD, bool PRUNED, bool SHAREDQK>
+template <int HD, bool PRUNED, bool SHAREDQK, int HDK = HD>
 static void attn_launch_variant(int variant, bool plain, const AttnArgs &a, hipStream_t st) {
     if constexpr (!PRUNED && !SHAREDQK) {
         if (plain) {
             if (variant == 0)
-                attn_launch_one<HD, 2, 4, false, false, true>(a, st);
+                attn_launch_one<HD, 2, 4, false, false, true, HDK>(a, st);
             else if (variant == 1)
-                attn_launch_one<HD, 1, 8, false, false, true>(a, st);
+                attn_launch_one<HD, 1, 8, false, false, true, HDK>(a, st);
             else
-                attn_launch_one<HD, 1, 4, false, false, true>(a, st);
+                attn_launch_one<HD, 1, 4, false, false, true, HDK>(a, st);
             return;
         }
     }
     if (variant == 0)
-        attn_launch_one<HD, 2, 4, PRUNED, SHAREDQK>(a, st);
+        attn_launch_one<HD, 2, 4, PRUNED, SHAREDQK, false, HDK>(a, st);
     else if (variant == 1)
-        attn_launch_one<HD, 1, 8, PRUNED, SHAREDQK>(a, st);
+        attn_launch_one<HD, 1, 8, PRUNED, SHAREDQK, false, HDK>(a, st);
     else
-        attn_launch_one<HD, 1, 4, PRUNED, SHAREDQK>(a, st);
+        attn_launch_one<HD, 1, 4, PRUNED, SHAREDQK, false, HDK>(a, st);
 }
 
 static int g_attn_variant = -1; // et_tuning_set("attn_variant"): -1 = automatic
@@ -807,8 +814,9 @@ static bool attach_mask_summary(AttnArgs &a) {
     return false;
 }
 
+// qk_width: columns per head in Q and K (0 = head_dim)
 static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedqk,
-                              hipStream_t st, const char *who) {
+                              hipStream_t st, const char *who, int qk_width = 0) {
     ET_REQUIRE(a.out && a.V, ET_ERR_INVALID_ARG, "%s: null pointer", who);
     ET_REQUIRE(sharedqk ? a.QK != nullptr : (a.Q && a.K), ET_ERR_INVALID_ARG, "%s: null pointer", who);
     ET_REQUIRE(a.seq_len > 0 && d_model > 0 && a.nhead > 0 && a.batch > 0, ET_ERR_INVALID_ARG,
@@ -848,6 +856,12 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
         else if (pruned) attn_launch_variant<HDV, true, false>(variant, false, a, st);                  \
         else attn_launch_variant<HDV, false, false>(variant, plain, a, st);                             \
     }
+    if (qk_width && qk_width != hd) {
+        ET_REQUIRE(hd == 64 && qk_width == 32 && !pruned && !sharedqk, ET_ERR_UNSUPPORTED,
+                   "%s: %d of %d columns per head in Q and K is not built (32 of 64 is)", who, qk_width, hd);
+        attn_launch_variant<64, false, false, 32>(variant, plain, a, st);
+        return launch_status(who);
+    }
     ET_ATTN_CASE(32)
     ET_ATTN_CASE(64)
     ET_ATTN_CASE(128)
@@ -877,6 +891,29 @@ extern "C" int et_OTF_attention(void *out, const void *Q, const void *K, const v
     a.log2_scale = log2_scale;
     return attention_dispatch(a, d_model, false, false, static_cast<hipStream_t>(stream),
                               "et_OTF_attention");
+}
+
+extern "C" int et_OTF_attention_qk_width(void *out, const void *Q, const void *K, const void *V,
+                                         const void *mask, int qk_width, int seq_len, int d_model,
+                                         int nhead, int batch, const int *seq_lens, float log2_scale,
+                                         void *stream) {
+    using namespace et;
+    ET_REQUIRE(qk_width > 0 && nhead > 0, ET_ERR_INVALID_ARG, "et_OTF_attention_qk_width: qk_width=%d", qk_width);
+    AttnArgs a = {};
+    a.out = static_cast<f16 *>(out);
+    a.Q = static_cast<const f16 *>(Q);
+    a.K = static_cast<const f16 *>(K);
+    a.V = static_cast<const f16 *>(V);
+    a.mask = static_cast<const f16 *>(mask);
+    a.seq_lens = seq_lens;
+    a.ldq = nhead * qk_width;
+    a.ldv = d_model;
+    a.seq_len = seq_len;
+    a.nhead = nhead;
+    a.batch = batch;
+    a.log2_scale = log2_scale;
+    return attention_dispatch(a, d_model, false, false, static_cast<hipStream_t>(stream),
+                              "et_OTF_attention_qk_width", qk_width);
 }
 
 extern "C" int et_OTF_attention_varlen(void *out, const void *Q, const void *K, const void *V,

@@ -117,6 +117,9 @@ class Linear_row {
     // (panel in LDS, pipelined weight stream) then serve the dense product too;
     // null when in_feat is not a multiple of 16
     et_tile_plan *plan;
+    // kept rows per head where every head keeps the same number and no padding
+    // row exists (head h is then columns h*w .. of the compact output), else 0
+    int uniform_head_width;
 
     static int multiple_16(int x) { return ((x + 15) / 16) * 16; }
 
@@ -126,7 +129,7 @@ class Linear_row {
         : in_feat(in_feat_), out_feat(out_feat_), size(size_), nhead(nhead_),
           weight(in_feat_ * multiple_16(row_id_size_)), row_id(row_id_, row_id_size_ > 0 ? row_id_size_ : 1),
           head_ptr(nhead_ + 1), nrow(multiple_16(row_id_size_)), row_id_size(row_id_size_),
-          bias(multiple_16(row_id_size_)), is_gelu(is_gelu_), plan(nullptr) {
+          bias(multiple_16(row_id_size_)), is_gelu(is_gelu_), plan(nullptr), uniform_head_width(0) {
         // padded rows must contribute nothing: zero the buffers first
         etChk(et_fill_zero(weight.get(), sizeof(half) * (size_t)in_feat * nrow, nullptr));
         etChk(et_fill_zero(bias.get(), sizeof(half) * (size_t)nrow, nullptr));
@@ -136,6 +139,12 @@ class Linear_row {
         std::vector<int> h_head_ptr(nhead + 1);
         etChk(et_head_ptr(row_id_, row_id_size, nhead, out_feat / nhead, h_head_ptr.data()));
         head_ptr.set(h_head_ptr.data());
+        if (nhead > 0 && row_id_size == nrow && row_id_size % nhead == 0) {
+            uniform_head_width = row_id_size / nhead;
+            for (int h = 0; h <= nhead; h++)
+                if (h_head_ptr[h] != h * uniform_head_width)
+                    uniform_head_width = 0;
+        }
         if (in_feat % 16 == 0) {
             const int bcols = in_feat / 16, brows = nrow / 16;
             std::vector<half> wpad((size_t)nrow * in_feat, (half)0), bpad(nrow, (half)0);
@@ -156,7 +165,8 @@ class Linear_row {
     Linear_row(Linear_row &&o) noexcept
         : in_feat(o.in_feat), out_feat(o.out_feat), size(o.size), nhead(o.nhead), weight(std::move(o.weight)),
           row_id(std::move(o.row_id)), head_ptr(std::move(o.head_ptr)), nrow(o.nrow),
-          row_id_size(o.row_id_size), bias(std::move(o.bias)), is_gelu(o.is_gelu), plan(o.plan) {
+          row_id_size(o.row_id_size), bias(std::move(o.bias)), is_gelu(o.is_gelu), plan(o.plan),
+          uniform_head_width(o.uniform_head_width) {
         o.plan = nullptr;
     }
     Linear_row(const Linear_row &) = delete;

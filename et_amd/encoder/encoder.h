@@ -230,9 +230,14 @@ class Encoder_attnaware : public Encoder_base {
             K_linear.run_rows(buffers[1], in, n, stream);
             V_linear.run_rows(buffers[2], in, n, stream);
         }
-        etChk(et_Prune_attention(buffers[3], buffers[0], buffers[1], buffers[2], Q_linear.head_ptr.get(),
-                                 Q_linear.nrow, nullptr, nullptr, d_model, mask_ptr(), seq_len, d_model,
-                                 nheads, batch, lens_ptr(), log2_scale, stream));
+        if (Q_linear.uniform_head_width == 32 && K_linear.uniform_head_width == 32 && d_model == 64 * nheads)
+            // every head keeps 32 of its 64 columns: the on-the-fly kernel with narrow Q/K heads
+            etChk(et_OTF_attention_qk_width(buffers[3], buffers[0], buffers[1], buffers[2], mask_ptr(), 32,
+                                            seq_len, d_model, nheads, batch, lens_ptr(), log2_scale, stream));
+        else
+            etChk(et_Prune_attention(buffers[3], buffers[0], buffers[1], buffers[2], Q_linear.head_ptr.get(),
+                                     Q_linear.nrow, nullptr, nullptr, d_model, mask_ptr(), seq_len, d_model,
+                                     nheads, batch, lens_ptr(), log2_scale, stream));
         O_linear.run_rows(buffers[0], buffers[3], n, stream);
         // expansion to model width, skip connection and LayerNorm in one launch
         O_linear.scatter_skip_layernorm(buffers[1], buffers[0], in, ln_gamma[0].get(), ln_beta[0].get(), n, stream);

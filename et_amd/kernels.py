@@ -67,6 +67,15 @@ def OTF_attention(Q, K, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2_sc
     return Z
 
 
+def OTF_attention_qk_width(Q, K, V, mask, qk_width, seq_len, nhead, batch=1, seq_lens=None, log2_scale=1.0, out=None):
+    """Q, K compact [rows x nhead*qk_width] (the same number of kept columns in every head); V full width"""
+    d_model = V.shape[1]
+    Z = out if out is not None else torch.empty_like(V)
+    check(lib().et_OTF_attention_qk_width(_h(Z), _h(Q), _h(K), _h(V), _h(mask), qk_width, seq_len, d_model, nhead,
+                                          batch, _i32(seq_lens), log2_scale, _stream()))
+    return Z
+
+
 def OTF_attention_varlen(Q, K, V, mask, cu_seqlens, max_seq_len, nhead, log2_scale=1.0, out=None):
     d_model = Q.shape[1]
     batch = cu_seqlens.numel() - 1

@@ -105,6 +105,21 @@ size_t et_attention_mask_summary_bytes(int seq_len);
 int et_attention_mask_summary(const void *mask, int seq_len, void *summary, void *stream);
 int et_attention_mask_summary_attach(const void *mask, int seq_len, const void *summary);
 
+/* et_OTF_attention with Q and K holding qk_width < head_dim columns per head,
+ * the same number in every head (attention-aware pruning that keeps the heads
+ * balanced): Q, K are [batch*seq_len x nhead*qk_width], head h at columns
+ * h*qk_width, the scores contract over qk_width and are scaled by
+ * half(1/sqrt(head_dim)) as before; V and out keep d_model columns.  Same
+ * result as et_Prune_attention with qk_head_ptr[h] = h*qk_width, through the
+ * faster on-the-fly kernel.  Built for qk_width 32 with head_dim 64
+ * (ET_ERR_UNSUPPORTED otherwise).  No counterpart in the reference, whose
+ * Prune_attention (kernels/kernels.h:26-30) prunes V only. */
+int et_OTF_attention_qk_width(void *out, const void *Q, const void *K,
+                              const void *V, const void *mask, int qk_width,
+                              int seq_len, int d_model, int nhead, int batch,
+                              const int *seq_lens, float log2_scale,
+                              void *stream);
+
 /* Variable-length (packed) form of et_OTF_attention for the
  * sequence-length-aware path: rows of sequence b are
  * cu_seqlens[b]..cu_seqlens[b+1]-1 of out/Q/K/V (no padding rows exist);

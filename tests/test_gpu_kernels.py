@@ -515,6 +515,33 @@ def test_prune_attention(K):
     check_close(got2, want2, max_abs=5e-3, mean_rel=1e-3, what="pruned attention, dense QK")
 
 
+@pytest.mark.parametrize("S,B,with_mask,with_lens", [(160, 2, True, True), (256, 3, False, False),
+                                                     (512, 2, True, False), (77, 1, False, True)])
+def test_otf_attention_narrow_qk_heads(K, S, B, with_mask, with_lens):
+    """every head keeps 32 of its 64 Q/K columns: the on-the-fly kernel on compact Q/K
+    == the pruned-attention oracle == et_Prune_attention with the matching head_ptr"""
+    r = rng(47 + S)
+    H, d = 12, 768
+    hd = d // H
+    Q, Kk, V = (randn_h(r, (B * S, d)) for _ in range(3))
+    mask = randn_h(r, (S, S), 0.3) if with_mask else None
+    lens = r.integers(1, S + 1, size=B).astype(np.int32) if with_lens else None
+    qk_id = orc.gen_head_balanced_rows(H, hd, 32, seed=2)
+    qk_hp = orc.head_ptr(qk_id, H, hd)
+    assert np.array_equal(qk_hp, 32 * np.arange(H + 1))
+    Qc, Kc = np.ascontiguousarray(Q[:, qk_id]), np.ascontiguousarray(Kk[:, qk_id])
+    md, ld = (None if mask is None else dev(mask)), (None if lens is None else dev(lens))
+    want = orc.prune_attention(Qc, Kc, V, qk_hp, None, None, mask, S, d, H, B, lens, f64=True)
+    got = host(K.OTF_attention_qk_width(dev(Qc), dev(Kc), dev(V), md, 32, S, H, B, ld))
+    other = host(K.Prune_attention(dev(Qc), dev(Kc), dev(V), dev(qk_hp), None, None, md, S, d, H, B, ld))
+    valid = np.ones(B * S, bool) if lens is None else np.concatenate([np.arange(S) < n for n in lens])
+    check_close(got[valid], want[valid], max_abs=5e-3, mean_rel=1e-3, what="narrow Q/K heads")
+    check_close(got[valid], other[valid], max_abs=2e-3, mean_rel=1e-3, what="narrow Q/K heads vs pruned kernel")
+    assert (got[~valid] == 0).all()
+    with pytest.raises(Exception):   # only 32 of 64 is built
+        K.OTF_attention_qk_width(dev(Qc[:, :192]), dev(Kc[:, :192]), dev(V), md, 16, S, H, B, ld)
+
+
 def test_sharedqk_attention_and_scores(K):
     r = rng(44)
     S, H, d, B = 200, 12, 768, 2
