@@ -1834,9 +1834,9 @@ static int choose_nb(int nrp, int nbr_max, int nlin) {
 constexpr int TL_BM64 = 2 * TL_BM;
 static int g_tile_bm64 = 1; // et_tuning_set("tile_bm64")
 
-template <bool GELU>
+template <int NB, bool GELU>
 static int launch_resident64(const TlArgs &a, size_t lds, hipStream_t st) {
-    auto k = tile_linear_resident_kernel<3, GELU, TL_WAVES, false, TL_BM64>;
+    auto k = tile_linear_resident_kernel<NB, GELU, TL_WAVES, false, TL_BM64>;
     ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_THREADS), lds, st, a);
@@ -1868,33 +1868,45 @@ static int tile_launch(const TlProblem *probs, int nlin, const f16 *X, int M, in
     if (mode == TL_PLAN && nchunk == 1 && g_tile_bm64 && g_tile_nb == 0) {
         // 64-row panels, one workgroup per CU: twice the rows per kilobyte of W
         // streamed.  Needs the panel and eight 64-row staging tiles in LDS and
-        // at least two items per CU.
+        // at least two items per CU.  Three or two block-rows per wave, and d
+        // consecutive items of a panel per workgroup: the pair with the least
+        // estimated time (a round of workgroups costs the panel load, 2/3 of a
+        // three-block-row item, plus its items).
         const int cus = std::max(et_device_cu_count(), 1);
-        const size_t lds64 = (size_t)TL_BM64 * (KC + ((KC & 31) ? 0 : TL_PAD)) * sizeof(f16) +
-                             (size_t)TL_WAVES * TL_BM64 * (16 * 3 + 8) * sizeof(f16);
         const int nrp64 = (M + TL_BM64 - 1) / TL_BM64;
-        const int ncg64 = (nbr_max + TL_WAVES * 3 - 1) / (TL_WAVES * 3);
-        const long items = (long)nrp64 * ncg64 * nlin;
-        if (lds64 <= 160 * 1024 && items >= (g_tile_bm64 >= 2 ? 1L : 2L * cus)) {
-            a.ncg = ncg64;
-            a.total = (int)items;
+        double best = 0.0;
+        int best_nb = 0, best_d = 1, best_ncg = 1;
+        size_t best_lds = 0;
+        for (int nb = 3; nb >= 2; nb--) {
+            const size_t lds64 = (size_t)TL_BM64 * (KC + ((KC & 31) ? 0 : TL_PAD)) * sizeof(f16) +
+                                 (size_t)TL_WAVES * TL_BM64 * (16 * nb + 8) * sizeof(f16);
+            const int ncg64 = (nbr_max + TL_WAVES * nb - 1) / (TL_WAVES * nb);
+            const long items = (long)nrp64 * ncg64 * nlin;
+            if (lds64 > 160 * 1024 || items < (g_tile_bm64 >= 2 ? 1L : 2L * cus))
+                continue;
             const int per_rp = ncg64 * nlin;
-            double best = 0.0;
-            a.ipw = 1;
-            for (int d = 1; d <= per_rp; d++) { // as below, with one workgroup slot per CU
+            for (int d = 1; d <= per_rp; d++) {
                 if (per_rp % d)
                     continue;
                 const long nwg = items / d, rounds = (nwg + cus - 1) / cus;
-                const double cost = (double)rounds * (2.0 / 3.0 + d);
-                if (d == 1 || cost < best * 0.999) {
+                const double cost = (double)rounds * (2.0 / 3.0 + d * nb / 3.0);
+                if (best_nb == 0 || cost < best * 0.999) {
                     best = cost;
-                    a.ipw = d;
+                    best_nb = nb;
+                    best_d = d;
+                    best_ncg = ncg64;
+                    best_lds = lds64;
                 }
             }
-            if (g_tile_ipw > 0)
-                a.ipw = g_tile_ipw;
+        }
+        if (best_nb) {
+            a.ncg = best_ncg;
+            a.total = nrp64 * best_ncg * nlin;
+            a.ipw = g_tile_ipw > 0 ? g_tile_ipw : best_d;
             a.per_xcd = ((a.total + a.ipw - 1) / a.ipw + 7) / 8;
-            return gelu ? launch_resident64<true>(a, lds64, st) : launch_resident64<false>(a, lds64, st);
+            if (best_nb == 3)
+                return gelu ? launch_resident64<3, true>(a, best_lds, st) : launch_resident64<3, false>(a, best_lds, st);
+            return gelu ? launch_resident64<2, true>(a, best_lds, st) : launch_resident64<2, false>(a, best_lds, st);
         }
     }
     const int nrp = (M + TL_BM - 1) / TL_BM;
