@@ -136,7 +136,7 @@ scatter_skip_layernorm_kernel(f16 *__restrict__ out, const f16 *__restrict__ com
     const long row = (long)blockIdx.x * 4 + wave;
     if (row >= num)
         return;
-    f16 *strip = reinterpret_cast<f16 *>(ln_smem) + wave * size;
+    f16 *strip = reinterpret_cast<f16 *>(ln_smem) + wave * (size + 8); // (the 8 halves behind a row take the writes of lanes past n)
     const int nchunk = size >> 3;
     const bool last_ok = lane + (NCH - 1) * 64 < nchunk;
     int ci[NCH];
@@ -168,8 +168,7 @@ scatter_skip_layernorm_kernel(f16 *__restrict__ out, const f16 *__restrict__ com
 #pragma unroll
         for (int k = 0; k < 8; k++) {
             const int c = col_id[min(j0 + k, n - 1)];
-            if (j0 + k < n)
-                strip[c] = v[k];
+            strip[j0 + k < n ? c : size] = v[k];
         }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
@@ -318,7 +317,7 @@ extern "C" int et_scatter_skip_layernorm(void *out, const void *compact, const i
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 grid((num + 3) / 4), block(256);
-    const size_t lds = (size_t)4 * size * sizeof(f16);
+    const size_t lds = (size_t)4 * (size + 8) * sizeof(f16);
     const float inv_n = 1.0f / (float)size;
 #define ET_SLN_CASE(NCH_)                                                                         \
     hipLaunchKernelGGL((scatter_skip_layernorm_kernel<NCH_>), grid, block, lds, st,               \
