@@ -79,6 +79,13 @@ __device__ __forceinline__ float xor_max_16_32(float v) {
 // PLAIN: the launcher has established that there is no mask (or an all-zero
 // one), every sequence has full length and seq_len is a multiple of the
 // workgroup's query rows - no guards, no mask bookkeeping.
+// Wave priority in the two MFMA sections of a key tile (0 in the softmax
+// between them): a wave that has its scores or its P ready issues its MFMAs
+// ahead of the waves that are in the vector-ALU part (-1 %).
+#ifndef AT_PRIO
+#define AT_PRIO 1
+#endif
+
 // HDK: width of a head in Q and K.  HDK < HD is attention-aware pruning with
 // the same number of kept columns in every head: Q and K are compact
 // [rows x nhead*HDK], head h at columns h*HDK, and the scores contract over
@@ -395,6 +402,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
         // 122 for one copy - which halved the waves per SIMD)
         auto tile_body = [&](int kb, const f16 *ks, const f16 *vt, const bool FAST, const bool MASKED) {
             // MASKED: this tile's mask values are in mk
+            __builtin_amdgcn_s_setprio(AT_PRIO);
             // ---- scores, transposed: st[ksub][qs][r] = S[q = c16][key = 16 ksub + 4 g4 + r]
             f32x4 st[4][QS];
             if (!SHAREDQK) {
@@ -447,6 +455,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 }
             }
 
+            __builtin_amdgcn_s_setprio(0);
             // ---- mask, online softmax, pack P as the B operand.  The running
             // maximum is only raised when a row's new maximum exceeds it by
             // more than 8 binades (P then stays <= 256, exact enough in half),
@@ -524,6 +533,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                                        ph[kk * 4 + 2][0], ph[kk * 4 + 2][1], ph[kk * 4 + 3][0], ph[kk * 4 + 3][1]};
             }
 
+            __builtin_amdgcn_s_setprio(AT_PRIO);
             // ---- O^T += V^T P^T, V^T fragments read one 16-column subtile ahead
             {
                 auto load_v = [&](int d, f16x8 (&dst)[2]) {
@@ -572,6 +582,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                     for (int qs = 0; qs < QS; qs++)
                         l_acc[qs] = mfma16x16x32(ones8, pf[qs][kk], l_acc[qs]);
             }
+            __builtin_amdgcn_s_setprio(0);
         };
 
         for (int t = 0; t < nt; t++) {

@@ -238,6 +238,12 @@ __device__ __forceinline__ void tl_epilogue_wave(const TlArgs &a, const TlCtx &x
 #ifndef TL_DEPTH
 #define TL_DEPTH 4
 #endif
+// Wave priority while a stream runs (0 outside and inside a flush): waves that
+// are streaming issue their loads and MFMAs ahead of waves that sit in the
+// vector-ALU work of a GELU flush or a LayerNorm (layer tail: -2 %).
+#ifndef TL_PRIO
+#define TL_PRIO 1
+#endif
 static_assert(TL_DEPTH % 2 == 0, "the X operand ping-pong needs an even pipeline depth");
 
 template <int I> using tl_ic = std::integral_constant<int, I>;
@@ -318,6 +324,7 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
     if (q0 >= qend)
         return;
     TL_STAMP(3);
+    __builtin_amdgcn_s_setprio(TL_PRIO);
     f32x4 cur0 = f32x4{0.f, 0.f, 0.f, 0.f}, cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
     int j = 0;
     int bend = __builtin_amdgcn_readlane(bvec, 1);
@@ -354,7 +361,9 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
             tl_load_pair_at(wp + I * 1024, op + I * 8, lane_lo, lane_lw, w[S], o[S]);
         if (q + I + 1 == bend) { // block-row j is complete
             TL_STAMP(2);
+            __builtin_amdgcn_s_setprio(0);
             flush(j, cur0, cur1);
+            __builtin_amdgcn_s_setprio(TL_PRIO);
             cur0 = f32x4{0.f, 0.f, 0.f, 0.f};
             cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
             j++;
@@ -375,6 +384,7 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
         if (q + decltype(ic)::value < qend)
             stage(ic, std::false_type());
     });
+    __builtin_amdgcn_s_setprio(0);
 }
 
 // The same stream over a 64-row panel: every W pair is used for four 16-row
