@@ -152,10 +152,13 @@ def test_encoder_prune_layer():
     check_close(got, want, what="Encoder_prune")
 
 
-def test_encoder_attnaware_layer_config4_wiring():
+@pytest.mark.parametrize("balanced", [True, False])
+def test_encoder_attnaware_layer_config4_wiring(balanced):
     """BASELINE config 4: Q/K keep 32 of 64 columns per head (same set), O/FFN1/FFN2 row-pruned at 70 %.
     Oracle = its own ops chained step by step; invariant = the same layer with DENSE linears whose pruned
-    rows are zero (and, for FFN2, the dropped hidden units' columns)."""
+    rows are zero (and, for FFN2, the dropped hidden units' columns).  balanced = False moves 12 kept
+    columns from head 0 to head 1 (20 and 44 columns): the ragged pruned-attention kernel instead of the
+    narrow-head one."""
     from et_amd.encoder import Encoder_attnaware, Linear_row, Linear_tile
     r = rng(650)
     d, H, dff, S, B = 768, 12, 3072, 64, 2
@@ -166,6 +169,10 @@ def test_encoder_attnaware_layer_config4_wiring():
     W = {k: randn_h(r, shp, 0.03) for k, shp in dict(q=(d, d), k=(d, d), v=(d, d), o=(d, d), m1=(dff, d), m2=(d, dff)).items()}
     bsz = {k: randn_h(r, (W[k].shape[0],), 0.05) for k in W}
     qk_id = orc.gen_head_balanced_rows(H, hd, 32, seed=11)       # 384 kept Q/K columns, 32 per head
+    if not balanced:
+        spare = np.setdiff1d(np.arange(hd, 2 * hd), qk_id)[:12]  # unused columns of head 1
+        qk_id = np.sort(np.concatenate([qk_id[12:], spare])).astype(np.int32)
+        assert np.array_equal(orc.head_ptr(qk_id, H, hd)[:3], [0, 20, 64])
     o_id = orc.gen_sparse_row_mat(d, 0.7, seed=12)               # 230 rows
     m1_id = orc.gen_sparse_row_mat(dff, 0.7, seed=13)            # 921 rows
     m2_id = orc.gen_sparse_row_mat(d, 0.7, seed=14)              # 230 rows
