@@ -178,11 +178,16 @@ int et_device_synchronize(void) {
     return ET_OK;
 }
 int et_device_cu_count(void) {
+    static int cached[16] = {}; // per device: the launchers ask on every call
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess)
         return 0;
+    if (dev >= 0 && dev < 16 && cached[dev] > 0)
+        return cached[dev];
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
         return 0;
+    if (dev >= 0 && dev < 16)
+        cached[dev] = n;
     return n;
 }
 

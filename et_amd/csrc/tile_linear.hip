@@ -69,6 +69,7 @@ struct TlProblem {
     const f16 *bias;
     int N;
     int nbr; // N / 16
+    int ntile = 0; // surviving tiles where known (plans), 0 otherwise
 };
 
 // kernel arguments; per-linear fields as separate arrays that are only ever
@@ -1637,11 +1638,148 @@ __global__ void __launch_bounds__(TL_THREADS) tile_linear_generic_kernel(const T
     }
     tl_epilogue<NB, GELU>(a, x, xs, Yp, N, nbr, acc, b4);
 }
+
+// ---------------------------------------------------------------------------
+// Few rows (a single short sequence).  Such a launch is a chain of memory
+// latencies, not a stream: the kernels above give a wave one (32-row panel,
+// block-row) unit whose tile pairs it requests TL_DEPTH at a time, one round
+// trip to memory per TL_DEPTH pairs and one more per K chunk of the panel
+// (BERT-base FFN2 on 128 rows: 20 us).  Here a workgroup of 16 waves takes a
+// 16-row panel with ALL of its K columns in LDS (16 x 3072 halves = 97 KB) and
+// 16/SPLIT block-rows; the pairs of a block-row are split over SPLIT waves (by
+// K chunk and by pair ranges inside a chunk - with the whole row of X in LDS
+// any partition works), and a wave requests up to TL_SK_D pairs at once, which
+// covers its whole share in the dense BERT-base cases: the panel and all of W
+// arrive in one round trip.  The SPLIT partial sums meet in LDS and are added
+// in a fixed order, so the result does not depend on timing.
+// ---------------------------------------------------------------------------
+constexpr int TL_SK_WAVES = 16;
+constexpr int TL_SK_BM = 16; // rows per panel
+constexpr int TL_SK_D = 12;  // pairs in flight per wave
+
+template <bool GELU, int SPLIT>
+__global__ void __launch_bounds__(TL_SK_WAVES * 64) tile_linear_splitk_kernel(const TlArgs a) {
+    constexpr int BR = TL_SK_WAVES / SPLIT; // block-rows per workgroup
+    extern __shared__ __attribute__((aligned(16))) unsigned char tl_smem[];
+    f16 *xs = reinterpret_cast<f16 *>(tl_smem);
+    const int vid = (blockIdx.x & 7) * a.per_xcd + (blockIdx.x >> 3); // a panel's workgroups on one XCD
+    if (vid >= a.total)
+        return;
+    const int per_rp = a.ncg * a.nlin;
+    const int rp = vid / per_rp, rest = vid - rp * per_rp;
+    const int lin = rest / a.ncg, grp = rest - lin * a.ncg;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int c16 = lane & 15, g4 = lane >> 4, khalf8 = (g4 & 1) * 8, hi = lane >> 5;
+    const int ldx = a.K + ((a.K & 31) ? 0 : TL_PAD); // row stride == 32 (mod 64) bytes
+    const int m0 = rp * TL_SK_BM;
+    f16 *const Yp = TL_SEL(Y);
+    const int *const cptr = TL_SEL(cptr);
+    const int *const poff = TL_SEL(row_offset);
+    const f16 *const data = TL_SEL(data);
+    const f16 *const bias = TL_SEL(bias);
+    const int N = TL_SEL(N);
+    const int nbr = N >> 4;
+
+    // the panel: wave w fetches row w (DMA, 16 bytes per lane and instruction)
+    if (m0 + wave < a.M) {
+        const f16 *src = a.X + (size_t)(m0 + wave) * a.K;
+        f16 *dstrow = xs + wave * ldx;
+        const int pcpr = a.K >> 3;
+        for (int c0 = 0; c0 < pcpr; c0 += 64)
+            if (c0 + lane < pcpr)
+                load_lds16(src + (c0 + lane) * 8, dstrow + c0 * 8);
+    }
+    const int j = wave % BR, sp = wave / BR; // block-row of the group, split
+    const int bn = grp * BR + j;
+    // this wave's pairs: chunk ck of the plan, part `sub` of `spc` of the block-row's segment there
+    const int spc = SPLIT / a.nchunk; // (nchunk divides SPLIT)
+    const int ck = sp / spc, sub = sp - ck * spc;
+    int qa = 0, qb = 0;
+    f16x4 b4 = f16x4{0, 0, 0, 0};
+    if (bn < nbr) {
+        const int p0 = cptr[ck * nbr + bn] >> 1, p1 = cptr[ck * nbr + bn + 1] >> 1;
+        const int len = p1 - p0;
+        qa = p0 + len * sub / spc;
+        qb = p0 + len * (sub + 1) / spc;
+        b4 = *reinterpret_cast<const f16x4 *>(bias + bn * 16 + g4 * 4);
+    }
+    qa = __builtin_amdgcn_readfirstlane(qa);
+    qb = __builtin_amdgcn_readfirstlane(qb);
+    // Pairs at or beyond qb are replaced by the plan's spare pair (all-zero W,
+    // behind the last real pair): every slot loads and multiplies, nothing
+    // inside a round is conditional.
+    const int qsp = __builtin_amdgcn_readfirstlane(cptr[a.nchunk * nbr] >> 1);
+    const unsigned lane_w = hi * 256 + c16 * 16 + khalf8;
+    f16x8 w[TL_SK_D];
+    int o[TL_SK_D];
+    // (requested while the panel is still arriving: loads return in order, the
+    // wait below covers both)
+#pragma unroll
+    for (int i = 0; i < TL_SK_D; i++)
+        tl_load_pair(data, poff, qa + i < qb ? qa + i : qsp, lane_w, hi, w[i], o[i]);
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    __syncthreads();
+
+    // chunk-local column offsets of a multi-chunk plan -> offsets in the full row
+    const char *xlane = reinterpret_cast<const char *>(xs + c16 * ldx + khalf8) + (size_t)ck * a.KC * 2;
+    f32x4 acc0 = f32x4{0.f, 0.f, 0.f, 0.f}, acc1 = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int q = qa;;) {
+#pragma unroll
+        for (int i = 0; i < TL_SK_D; i += 2) { // two accumulators: two independent MFMA chains
+            acc0 = mfma16x16x32(w[i], *reinterpret_cast<const f16x8 *>(xlane + o[i]), acc0);
+            acc1 = mfma16x16x32(w[i + 1], *reinterpret_cast<const f16x8 *>(xlane + o[i + 1]), acc1);
+        }
+        q += TL_SK_D;
+        if (q >= qb)
+            break;
+#pragma unroll
+        for (int i = 0; i < TL_SK_D; i++)
+            tl_load_pair(data, poff, q + i < qb ? q + i : qsp, lane_w, hi, w[i], o[i]);
+    }
+    const f32x4 acc = acc0 + acc1;
+
+    // partial sums -> LDS (behind the panel), summed by the first wave of each block-row
+    f32x4 *red = reinterpret_cast<f32x4 *>(xs + TL_SK_BM * ldx);
+    red[(sp * BR + j) * 64 + lane] = acc;
+    __syncthreads();
+    if (sp == 0 && bn < nbr) {
+        f32x4 t = red[j * 64 + lane];
+#pragma unroll
+        for (int k = 1; k < SPLIT; k++)
+            t += red[(k * BR + j) * 64 + lane];
+        f16x4 ov = __builtin_convertvector(t + __builtin_convertvector(b4, f32x4), f16x4);
+        if (GELU)
+            ov = gelu4(ov);
+        if (m0 + c16 < a.M)
+            *reinterpret_cast<f16x4 *>(Yp + (size_t)(m0 + c16) * N + bn * 16 + g4 * 4) = ov;
+    }
+}
+
 #undef TL_SEL
 
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
+// Dynamic LDS above the 64 KB default has to be allowed per kernel.  The call
+// goes to the driver, so it is made only when a kernel needs more than it was
+// last given (one record per kernel instance and device).
+template <auto KERN>
+static hipError_t allow_lds(size_t lds) {
+    static size_t allowed[16] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
+        return hipFuncSetAttribute(reinterpret_cast<const void *>(KERN),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (lds <= allowed[dev])
+        return hipSuccess;
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(KERN),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess)
+        allowed[dev] = lds;
+    return e;
+}
+
 template <int NB, bool GELU, int MODE>
 static void launch_inst(const TlArgs &a, size_t lds, hipStream_t st) {
     const dim3 grid(a.per_xcd * 8), block(TL_THREADS);
@@ -1675,14 +1813,12 @@ template <int NB>
 static int launch_ln_inst(const TlArgs &a, size_t lds, hipStream_t st) {
     const dim3 grid(a.per_xcd * 8), block(TL_LN_WAVES * 64);
     if (a.nchunk == 1) {
-        auto k = tile_linear_resident_kernel<NB, false, TL_LN_WAVES, true>;
-        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        constexpr auto k = &tile_linear_resident_kernel<NB, false, TL_LN_WAVES, true>;
+        ET_HIP(allow_lds<k>(lds));
         hipLaunchKernelGGL(k, grid, block, lds, st, a);
     } else {
-        auto k = tile_linear_plan_kernel<NB, false, TL_LN_WAVES, true>;
-        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        constexpr auto k = &tile_linear_plan_kernel<NB, false, TL_LN_WAVES, true>;
+        ET_HIP(allow_lds<k>(lds));
         hipLaunchKernelGGL(k, grid, block, lds, st, a);
     }
     return launch_status("tile_linear+LayerNorm launch");
@@ -1697,9 +1833,8 @@ static int ln_block_rows(int nbr) {
 
 template <int NB>
 static int launch_chunked_ln_inst(const TlArgs &a, size_t lds, hipStream_t st) {
-    auto k = tile_linear_chunked_ln_kernel<NB>;
-    ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    constexpr auto k = &tile_linear_chunked_ln_kernel<NB>;
+    ET_HIP(allow_lds<k>(lds));
     hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_CTHREADS), lds, st, a);
     return launch_status("tile_linear+LayerNorm (chunked) launch");
 }
@@ -1753,14 +1888,12 @@ static int tile_launch_ffn(const TlProblem *pO, const TlProblem &p1, const TlPro
     a.beta = beta;
     const size_t lds = ffn_lds_bytes(K1, KC2);
     if (pO) {
-        auto k = tile_ffn_fused_kernel<3, true>;
-        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        constexpr auto k = &tile_ffn_fused_kernel<3, true>;
+        ET_HIP(allow_lds<k>(lds));
         hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_FFN_WAVES * 64), lds, st, a);
     } else {
-        auto k = tile_ffn_fused_kernel<3, false>;
-        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        constexpr auto k = &tile_ffn_fused_kernel<3, false>;
+        ET_HIP(allow_lds<k>(lds));
         hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_FFN_WAVES * 64), lds, st, a);
     }
     return launch_status("fused feed-forward launch");
@@ -1843,12 +1976,13 @@ static int choose_nb(int nrp, int nbr_max, int nlin) {
 
 constexpr int TL_BM64 = 2 * TL_BM;
 static int g_tile_bm64 = 1; // et_tuning_set("tile_bm64")
+static int g_tile_splitk_k1 = 0;
+static int g_tile_splitk_rows = -1; // et_tuning_set("tile_splitk_rows"): row count up to which the few-rows kernel runs, -1 automatic
 
 template <int NB, bool GELU>
 static int launch_resident64(const TlArgs &a, size_t lds, hipStream_t st) {
-    auto k = tile_linear_resident_kernel<NB, GELU, TL_WAVES, false, TL_BM64>;
-    ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    constexpr auto k = &tile_linear_resident_kernel<NB, GELU, TL_WAVES, false, TL_BM64>;
+    ET_HIP(allow_lds<k>(lds));
     hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_THREADS), lds, st, a);
     return launch_status("tile_linear (64-row panels) launch");
 }
@@ -1875,6 +2009,43 @@ static int tile_launch(const TlProblem *probs, int nlin, const f16 *X, int M, in
     a.K = K;
     a.KC = KC;
     a.nchunk = nchunk;
+    // Few rows and K in several chunks: up to 128 rows, up to 256 where at
+    // least three quarters of the tiles survive (each 16-row panel streams W
+    // once more, which a long dense stream repays for longer than a short one).
+    // With K in one chunk the kernels below are as fast.
+    int sk_rows = g_tile_splitk_rows;
+    if (sk_rows < 0) {
+        const long all_tiles = (long)nbr_max * (K / 16);
+        sk_rows = nlin == 1 && 4L * probs[0].ntile >= 3 * all_tiles ? 256 : 128;
+    }
+    if (mode == TL_PLAN && M <= sk_rows && (nchunk == 2 || nchunk == 4 || nchunk == 8 || g_tile_splitk_k1) &&
+        (nchunk == 1 || nchunk == 2 || nchunk == 4 || nchunk == 8) && g_tile_nb == 0) {
+        // few rows: 16-row panels with the whole of K in LDS, a block-row's pairs split over 4 or 8 waves
+        const int split = nchunk == 1 ? 4 : 8;
+        const int br = TL_SK_WAVES / split;
+        const size_t lds_sk = (size_t)TL_SK_BM * (K + ((K & 31) ? 0 : TL_PAD)) * sizeof(f16) +
+                              (size_t)TL_SK_WAVES * 64 * sizeof(f32x4);
+        if (lds_sk <= 160 * 1024) {
+            a.ncg = (nbr_max + br - 1) / br;
+            a.total = ((M + TL_SK_BM - 1) / TL_SK_BM) * a.ncg * nlin;
+            a.ipw = 1;
+            a.per_xcd = (a.total + 7) / 8;
+            const dim3 grid(a.per_xcd * 8), block(TL_SK_WAVES * 64);
+#define TL_SK_LAUNCH(GELU_, SPLIT_)                                                               \
+    {                                                                                             \
+        constexpr auto k = &tile_linear_splitk_kernel<GELU_, SPLIT_>;                                        \
+        ET_HIP(allow_lds<k>(lds_sk));     \
+        hipLaunchKernelGGL(k, grid, block, lds_sk, st, a);                                        \
+    }
+            if (split == 4) {
+                if (gelu) TL_SK_LAUNCH(true, 4) else TL_SK_LAUNCH(false, 4)
+            } else {
+                if (gelu) TL_SK_LAUNCH(true, 8) else TL_SK_LAUNCH(false, 8)
+            }
+#undef TL_SK_LAUNCH
+            return launch_status("tile_linear (few rows) launch");
+        }
+    }
     if (mode == TL_PLAN && nchunk == 1 && g_tile_bm64 && g_tile_nb == 0) {
         // 64-row panels, one workgroup per CU: twice the rows per kilobyte of W
         // streamed.  Needs the panel and eight 64-row staging tiles in LDS and
@@ -2010,6 +2181,14 @@ static int raw_tile_linear(void *Y, const void *X, const int *row_ptr, const int
 } // namespace et
 
 extern "C" int et_tuning_set(const char *key, int value) {
+    if (key && !strcmp(key, "tile_splitk_k1")) {
+        et::g_tile_splitk_k1 = value;
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "tile_splitk_rows")) {
+        et::g_tile_splitk_rows = value;
+        return ET_OK;
+    }
     if (key && !strcmp(key, "tile_nb")) {
         et::g_tile_nb = value;
         return ET_OK;
@@ -2453,6 +2632,7 @@ extern "C" int et_tile_plan_run(const et_tile_plan *plan, void *Y, const void *X
     pr.bias = plan->d_bias;
     pr.N = plan->out_feat;
     pr.nbr = plan->out_feat / 16;
+    pr.ntile = plan->ntile;
     return tile_launch(&pr, 1, static_cast<const f16 *>(X), M, plan->in_feat, plan->KC,
                        plan->nchunk, gelu != 0, TL_PLAN, static_cast<hipStream_t>(stream));
 }

@@ -361,7 +361,13 @@ int et_device_synchronize(void);
  *   "tile_ln_min_panels" fewest 32-row panels for which et_tile_plan_run_ln
  *                     fuses (default 96; below, two launches are faster)
  *   "tile_bm64"       0: planned linears always use 32-row panels; 1 (default):
- *                     64-row panels where two such items per CU exist
+ *                     64-row panels where two such items per CU exist; 2: also
+ *                     with fewer items
+ *   "tile_splitk_rows" most rows for which a planned linear with K > 992 runs
+ *                     the few-rows kernel (16-row panels, a block-row's tile
+ *                     pairs split over several waves); -1 (default): 128, or
+ *                     256 where at least 3/4 of the tiles survive; 0: never
+ *   "tile_splitk_k1"  1: the few-rows kernel also for K <= 992 (default 0)
  *   "tile_fuse_ffn"   0: et_tile_plan_ffn_fusable answers no (the feed-forward
  *                     block runs as separate launches); 1: the block is fused
  *                     but et_tile_plan_tail_fusable answers no; 2 (default)
