@@ -309,6 +309,20 @@ def run_extras(torch, orc, K, dev):
     out["config1_dense_layer_b1_s128"] = {"us": round(us, 2), "seqs_per_s": round(1e6 / us, 1),
                                           "us_as_hip_graph": round(us_g, 2)}
 
+    # the headline layer (80 % tile-pruned) at seq 128: batch 64, the same number of rows
+    r = rng(12)
+    S, B = 128, 64
+    lins, ln = build_layer(orc, r, 0.8, seed=60)
+    x = torch.from_numpy(randn_h(r, (S * B, D))).to(dev)
+    ws = torch.empty(Encoder_tile.buffer_size(D, S, H, B) // 2, dtype=torch.float16, device=dev)
+    L = [Linear_tile(l["K"], l["N"], S * B, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], j == 4)
+         for j, l in enumerate(lins)]
+    enc128 = Encoder_tile(D, S, H, ws, *L, *ln, np.zeros((S, S), np.float16), B)
+    o = torch.empty_like(x)
+    us = timeit(lambda: enc128.run(o, x))
+    out["pruned_layer_80pct_b64_s128"] = {"us": round(us, 2), "seqs_per_s": round(B * 1e6 / us, 1)}
+    del enc128, ws
+
     # config 4: attention-aware pruned layer, batch 32 x seq 256 (Q/K keep 32 of 64 columns per head,
     # O/FFN1/FFN2 row-pruned at 70 %)
     from et_amd.encoder import Encoder_attnaware, Linear_row
