@@ -23,6 +23,8 @@ PROTOTYPES = {
     "et_tile_spmm_add_bias_gelu": (_i, [_vp, _vp, _ip, _ip, _vp, _i, _i, _i, _vp, _vp]),
     "et_row_spmm_add_bias_gelu": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "et_row_spmm_add_bias": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "et_row_spmm_add_bias_multi": (_i, [C.POINTER(_vp), _vp, C.POINTER(_vp), C.POINTER(_vp), _ip, _i, _i, _i, _vp]),
+    "et_row_spmm_prefers_gemm": (_i, [_i, _i, _i]),
     "et_OTF_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _ip, _f, _vp]),
     "et_attention_mask_summary_bytes": (C.c_size_t, [_i]),
     "et_attention_mask_summary": (_i, [_vp, _i, _vp, _vp]),

@@ -93,6 +93,22 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// GELU of four halves: x^3 in (packed) half, the sigmoid form of
+// 0.5(1+tanh u) = 1/(1+exp(-2u)) in fp32, rounded to half, times x in half
+// (kernels/linear.cu:36-48).
+__device__ __forceinline__ f16x4 gelu4(f16x4 v) {
+    const f16x4 x2 = v * v;
+    const f16x4 x3 = v * x2;
+    f32x4 t;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const float s = __builtin_fmaf(0.044715f, (float)x3[r], (float)v[r]);
+        const float e = __builtin_amdgcn_exp2f(s * (-1.5957691216057308f * 1.4426950408889634f));
+        t[r] = __builtin_amdgcn_rcpf(1.0f + e);
+    }
+    return v * __builtin_convertvector(t, f16x4);
+}
+
 __device__ __forceinline__ float f16_bits_to_float(uint16_t b) {
     return (float)__builtin_bit_cast(f16, b);
 }

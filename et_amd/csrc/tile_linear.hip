@@ -820,22 +820,6 @@ struct TlItem {
     const f16 *bias;
 };
 
-// GELU of four halves: x^3 in (packed) half, the sigmoid form of
-// 0.5(1+tanh u) = 1/(1+exp(-2u)) in fp32, rounded to half, times x in half
-// (kernels/linear.cu:36-48).
-__device__ __forceinline__ f16x4 gelu4(f16x4 v) {
-    const f16x4 x2 = v * v;
-    const f16x4 x3 = v * x2;
-    f32x4 t;
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const float s = __builtin_fmaf(0.044715f, (float)x3[r], (float)v[r]);
-        const float e = __builtin_amdgcn_exp2f(s * (-1.5957691216057308f * 1.4426950408889634f));
-        t[r] = __builtin_amdgcn_rcpf(1.0f + e);
-    }
-    return v * __builtin_convertvector(t, f16x4);
-}
-
 // one finished 32x16 block-row tile -> wave-private staging tile
 template <bool GELU>
 __device__ __forceinline__ void tl_stage_tile(f16 *dst, int lds, f32x4 c0, f32x4 c1, f16x4 bj) {
@@ -1976,6 +1960,10 @@ static int choose_nb(int nrp, int nbr_max, int nlin) {
 
 constexpr int TL_BM64 = 2 * TL_BM;
 static int g_tile_bm64 = 1; // et_tuning_set("tile_bm64")
+// rows from which the row-pruned linear runs the register-blocked GEMM (et_tuning_set("row_gemm_min_rows");
+// below, 128 x 128 blocks leave most CUs without work and the tile kernels win)
+static int g_row_gemm_min_rows = 1024;
+
 static int g_tile_splitk_k1 = 0;
 static int g_tile_splitk_rows = -1; // et_tuning_set("tile_splitk_rows"): row count up to which the few-rows kernel runs, -1 automatic
 
@@ -2189,6 +2177,10 @@ extern "C" int et_tuning_set(const char *key, int value) {
         et::g_tile_splitk_rows = value;
         return ET_OK;
     }
+    if (key && !strcmp(key, "row_gemm_min_rows")) {
+        et::g_row_gemm_min_rows = value;
+        return ET_OK;
+    }
     if (key && !strcmp(key, "tile_nb")) {
         et::g_tile_nb = value;
         return ET_OK;
@@ -2249,6 +2241,9 @@ extern "C" int et_tile_spmm_add_bias_gelu(void *Y, const void *X, const int *W_r
 }
 
 namespace et {
+// dense_gemm.hip
+int dense_gemm_launch(void *const *Ys, const void *X, const void *const *Ws, const void *const *biases,
+                      const int *Ns, int nlin, int M, int K, bool gelu, hipStream_t st);
 static int row_linear(void *out, const void *in, const void *weight, const void *bias, int M, int N,
                       int K, bool gelu, void *stream) {
     ET_REQUIRE(out && in && weight && bias, ET_ERR_INVALID_ARG, "et_row_spmm_add_bias: null pointer");
@@ -2260,6 +2255,11 @@ static int row_linear(void *out, const void *in, const void *weight, const void 
                ET_ERR_ALIGNMENT, "et_row_spmm_add_bias: pointers must be 16-byte aligned");
     if (M == 0)
         return ET_OK;
+    if (g_row_gemm_min_rows > 0 && M >= g_row_gemm_min_rows) {
+        const int rc = dense_gemm_launch(&out, in, &weight, &bias, &N, 1, M, K, gelu, static_cast<hipStream_t>(stream));
+        if (rc != ET_ERR_UNSUPPORTED)
+            return rc;
+    }
     TlProblem p;
     p.Y = static_cast<f16 *>(out);
     p.cptr = nullptr;
@@ -2274,6 +2274,35 @@ static int row_linear(void *out, const void *in, const void *weight, const void 
                        static_cast<hipStream_t>(stream));
 }
 } // namespace et
+
+extern "C" int et_row_spmm_prefers_gemm(int M, int N, int K) {
+    return et::g_row_gemm_min_rows > 0 && M >= et::g_row_gemm_min_rows && N > 0 && N % 16 == 0 && K >= 32 &&
+                   K % 32 == 0
+               ? 1
+               : 0;
+}
+
+extern "C" int et_row_spmm_add_bias_multi(void *const *outs, const void *in, const void *const *weights,
+                                          const void *const *biases, const int *Ns, int n, int M, int K,
+                                          void *stream) {
+    using namespace et;
+    ET_REQUIRE(outs && in && weights && biases && Ns, ET_ERR_INVALID_ARG, "et_row_spmm_add_bias_multi: null pointer");
+    ET_REQUIRE(n >= 1 && n <= 3 && M >= 0 && K > 0, ET_ERR_INVALID_ARG, "et_row_spmm_add_bias_multi: n=%d M=%d K=%d",
+               n, M, K);
+    if (M == 0)
+        return ET_OK;
+    if (et_row_spmm_prefers_gemm(M, Ns[0], K)) {
+        const int rc = dense_gemm_launch(outs, in, weights, biases, Ns, n, M, K, false, static_cast<hipStream_t>(stream));
+        if (rc != ET_ERR_UNSUPPORTED)
+            return rc;
+    }
+    for (int i = 0; i < n; i++) { // one after the other
+        const int rc = row_linear(outs[i], in, weights[i], biases[i], M, Ns[i], K, false, stream);
+        if (rc != ET_OK)
+            return rc;
+    }
+    return ET_OK;
+}
 
 extern "C" int et_row_spmm_add_bias(void *out, const void *in, const void *weight,
                                     const void *bias, int M, int N, int K, void *stream) {

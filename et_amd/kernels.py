@@ -49,13 +49,26 @@ def tile_spmm_add_bias(X, row_ptr, row_offset, data, bias, N, gelu=False, out=No
     return Y
 
 
-def row_spmm_add_bias(X, weight, bias, out=None):
+def row_spmm_add_bias(X, weight, bias, out=None, gelu=False):
     """out = X weight^T + bias, weight[N x K] row-major; kernels/kernels.h:7-11"""
     M, K = X.shape
     N = weight.shape[0]
     Y = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=X.device)
-    check(lib().et_row_spmm_add_bias(_h(Y), _h(X), _h(weight), _h(bias), M, N, K, _stream()))
+    fn = lib().et_row_spmm_add_bias_gelu if gelu else lib().et_row_spmm_add_bias
+    check(fn(_h(Y), _h(X), _h(weight), _h(bias), M, N, K, _stream()))
     return Y
+
+
+def row_spmm_add_bias_multi(X, weights, biases):
+    """several row linears over the same input in one launch"""
+    import ctypes as C
+    M, K = X.shape
+    n = len(weights)
+    outs = [torch.empty((M, w.shape[0]), dtype=torch.float16, device=X.device) for w in weights]
+    arr = lambda ts: (C.c_void_p * n)(*[_h(t) for t in ts])
+    ns = (C.c_int * n)(*[w.shape[0] for w in weights])
+    check(lib().et_row_spmm_add_bias_multi(arr(outs), _h(X), arr(weights), arr(biases), ns, n, M, K, _stream()))
+    return outs
 
 
 def OTF_attention(Q, K, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2_scale=1.0, out=None):

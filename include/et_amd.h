@@ -75,6 +75,18 @@ int et_row_spmm_add_bias(void *out, const void *in, const void *weight,
 int et_row_spmm_add_bias_gelu(void *out, const void *in, const void *weight,
                               const void *bias, int M, int N, int K,
                               void *stream);
+/* n <= 3 such linears over the same input in one launch (Q and K of the
+ * attention-aware pruned layer): outs[i][M x Ns[i]] = in * weights[i]^T +
+ * biases[i].  No counterpart in the reference. */
+int et_row_spmm_add_bias_multi(void *const *outs, const void *in,
+                               const void *const *weights,
+                               const void *const *biases, const int *Ns, int n,
+                               int M, int K, void *stream);
+/* 1 where the two functions above run the register-blocked dense GEMM kernel
+ * for these sizes (from 1024 rows, K a multiple of 32) and 0 where they run
+ * the tile kernels on W taken as is: a caller that also holds the weights as
+ * a planned tile_mat (Linear_row does) runs the plan in the second case. */
+int et_row_spmm_prefers_gemm(int M, int N, int K);
 
 /* Replaces OTF_attention_kernelLauncher (kernels/kernels.h:22-24,
  * kernels/attention.cu:122-134).  out, Q, K, V are [batch*seq_len x d_model];
@@ -368,6 +380,8 @@ int et_device_synchronize(void);
  *                     pairs split over several waves); -1 (default): 128, or
  *                     256 where at least 3/4 of the tiles survive; 0: never
  *   "tile_splitk_k1"  1: the few-rows kernel also for K <= 992 (default 0)
+ *   "row_gemm_min_rows" rows from which et_row_spmm_add_bias runs the dense
+ *                     GEMM kernel (default 1024; 0: never)
  *   "tile_fuse_ffn"   0: et_tile_plan_ffn_fusable answers no (the feed-forward
  *                     block runs as separate launches); 1: the block is fused
  *                     but et_tile_plan_tail_fusable answers no; 2 (default)

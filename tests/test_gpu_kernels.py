@@ -387,6 +387,51 @@ def test_tile_linear_few_rows_kernel(K, M, N, Kd, sp, gelu):
     assert np.abs(got.astype(np.float32) - other.astype(np.float32)).max() <= 2.0 ** -7
 
 
+@pytest.mark.parametrize("M,N,Kd,gelu", [
+    (1024, 384, 768, False),    # Q / K of the attention-aware pruned layer
+    (1100, 240, 768, False),    # ragged rows, columns not a multiple of the 128-wide block
+    (2048, 928, 768, True),     # row-pruned FFN1
+    (1024, 240, 928, False),    # K = 14.5 steps of 64
+    (1500, 16, 32, False),      # the smallest shapes
+    (4096, 768, 3072, False),
+])
+def test_row_linear_dense_gemm(K, M, N, Kd, gelu):
+    """from 1024 rows the row-pruned linear runs the register-blocked GEMM kernel: against a float64
+    product on a row sample and, everywhere, against the tile kernels on the same operands"""
+    from et_amd import lib
+    r = rng(35 + N + Kd)
+    X, W, b = randn_h(r, (M, Kd)), randn_h(r, (N, Kd), 0.05), randn_h(r, (N,), 0.2)
+    assert lib().et_row_spmm_prefers_gemm(M, N, Kd) == 1 and lib().et_row_spmm_prefers_gemm(512, N, Kd) == 0
+    got = host(K.row_spmm_add_bias(dev(X), dev(W), dev(b), gelu=gelu))
+    try:
+        lib().et_tuning_set(b"row_gemm_min_rows", 0)
+        other = host(K.row_spmm_add_bias(dev(X), dev(W), dev(b), gelu=gelu))
+    finally:
+        lib().et_tuning_set(b"row_gemm_min_rows", 1024)
+    rows = np.unique(np.concatenate([np.arange(0, 130), r.integers(0, M, 100), np.arange(M - 130, M)]))
+    want = (X[rows].astype(np.float64) @ W.astype(np.float64).T + b.astype(np.float64)).astype(np.float16)
+    if gelu:
+        want = orc.gelu(want)
+    check_close(got[rows], want, max_abs=8e-3, mean_rel=5e-4, what="dense GEMM")
+    assert np.abs(got.astype(np.float32) - other.astype(np.float32)).max() <= 2.0 ** -6
+    assert (got != other).mean() < 0.02
+
+
+def test_row_linear_multi_one_launch(K):
+    r = rng(36)
+    M, Kd = 1300, 768
+    Ws = [randn_h(r, (n, Kd), 0.05) for n in (384, 384, 240)]
+    bs = [randn_h(r, (w.shape[0],), 0.2) for w in Ws]
+    X = randn_h(r, (M, Kd))
+    outs = K.row_spmm_add_bias_multi(dev(X), [dev(w) for w in Ws], [dev(b) for b in bs])
+    for w, b, o in zip(Ws, bs, outs):
+        assert np.array_equal(host(o), host(K.row_spmm_add_bias(dev(X), dev(w), dev(b))))
+    few = K.row_spmm_add_bias_multi(dev(X[:100]), [dev(w) for w in Ws], [dev(b) for b in bs])   # tile kernels
+    for w, b, o in zip(Ws, bs, few):
+        want = (X[:100].astype(np.float64) @ w.astype(np.float64).T + b.astype(np.float64)).astype(np.float16)
+        check_close(host(o), want, max_abs=8e-3, mean_rel=5e-4, what="row linears, few rows")
+
+
 def test_tile_linear_full_size_config2_rows_sample(K):
     """config-2 shape (4096x768 -> 3072, 80 %): rows are independent, so a row sample pins the full-size launch"""
     r = rng(32)
