@@ -164,14 +164,19 @@ def main():
     for _ in range(5):
         for _, fn, *_ in steps_def:
             fn()
-    ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nk)] for _ in range(reps)]
+    # (the first passes after the events are created are not counted: the first launch behind a fresh
+    # batch of event records has been seen to block the host for tens of milliseconds)
+    skip = 3
+    ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nk)]
+          for _ in range(reps + skip)]
     torch.cuda.synchronize()
-    for i in range(reps):
+    for i in range(reps + skip):
         for j, (_, fn, *_r) in enumerate(steps_def):
             ev[i][j][0].record()
             fn()
             ev[i][j][1].record()
     torch.cuda.synchronize()
+    ev = ev[skip:]
     kern = []
     for j, (name, _, flops, nbytes, bound) in enumerate(steps_def):
         us = float(np.mean([ev[i][j][0].elapsed_time(ev[i][j][1]) for i in range(reps)])) * 1e3
