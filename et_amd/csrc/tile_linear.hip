@@ -1938,6 +1938,10 @@ static int g_tile_min_wgs = 512;
 static int g_tile_ipw = 0;
 static int g_tile_fuse_ln = 1;
 static int g_tile_ln_min_panels = 96;
+// the layer tail in one launch: from fewer panels than the linear + LayerNorm kernels (measured on
+// BERT-base at 80 %: one launch 42 us for any count below one per CU, step by step 37 / 43 / 54 us
+// at 52 / 80 / 95 panels)
+static int g_tile_tail_min_panels = 72;
 
 // Block-rows per wave.  Measured on the BERT-base shapes (rows 4096..8192):
 // three block-rows per wave is the best trade between panel re-reads (fewer
@@ -2203,6 +2207,7 @@ extern "C" int et_tuning_set(const char *key, int value) {
     }
     if (key && !strcmp(key, "tile_ln_min_panels")) {
         et::g_tile_ln_min_panels = value > 0 ? value : 96;
+        et::g_tile_tail_min_panels = value > 0 ? value : 72;
         return ET_OK;
     }
     if (key && !strcmp(key, "tile_fuse_ln")) {
@@ -2465,6 +2470,7 @@ extern "C" int et_tile_plan_ln_fusable(const et_tile_plan *plan) {
 // The fused kernels run one workgroup per 32-row panel; with few rows that
 // leaves most CUs idle and the two-launch form (more, smaller workgroups) wins.
 static bool ln_fusion_pays(int M) { return M >= 32 * et::g_tile_ln_min_panels; }
+static bool tail_fusion_pays(int M) { return M >= 32 * et::g_tile_tail_min_panels; }
 
 extern "C" int et_tile_plan_run_ln(const et_tile_plan *plan, void *Y, const void *X,
                                    const void *skip, const void *gamma, const void *beta, int M,
@@ -2584,7 +2590,7 @@ extern "C" int et_tile_plan_run_tail(const et_tile_plan *pO, const et_tile_plan 
                ET_ERR_ALIGNMENT, "et_tile_plan_run_tail: pointers must be 16-byte aligned");
     if (M == 0)
         return ET_OK;
-    if (!et_tile_plan_tail_fusable(pO, p1, p2) || (mid && !ln_fusion_pays(M))) {
+    if (!et_tile_plan_tail_fusable(pO, p1, p2) || (mid && !tail_fusion_pays(M))) {
         // step by step through the caller's buffers
         ET_REQUIRE(mid, ET_ERR_UNSUPPORTED,
                    "et_tile_plan_run_tail: these shapes need the mid buffer (%d x %d halves)", M, pO->out_feat);
@@ -2601,7 +2607,7 @@ extern "C" int et_tile_plan_run_tail(const et_tile_plan *pO, const et_tile_plan 
     if (mid && hidden) {
         const int cus = std::max(et_device_cu_count(), 1);
         const int panels = (M + TL_BM - 1) / TL_BM, full = panels / cus * cus, rem = panels - full;
-        if (full > 0 && rem > 0 && rem < g_tile_ln_min_panels) {
+        if (full > 0 && rem > 0 && rem < g_tile_tail_min_panels) {
             const int M1 = full * TL_BM;
             int rc = et_tile_plan_run_tail(pO, p1, p2, Y, attn, input, nullptr, nullptr, gamma1, beta1, gamma2,
                                            beta2, M1, stream);

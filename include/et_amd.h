@@ -371,7 +371,9 @@ int et_device_synchronize(void);
  *   "tile_fuse_ln"    0: et_tile_plan_run_ln runs the linear and the LayerNorm
  *                     as two launches; 1 (default): fused where the rows fit
  *   "tile_ln_min_panels" fewest 32-row panels for which et_tile_plan_run_ln
- *                     fuses (default 96; below, two launches are faster)
+ *                     fuses (default 96; below, two launches are faster); a
+ *                     value > 0 also replaces the 72 panels from which
+ *                     et_tile_plan_run_tail runs as one launch
  *   "tile_bm64"       0: planned linears always use 32-row panels; 1 (default):
  *                     64-row panels where two such items per CU exist; 2: also
  *                     with fewer items
