@@ -314,6 +314,22 @@ def run_extras(torch, orc, K, dev):
     out["config1_dense_layer_b1_s128"] = {"us": round(us, 2), "seqs_per_s": round(1e6 / us, 1),
                                           "us_as_hip_graph": round(us_g, 2)}
 
+    # stand-alone skip + LayerNorm (the launcher replacement; the layer itself runs the fused form):
+    # 6 bytes per element moved.  8192 rows (config 3's count) are a launch too short to reach the
+    # streaming rate and their 38 MB stay in the last-level cache; the larger counts stream from HBM.
+    ln_rows = []
+    gam = torch.ones(D, dtype=torch.float16, device=dev)
+    bet = torch.zeros(D, dtype=torch.float16, device=dev)
+    for rows in (8192, 32768, 131072, 524288):
+        a_ = torch.randn((rows, D), device=dev).to(torch.float16)
+        s_ = torch.randn((rows, D), device=dev).to(torch.float16)
+        us = timeit(lambda: K.skip_layernorm(a_, s_, gam, bet), reps=100 if rows <= 32768 else 30)
+        nbytes = 6.0 * rows * D + 4 * D
+        ln_rows.append({"rows": rows, "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                        "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+        del a_, s_
+    out["skip_layernorm_768_wide"] = ln_rows
+
     # the headline layer (80 % tile-pruned) at seq 128: batch 64, the same number of rows
     r = rng(12)
     S, B = 128, 64
