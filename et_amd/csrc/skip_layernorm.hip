@@ -10,6 +10,13 @@
 
 namespace et {
 
+template <bool NT>
+__device__ __forceinline__ f16x8 ln_load(const f16 *row, int chunk) {
+    if (NT)
+        return __builtin_bit_cast(f16x8, __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row) + chunk));
+    return reinterpret_cast<const f16x8 *>(row)[chunk];
+}
+
 // One wave handles ROWS consecutive rows, one after the other; a row is held
 // as NCH = ceil(size / 512) chunks of 8 halves per lane, chunk c of a row in
 // lane c % 64 (the fused linear + LayerNorm kernels keep a row the same way,
@@ -19,7 +26,11 @@ namespace et {
 // a row's loads are in flight together) and are masked out of the sums and the
 // store.  The next row's loads are issued before the current row is reduced,
 // so every wave keeps reads in flight while it computes and stores.
-template <int NCH, int ROWS>
+// NT: the row operands are loaded with the non-temporal hint - for launches
+// whose operands exceed the last-level cache (streaming from HBM: 131072 rows
+// of 768 98 -> 85 us); smaller ones are faster with ordinary loads (their
+// operands are usually still cached from the kernel that produced them).
+template <int NCH, int ROWS, bool NT>
 __global__ void __launch_bounds__(256)
 skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip,
                           const f16 *__restrict__ gamma,
@@ -56,8 +67,8 @@ skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip
     vec gg[NCH], bb[NCH];
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
-        an[i] = reinterpret_cast<const vec *>(in_out + row0 * size)[ci[i]];
-        sn[i] = reinterpret_cast<const vec *>(skip + row0 * size)[ci[i]];
+        an[i] = ln_load<NT>(in_out + row0 * size, ci[i]);
+        sn[i] = ln_load<NT>(skip + row0 * size, ci[i]);
     }
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
@@ -84,8 +95,8 @@ skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip
         if (r + 1 < ROWS && row + 1 < num) {
 #pragma unroll
             for (int i = 0; i < NCH; i++) {
-                an[i] = reinterpret_cast<const vec *>(in_out + (row + 1) * size)[ci[i]];
-                sn[i] = reinterpret_cast<const vec *>(skip + (row + 1) * size)[ci[i]];
+                an[i] = ln_load<NT>(in_out + (row + 1) * size, ci[i]);
+                sn[i] = ln_load<NT>(skip + (row + 1) * size, ci[i]);
             }
         }
         const float mean = wave_sum(sum) * inv_n;
@@ -269,16 +280,20 @@ extern "C" int et_skip_layernorm(void *in_out, const void *skip, const void *gam
         const float inv_n = 1.0f / (float)size;
         // rows per wave: enough waves to fill the chip first (256 CUs x 32 waves); two from there
         // (four rows per wave measured 4-5 % slower from 131072 rows up)
-        const int rows = g_ln_rows > 0 ? g_ln_rows : (num >= 2 * 8192 ? 2 : 1);
+        // both operands together beyond the 256 MB last-level cache: streaming loads, two rows per wave
+        const bool nt = g_ln_rows == 0 && (size_t)num * size * 4 > (size_t)256 << 20;
+        const int rows = nt ? 2 : g_ln_rows > 0 ? g_ln_rows : (num >= 2 * 8192 ? 2 : 1);
         const dim3 grid((num + 4 * rows - 1) / (4 * rows));
 #define ET_LN_CASE(NCH_)                                                                          \
     {                                                                                             \
-    if (rows >= 4)                                                                                \
-        hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 4>), grid, block, 0, st, a, s, g, b, num, size, inv_n); \
+    if (nt)                                                                                       \
+        hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 2, true>), grid, block, 0, st, a, s, g, b, num, size, inv_n); \
+    else if (rows >= 4)                                                                           \
+        hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 4, false>), grid, block, 0, st, a, s, g, b, num, size, inv_n); \
     else if (rows >= 2)                                                                           \
-        hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 2>), grid, block, 0, st, a, s, g, b, num, size, inv_n); \
+        hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 2, false>), grid, block, 0, st, a, s, g, b, num, size, inv_n); \
     else                                                                                          \
-        hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 1>), grid, block, 0, st, a, s, g, b, num, size, inv_n); \
+        hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 1, false>), grid, block, 0, st, a, s, g, b, num, size, inv_n); \
     }
         {
             switch (nch8) { // size <= 4096: at most 8 chunks

@@ -44,6 +44,29 @@ def test_skip_layernorm(K, rows, size):
     assert (got != want).mean() < 0.02   # fp32 reduction order only
 
 
+def test_skip_layernorm_streaming_form(K):
+    """operands beyond the last-level cache take non-temporal loads: same bits as the ordinary form"""
+    from et_amd import lib
+    rows, size = 90000, 768          # 2 x 138 MB of operands
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = torch.randn((rows, size), device="cuda", generator=g).to(torch.float16)
+    s = torch.randn((rows, size), device="cuda", generator=g).to(torch.float16)
+    gam = (torch.randn(size, device="cuda", generator=g) * 0.3 + 1).to(torch.float16)
+    bet = (torch.randn(size, device="cuda", generator=g) * 0.3).to(torch.float16)
+    got = a.clone()
+    K.skip_layernorm(got, s, gam, bet)
+    try:
+        lib().et_tuning_set(b"ln_rows", 2)   # a fixed row count per wave also keeps the ordinary loads
+        ref = a.clone()
+        K.skip_layernorm(ref, s, gam, bet)
+    finally:
+        lib().et_tuning_set(b"ln_rows", 0)
+    assert torch.equal(got, ref)
+    sel = np.r_[0:40, rows - 40:rows]
+    want = orc.skip_layernorm(host(a[sel]), host(s[sel]), host(gam), host(bet), f64=True)
+    check_close(host(got[sel]), want, what="skip + LayerNorm, streaming form")
+
+
 def test_skip_layernorm_constant_row_and_unit_stats(K):
     d = 768
     g, b = np.ones(d, np.float16), np.zeros(d, np.float16)
