@@ -873,11 +873,13 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
 #define TL_PANEL(rp_)                                                                             \
     {                                                                                             \
         const int pcpr = a.K >> 3;                                                                \
-        _Pragma("unroll") for (int rr = 0; rr < BM / NW; rr++) {                               \
-            const int row = (rp_) * BM + wave * (BM / NW) + rr;                             \
-            if (row < a.M) {                                                                      \
+        constexpr int RPW = (BM + NW - 1) / NW; /* panel rows per wave */                         \
+        _Pragma("unroll") for (int rr = 0; rr < RPW; rr++) {                                      \
+            const int prow = wave * RPW + rr;                                                     \
+            const int row = (rp_) * BM + prow;                                                    \
+            if (row < a.M && (BM % NW == 0 || prow < BM)) {                                       \
                 const f16 *src = a.X + (size_t)row * a.K;                                         \
-                f16 *dstrow = xs + (wave * (BM / NW) + rr) * ldx;                                       \
+                f16 *dstrow = xs + prow * ldx;                                                    \
                 if (lane < pcpr)                                                                  \
                     load_lds16(src + lane * 8, dstrow);                                           \
                 if (64 + lane < pcpr)                                                             \
@@ -1971,11 +1973,11 @@ static int g_row_gemm_min_rows = 1024;
 static int g_tile_splitk_k1 = 0;
 static int g_tile_splitk_rows = -1; // et_tuning_set("tile_splitk_rows"): row count up to which the few-rows kernel runs, -1 automatic
 
-template <int NB, bool GELU>
+template <int NB, bool GELU, int NW = TL_WAVES>
 static int launch_resident64(const TlArgs &a, size_t lds, hipStream_t st) {
-    constexpr auto k = &tile_linear_resident_kernel<NB, GELU, TL_WAVES, false, TL_BM64>;
+    constexpr auto k = &tile_linear_resident_kernel<NB, GELU, NW, false, TL_BM64>;
     ET_HIP(allow_lds<k>(lds));
-    hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TL_THREADS), lds, st, a);
+    hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(NW * 64), lds, st, a);
     return launch_status("tile_linear (64-row panels) launch");
 }
 
@@ -2040,44 +2042,55 @@ static int tile_launch(const TlProblem *probs, int nlin, const f16 *X, int M, in
     }
     if (mode == TL_PLAN && nchunk == 1 && g_tile_bm64 && g_tile_nb == 0) {
         // 64-row panels, one workgroup per CU: twice the rows per kilobyte of W
-        // streamed.  Needs the panel and eight 64-row staging tiles in LDS and
-        // at least two items per CU.  Three or two block-rows per wave, and d
-        // consecutive items of a panel per workgroup: the pair with the least
-        // estimated time (a round of workgroups costs the panel load, 2/3 of a
-        // three-block-row item, plus its items).
+        // streamed.  Needs the panel and one 64-row staging tile per wave in LDS
+        // and at least two items per CU.  Twelve waves of two block-rows (where
+        // the LDS holds their staging tiles: K <= 784), or eight waves of three
+        // or of two, and d consecutive items of a panel per workgroup: the
+        // combination with the least estimated time (a round of workgroups costs
+        // the panel load, 2/3 of a 24-block-row item, plus its items).  Twelve
+        // waves come first and win ties: the same items as eight waves of three,
+        // with three waves per SIMD instead of two to cover the stream's waits
+        // (Q/K/V of the benchmark: 20 -> 17.5 us).
         const int cus = std::max(et_device_cu_count(), 1);
         const int nrp64 = (M + TL_BM64 - 1) / TL_BM64;
+        static const int cand[3][2] = {{12, 2}, {8, 3}, {8, 2}}; // waves, block-rows per wave
         double best = 0.0;
-        int best_nb = 0, best_d = 1, best_ncg = 1;
+        int best_c = -1, best_d = 1, best_ncg = 1;
         size_t best_lds = 0;
-        for (int nb = 3; nb >= 2; nb--) {
+        for (int c = 0; c < 3; c++) {
+            const int nw = cand[c][0], nb = cand[c][1];
+            if (nw == 12 && g_tile_bm64 == 4)
+                continue; // (tuning: eight waves only)
             const size_t lds64 = (size_t)TL_BM64 * (KC + ((KC & 31) ? 0 : TL_PAD)) * sizeof(f16) +
-                                 (size_t)TL_WAVES * TL_BM64 * (16 * nb + 8) * sizeof(f16);
-            const int ncg64 = (nbr_max + TL_WAVES * nb - 1) / (TL_WAVES * nb);
+                                 (size_t)nw * TL_BM64 * (16 * nb + 8) * sizeof(f16);
+            const int ncg64 = (nbr_max + nw * nb - 1) / (nw * nb);
             const long items = (long)nrp64 * ncg64 * nlin;
-            if (lds64 > 160 * 1024 || items < (g_tile_bm64 >= 2 ? 1L : 2L * cus))
+            if (lds64 > 160 * 1024 || items < (g_tile_bm64 == 2 ? 1L : 2L * cus))
                 continue;
             const int per_rp = ncg64 * nlin;
             for (int d = 1; d <= per_rp; d++) {
                 if (per_rp % d)
                     continue;
                 const long nwg = items / d, rounds = (nwg + cus - 1) / cus;
-                const double cost = (double)rounds * (2.0 / 3.0 + d * nb / 3.0);
-                if (best_nb == 0 || cost < best * 0.999) {
+                const double cost = (double)rounds * (2.0 / 3.0 + d * (nw * nb) / 24.0);
+                if (best_c < 0 || cost < best * 0.999) {
                     best = cost;
-                    best_nb = nb;
+                    best_c = c;
                     best_d = d;
                     best_ncg = ncg64;
                     best_lds = lds64;
                 }
             }
         }
-        if (best_nb) {
+        if (best_c >= 0) {
             a.ncg = best_ncg;
             a.total = nrp64 * best_ncg * nlin;
             a.ipw = g_tile_ipw > 0 ? g_tile_ipw : best_d;
             a.per_xcd = ((a.total + a.ipw - 1) / a.ipw + 7) / 8;
-            if (best_nb == 3)
+            if (best_c == 0)
+                return gelu ? launch_resident64<2, true, 12>(a, best_lds, st)
+                            : launch_resident64<2, false, 12>(a, best_lds, st);
+            if (best_c == 1)
                 return gelu ? launch_resident64<3, true>(a, best_lds, st) : launch_resident64<3, false>(a, best_lds, st);
             return gelu ? launch_resident64<2, true>(a, best_lds, st) : launch_resident64<2, false>(a, best_lds, st);
         }

@@ -376,7 +376,8 @@ int et_device_synchronize(void);
  *                     et_tile_plan_run_tail runs as one launch
  *   "tile_bm64"       0: planned linears always use 32-row panels; 1 (default):
  *                     64-row panels where two such items per CU exist; 2: also
- *                     with fewer items
+ *                     with fewer items; 4: as 1 with eight waves per workgroup
+ *                     only (no twelve-wave form)
  *   "tile_splitk_rows" most rows for which a planned linear with K > 992 runs
  *                     the few-rows kernel (16-row panels, a block-row's tile
  *                     pairs split over several waves); -1 (default): 128, or
