@@ -37,9 +37,9 @@ D, H, DFF = 768, 12, 3072
 # default workload and scaled by the 64 MiB copy kernel launched below; commands and raw figures are in
 # profiles/encoder_layer_b16_s512_hbm_traffic.txt.  Only valid for batch 16 x seq 512 at 80 % sparsity.
 MEASURED_TRAFFIC_MIB = {
-    "tile_linear qkv (3 x 768->768, one launch)": 17.98 + 36.02,
+    "tile_linear qkv (3 x 768->768, one launch)": 17.95 + 36.01,
     "attention (on-the-fly)": 36.08 + 12.00,
-    "layer tail: o + skip + LayerNorm + feed-forward (gelu) + skip + LayerNorm, fused": 43.43 + 14.00,
+    "layer tail: o + skip + LayerNorm + feed-forward (gelu) + skip + LayerNorm, fused": 43.44 + 14.00,
 }
 
 
