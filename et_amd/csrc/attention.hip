@@ -49,10 +49,28 @@ struct AttnArgs {
     float log2_scale, scale;
 };
 
+// eight (four) halves at p + d0 of which those at or beyond n read as zero.
+// Whole groups are one load that needs no more than the 2-byte alignment of a
+// half (compact operands start at arbitrary columns; the hardware takes
+// unaligned multi-dword accesses to global memory), only a group that straddles
+// n is fetched element by element.
+typedef f16x8 f16x8_u __attribute__((aligned(2)));
+typedef f16x4 f16x4_u __attribute__((aligned(2)));
 __device__ __forceinline__ f16x8 load8_guard(const f16 *p, int d0, int n) {
+    if (d0 + 8 <= n)
+        return *reinterpret_cast<const f16x8_u *>(p + d0);
     f16x8 v;
 #pragma unroll
     for (int j = 0; j < 8; j++)
+        v[j] = (d0 + j < n) ? p[d0 + j] : (f16)0;
+    return v;
+}
+__device__ __forceinline__ f16x4 load4_guard(const f16 *p, int d0, int n) {
+    if (d0 + 4 <= n)
+        return *reinterpret_cast<const f16x4_u *>(p + d0);
+    f16x4 v;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
         v[j] = (d0 + j < n) ? p[d0 + j] : (f16)0;
     return v;
 }
@@ -244,9 +262,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                         (FULL || key < len)) { // rows at or beyond len read as zero
                         const f16 *vrow = a.V + (size_t)(row0 + key) * a.ldv + vc0;
                         if (PRUNED) {
-#pragma unroll
-                            for (int e = 0; e < 4; e++)
-                                v[e] = (dq * 4 + e < nv) ? vrow[dq * 4 + e] : (f16)0;
+                            v = load4_guard(vrow, dq * 4, nv);
                         } else {
                             v = *reinterpret_cast<const f16x4 *>(vrow + dq * 4);
                         }
@@ -563,6 +579,10 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 load_v(0, vfr[0]);
 #pragma unroll
                 for (int d = 0; d < DV; d++) {
+                    // (a head that keeps nv < 64 value columns has nothing in the
+                    // subtiles from ceil(nv / 16) on: wave-uniform skip)
+                    if (PRUNED && d * 16 >= nv)
+                        break;
                     if (d + 1 < DV)
                         load_v(d + 1, vfr[(d + 1) & 1]);
                     __builtin_amdgcn_sched_barrier(0);
