@@ -170,10 +170,18 @@ class Encoder_prune : public Encoder_base {
         etRequire(MLP1_linear.is_gelu, "Encoder_prune: MLP1_linear must be the GELU variant");
     }
     void run(half *out, half *in) override {
-        const Linear_tile *qk[2] = {&Q_linear, &K_linear};
-        half *outs[2] = {buffers[0], buffers[1]};
-        Linear_tile::run_multi(qk, outs, 2, in, rows(), stream);
-        V_linear.run_rows(buffers[2], in, rows(), stream);
+        if (V_linear.plan && V_linear.in_feat == Q_linear.in_features() &&
+            K_linear.in_features() == Q_linear.in_features()) {
+            // the three projections in one launch (V compact, [rows x nrow])
+            const et_tile_plan *plans[3] = {Q_linear.tile_plan(), K_linear.tile_plan(), V_linear.plan};
+            void *ys[3] = {buffers[0], buffers[1], buffers[2]};
+            etChk(et_tile_plan_run_multi(plans, ys, 3, in, rows(), stream));
+        } else {
+            const Linear_tile *qk[2] = {&Q_linear, &K_linear};
+            half *outs[2] = {buffers[0], buffers[1]};
+            Linear_tile::run_multi(qk, outs, 2, in, rows(), stream);
+            V_linear.run_rows(buffers[2], in, rows(), stream);
+        }
         // compact V has leading dimension nrow (what the GEMM wrote); the
         // reference passes row_id_size here (encoder/encoder.cu:78) and reads
         // the wrong rows whenever that is not a multiple of 16
