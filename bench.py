@@ -344,6 +344,24 @@ def run_extras(torch, orc, K, dev):
     out["pruned_layer_80pct_b64_s128"] = {"us": round(us, 2), "seqs_per_s": round(B * 1e6 / us, 1)}
     del enc128, ws
 
+    # the reference's own pruned wiring (test/prune_test.cu: tile-pruned Q, K, O, FFN; row-pruned V,
+    # pruned attention), batch 16 x seq 512, 80 % tiles, V keeps 230 of 768 rows
+    from et_amd.encoder import Encoder_prune, Linear_row
+    r = rng(13)
+    S, B = 512, 16
+    lins, ln = build_layer(orc, r, 0.8, seed=70)
+    v_id = orc.gen_sparse_row_mat(D, 0.7, seed=16)
+    mk = lambda l, g=False: Linear_tile(l["K"], l["N"], S * B, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], g)
+    Lv = Linear_row(D, D, S * B, randn_h(r, (v_id.size, D), 0.02), v_id, v_id.size, np.zeros(v_id.size, np.float16), H)
+    ws = torch.empty(Encoder_prune.buffer_size(D, S, H, B) // 2, dtype=torch.float16, device=dev)
+    encp = Encoder_prune(D, S, H, ws, mk(lins[0]), mk(lins[1]), Lv, mk(lins[3]), mk(lins[4], True), mk(lins[5]), *ln,
+                         np.zeros((S, S), np.float16), B)
+    x = torch.from_numpy(randn_h(r, (S * B, D))).to(dev)
+    o = torch.empty_like(x)
+    us = timeit(lambda: encp.run(o, x))
+    out["reference_prune_wiring_b16_s512"] = {"us": round(us, 2), "seqs_per_s": round(B * 1e6 / us, 1)}
+    del encp, ws
+
     # config 4: attention-aware pruned layer, batch 32 x seq 256 (Q/K keep 32 of 64 columns per head,
     # O/FFN1/FFN2 row-pruned at 70 %)
     from et_amd.encoder import Encoder_attnaware, Linear_row
