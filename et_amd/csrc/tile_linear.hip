@@ -857,7 +857,6 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
     f16 *const stage0 = xs + BM * ldx;
     f16 *const stage = stage0 + wave * (BM * (16 * NB + 8));
     f16 *const stage_lane = stage + c16 * lds + g4 * 4;
-    const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     const int lane_w = hi * 256 + c16 * 16 + khalf8; // lane's halves inside a 1 KB tile pair
 
     // pair-index boundaries of a wave's block-rows: lane j holds the start of
@@ -1170,7 +1169,6 @@ __global__ void __launch_bounds__(TL_CTHREADS) tile_linear_chunked_ln_kernel(con
         const f16 *const data = a.data[0];
         const int *const poff = a.row_offset[0];
         const unsigned lane_w = hi * 256 + x.c16 * 16 + x.khalf8; // lane's halves inside a 1 KB tile pair
-        const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
         // pair-index boundaries of the wave's block-rows in the current chunk
         // (see tile_linear_plan_kernel); the next chunk's are requested a chunk ahead
         int bvec = cptr[min(x.bn0 + min(lane, NB), nbr)] >> 1;
