@@ -710,3 +710,51 @@ def test_scatter_skip_layernorm_one_launch(K, rows, d, n, ld):
         sk = dev(skip)
         K.scatter_skip_layernorm(dev(comp), dev(ids), sk, dev(g), dev(b), out=sk)
         assert np.array_equal(host(sk), got)
+
+
+# ------------------------------------------------------- empty inputs, bad arguments
+def test_launchers_with_no_rows_touch_nothing_and_bad_arguments_fail_cleanly(K):
+    """row count 0 is a valid call that does nothing; null pointers, misaligned operands and unsupported
+    sizes come back as error codes with a message (nothing is launched, nothing exits)"""
+    import ctypes as C
+    from et_amd import lib
+    from et_amd._lib import EtError, check
+    L = lib()
+    d = 768
+    sentinel = torch.full((64, d), 7.0, dtype=torch.float16, device="cuda")
+    x = torch.zeros((64, d), dtype=torch.float16, device="cuda")
+    g = torch.ones(d, dtype=torch.float16, device="cuda")
+    ids = torch.arange(16, dtype=torch.int32, device="cuda")
+    p = lambda t: t.data_ptr()
+    st = torch.cuda.current_stream().cuda_stream
+    # zero rows
+    check(L.et_skip_layernorm(p(sentinel), p(x), p(g), p(g), 0, d, st))
+    check(L.et_scatter_skip_layernorm(p(sentinel), p(x), p(ids), 16, 16, p(x), p(g), p(g), 0, d, st))
+    check(L.et_row_spmm_add_bias(p(sentinel), p(x), p(x), p(g), 0, 16, d, st))
+    outs, ws, bs = (C.c_void_p * 1)(p(sentinel)), (C.c_void_p * 1)(p(x)), (C.c_void_p * 1)(p(g))
+    check(L.et_row_spmm_add_bias_multi(outs, p(x), ws, bs, (C.c_int * 1)(16), 1, 0, d, st))
+    lin = make_tile_linear(rng(1), d, d, 0.8, seed=2)
+    from et_amd.encoder import Linear_tile
+    lt = Linear_tile(d, d, 64, lin["row_offset"].size, lin["data"], lin["row_ptr"], lin["row_offset"], lin["bias"])
+    lt.run(x, out=sentinel, rows=0)
+    torch.cuda.synchronize()
+    assert (sentinel == 7).all()
+    # bad arguments
+    for call in (
+        lambda: check(L.et_skip_layernorm(None, p(x), p(g), p(g), 4, d, st)),
+        lambda: check(L.et_skip_layernorm(p(sentinel), p(x), p(g), p(g), -1, d, st)),
+        lambda: check(L.et_scatter_skip_layernorm(p(sentinel), p(sentinel), p(ids), 16, 16, p(x), p(g), p(g), 4, d, st)),
+        lambda: check(L.et_scatter_skip_layernorm(p(sentinel), p(x), p(ids), 32, 16, p(x), p(g), p(g), 4, d, st)),
+        lambda: check(L.et_row_spmm_add_bias(p(sentinel), p(x), p(x), p(g), 4, 24, d, st)),          # N not a multiple of 16
+        lambda: check(L.et_row_spmm_add_bias(p(sentinel) + 2, p(x), p(x), p(g), 4, 16, d, st)),      # misaligned
+        lambda: check(L.et_OTF_attention(p(sentinel), p(x), p(x), p(x), None, 64, 770, 12, 1, None, 1.0, st)),   # d_model % nhead
+        lambda: check(L.et_OTF_attention(p(sentinel), p(x), p(x), p(x), None, 64, 768, 16, 1, None, 1.0, st)),   # head_dim 48
+        lambda: check(L.et_OTF_attention_qk_width(p(sentinel), p(x), p(x), p(x), None, 0, 64, 768, 12, 1, None, 1.0, st)),
+        lambda: check(L.et_pack_rows_ordered(p(sentinel), None, p(ids), p(ids), 2, 8, d, st)),
+    ):
+        with pytest.raises(EtError):
+            call()
+    torch.cuda.synchronize()
+    assert (sentinel == 7).all()
+    assert L.et_last_error().decode() != ""
+
