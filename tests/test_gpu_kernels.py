@@ -584,6 +584,30 @@ def test_attention_mask_summary(K, S):
         check_close(fast, want, max_abs=5e-3, mean_rel=1e-3, what="attention with mask summary")
 
 
+@pytest.mark.parametrize("S,H,d,B,lens", [(2048, 12, 768, 1, [1500]), (4160, 2, 128, 2, [4160, 4097])])
+def test_otf_attention_long_sequences(K, S, H, d, B, lens):
+    """key tiles are walked with running statistics: no limit on seq_len (4160 = 65 tiles is past the
+    64 tiles whose mask summary a workgroup keeps in registers)"""
+    r = rng(48 + S)
+    Q, Kk, V = (randn_h(r, (B * S, d)) for _ in range(3))
+    mask = randn_h(r, (S, S), 0.5)
+    mask[:, S // 2:S // 2 + 300] = 0          # some all-zero mask tiles
+    lens = np.array(lens, np.int32)
+    md = dev(mask)
+    want = orc.otf_attention(Q, Kk, V, mask, S, H, B, lens, 1.0, f64=True)
+    got = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), md, S, H, B, dev(lens), 1.0))
+    summ = K.attention_mask_summary(md, S)
+    K.attention_mask_summary_attach(md, S, summ)
+    try:
+        fast = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), md, S, H, B, dev(lens), 1.0))
+    finally:
+        K.attention_mask_summary_attach(md, S, None)
+    assert np.array_equal(got, fast)
+    valid = np.concatenate([np.arange(S) < n for n in lens])
+    check_close(got[valid], want[valid], max_abs=5e-3, mean_rel=1e-3, what="attention, long sequence")
+    assert (got[~valid] == 0).all()
+
+
 def test_otf_attention_varlen_equals_padded(K):
     r = rng(42)
     S, H, d, B = 256, 12, 768, 4
