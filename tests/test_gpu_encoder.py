@@ -62,6 +62,27 @@ def test_encoder_tile_layer(S, B, sp, ls, use_mask):
     assert np.array_equal(got2, got)
 
 
+@pytest.mark.parametrize("d,H,dff,S,B,sp", [
+    (1024, 16, 4096, 128, 8, 0.8),    # BERT-large widths: K = 1024 needs two panel chunks everywhere
+    (1024, 16, 4096, 64, 1, 0.5),     # ... and on few rows
+    (512, 8, 2048, 96, 40, 0.7),      # 3840 rows of 512: the one-launch tail on another width
+    (384, 12, 1536, 50, 3, 0.6),      # head_dim 32
+    (1024, 8, 2048, 80, 2, 0.8),      # head_dim 128
+])
+def test_encoder_tile_layer_other_widths(d, H, dff, S, B, sp):
+    from et_amd.encoder import Encoder_tile
+    r = rng(540 + d + S)
+    lins, ln = make_layer(r, d, dff, sp, seed=905, std=0.03)
+    x = randn_h(r, (B * S, d))
+    mask = randn_h(r, (S, S), 0.5)
+    want = orc.encoder_tile_layer(x, lins, ln, mask, S, H, B, None, 1.0)
+    enc = Encoder_tile(d, S, H, workspace(Encoder_tile, d, S, H, B), *build_linears(lins, B * S), *ln, mask, B)
+    xd = dev(x)
+    got = host(enc.run(torch.empty_like(xd), xd))
+    check_close(got, want, what=f"Encoder_tile, d_model {d}")
+    assert np.array_equal(host(enc.run(xd, xd)), got)
+
+
 @pytest.mark.parametrize("S,B", [(128, 2), (200, 3)])
 def test_encoder_tile_layer_fused_tail_forced(S, B):
     """the one-launch layer tail (normally used from 96 row panels up) inside Encoder_tile, forced on small shapes"""
