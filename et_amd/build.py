@@ -54,7 +54,23 @@ def build(verbose: bool = False) -> str:
         raise RuntimeError("\n".join(f"--- {s} ---\n{o}" for s, o in failed))
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     subprocess.check_call(cmd)
+    build_examples(verbose)
     return LIB
+
+
+def build_examples(verbose: bool = False) -> str:
+    """The C++ caller of et_amd/examples (the reference's test/tile_test.cu on this library): host C++
+    only, compiled with the ROCm clang++ (half is _Float16) and linked against the library above."""
+    cxx = os.path.join(os.path.dirname(os.path.realpath(hipcc())), "..", "lib", "llvm", "bin", "clang++")
+    if not os.path.exists(cxx):
+        cxx = "/opt/rocm/lib/llvm/bin/clang++"
+    src = os.path.join(HERE, "examples", "tile_test.cpp")
+    exe = os.path.join(HERE, "examples", "tile_test")
+    cmd = [cxx, "-std=c++17", "-O2", "-Wall", "-o", exe, src, "-L", HERE, "-let_amd", "-Wl,-rpath,$ORIGIN/.."]
+    if verbose:
+        print(" ".join(cmd))
+    subprocess.check_call(cmd)
+    return exe
 
 
 if __name__ == "__main__":

@@ -147,7 +147,7 @@ class Linear_row {
         }
         if (in_feat % 16 == 0) {
             const int bcols = in_feat / 16, brows = nrow / 16;
-            std::vector<half> wpad((size_t)nrow * in_feat, (half)0), bpad(nrow, (half)0);
+            std::vector<half> wpad((size_t)nrow * in_feat), bpad(nrow); // (value-initialised: zero)
             std::copy(weight_, weight_ + (size_t)row_id_size * in_feat, wpad.begin());
             std::copy(bias_, bias_ + row_id_size, bpad.begin());
             std::vector<int> rp(brows + 1), ro((size_t)brows * bcols);

@@ -150,3 +150,19 @@ def test_pruned_weight_containers_round_trip_and_reject_damage(tmp_path):
     assert e.value.code == -6
     with pytest.raises(EtError):                                      # unsorted row ids are refused on save
         formats.row_mat_save(tmp_path / "x", K, N, ids[::-1], W[ids], bias)
+
+
+def test_class_headers_compile_with_a_plain_host_compiler(tmp_path):
+    """et_amd/encoder/*.h (the reference's class surface) need no HIP headers: g++ takes them as is"""
+    import shutil
+    import subprocess
+    gxx = shutil.which("g++")
+    if gxx is None:
+        pytest.skip("no g++ here")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    tu = tmp_path / "tu.cpp"
+    tu.write_text('#include "et_amd/encoder/encoder.h"\n'
+                  'size_t f() { return Encoder_tile::buffer_size(768, 128, 12, 2) + Encoder_length::buffer_size(768, 128, 12); }\n')
+    res = subprocess.run([gxx, "-std=c++17", "-Wall", "-fsyntax-only", "-I", root, str(tu)], capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+

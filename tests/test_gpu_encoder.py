@@ -346,3 +346,42 @@ def test_encoder_runs_inside_a_captured_hip_graph():
             again = host(run(torch.empty_like(inputs[k]), inputs[k]))
             assert np.array_equal(again, eager[k])
         del graph
+
+
+def test_cpp_caller_of_the_reference_classes(tmp_path):
+    """et_amd/examples/tile_test.cpp is the reference's test/tile_test.cu on this library's headers (plain
+    C++, no HIP headers, linked with -let_amd).  Its output equals the same layer built through the Python
+    binding, bit for bit, and the oracle within tolerance."""
+    import os
+    import subprocess
+    from et_amd import formats
+    from et_amd.encoder import Encoder_tile, Linear_tile
+    exe = os.path.join(os.path.dirname(os.path.abspath(formats.__file__)), "examples", "tile_test")
+    assert os.path.exists(exe), "built by et_amd.build (build_examples)"
+    S, B, sp = 128, 2, 0.8
+    d, H, dff = 768, 12, 3072
+    out_path = str(tmp_path / "out.bin")
+    res = subprocess.run([exe, out_path, str(S), str(B), str(sp)], capture_output=True, text=True, timeout=110)
+    assert res.returncode == 0, res.stderr
+    got = np.fromfile(out_path, dtype=np.float16).reshape(B * S, d)
+    # the same layer here: seeds 1..6, surviving weights 0.01, biases 0.1, gamma 1, beta 0, zero mask
+    shapes = [(d, d)] * 4 + [(dff, d), (d, dff)]
+    lins = []
+    for seed, (N, Kd) in enumerate(shapes, start=1):
+        rp, ro = formats.gen_sparse_tile_mat(N, Kd, sp, seed)
+        lins.append(dict(N=N, K=Kd, row_ptr=rp, row_offset=ro, data=np.full(ro.size * 256, 0.01, np.float16),
+                         bias=np.full(N, 0.1, np.float16)))
+    s, vals = 12345, np.empty(B * S * d, np.float32)
+    for i in range(vals.size):          # the program's 64-bit LCG
+        s = (s * 6364136223846793005 + 1442695040888963407) & 0xFFFFFFFFFFFFFFFF
+        vals[i] = np.float32(s >> 40) * np.float32(1.0 / 8388608.0) - np.float32(1.0)
+    x = vals.astype(np.float16).reshape(B * S, d)
+    ln = [np.ones(d, np.float16), np.zeros(d, np.float16)] * 2
+    mask = np.zeros((S, S), np.float16)
+    enc = Encoder_tile(d, S, H, workspace(Encoder_tile, d, S, H, B), *build_linears(lins, B * S), *ln, mask, B)
+    xd = dev(x)
+    same = host(enc.run(torch.empty_like(xd), xd))
+    assert np.array_equal(got, same)
+    want = orc.encoder_tile_layer(x, lins, ln, mask, S, H, B, None, 1.0)
+    check_close(got, want, what="C++ caller")
+
