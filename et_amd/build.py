@@ -59,18 +59,20 @@ def build(verbose: bool = False) -> str:
 
 
 def build_examples(verbose: bool = False) -> str:
-    """The C++ caller of et_amd/examples (the reference's test/tile_test.cu on this library): host C++
+    """The C++ callers of et_amd/examples (the reference's three test programs on this library): host C++
     only, compiled with the ROCm clang++ (half is _Float16) and linked against the library above."""
     cxx = os.path.join(os.path.dirname(os.path.realpath(hipcc())), "..", "lib", "llvm", "bin", "clang++")
     if not os.path.exists(cxx):
         cxx = "/opt/rocm/lib/llvm/bin/clang++"
-    src = os.path.join(HERE, "examples", "tile_test.cpp")
-    exe = os.path.join(HERE, "examples", "tile_test")
-    cmd = [cxx, "-std=c++17", "-O2", "-Wall", "-o", exe, src, "-L", HERE, "-let_amd", "-Wl,-rpath,$ORIGIN/.."]
-    if verbose:
-        print(" ".join(cmd))
-    subprocess.check_call(cmd)
-    return exe
+    exe = ""
+    for name in ("tile_test", "prune_test", "length_test"):
+        src = os.path.join(HERE, "examples", name + ".cpp")
+        exe = os.path.join(HERE, "examples", name)
+        cmd = [cxx, "-std=c++17", "-O2", "-Wall", "-o", exe, src, "-L", HERE, "-let_amd", "-Wl,-rpath,$ORIGIN/.."]
+        if verbose:
+            print(" ".join(cmd))
+        subprocess.check_call(cmd)
+    return os.path.dirname(exe)
 
 
 if __name__ == "__main__":

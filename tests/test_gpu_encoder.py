@@ -348,22 +348,23 @@ def test_encoder_runs_inside_a_captured_hip_graph():
         del graph
 
 
-def test_cpp_caller_of_the_reference_classes(tmp_path):
-    """et_amd/examples/tile_test.cpp is the reference's test/tile_test.cu on this library's headers (plain
-    C++, no HIP headers, linked with -let_amd).  Its output equals the same layer built through the Python
-    binding, bit for bit, and the oracle within tolerance."""
+@pytest.mark.parametrize("program", ["tile_test", "prune_test", "length_test"])
+def test_cpp_caller_of_the_reference_classes(tmp_path, program):
+    """et_amd/examples/*.cpp are the reference's test/tile_test.cu, prune_test.cu and length_test.cu on this
+    library's headers (plain C++, no HIP headers, linked with -let_amd).  Each one's output equals the same
+    layer built through the Python binding, bit for bit, and the oracle within tolerance."""
     import os
     import subprocess
     from et_amd import formats
-    from et_amd.encoder import Encoder_tile, Linear_tile
-    exe = os.path.join(os.path.dirname(os.path.abspath(formats.__file__)), "examples", "tile_test")
+    from et_amd.encoder import Encoder_length, Encoder_prune, Encoder_tile, Linear_row
+    exe = os.path.join(os.path.dirname(os.path.abspath(formats.__file__)), "examples", program)
     assert os.path.exists(exe), "built by et_amd.build (build_examples)"
     S, B, sp = 128, 2, 0.8
     d, H, dff = 768, 12, 3072
     out_path = str(tmp_path / "out.bin")
     res = subprocess.run([exe, out_path, str(S), str(B), str(sp)], capture_output=True, text=True, timeout=110)
     assert res.returncode == 0, res.stderr
-    got = np.fromfile(out_path, dtype=np.float16).reshape(B * S, d)
+    got = np.fromfile(out_path, dtype=np.float16).reshape(-1, d)
     # the same layer here: seeds 1..6, surviving weights 0.01, biases 0.1, gamma 1, beta 0, zero mask
     shapes = [(d, d)] * 4 + [(dff, d), (d, dff)]
     lins = []
@@ -372,16 +373,39 @@ def test_cpp_caller_of_the_reference_classes(tmp_path):
         lins.append(dict(N=N, K=Kd, row_ptr=rp, row_offset=ro, data=np.full(ro.size * 256, 0.01, np.float16),
                          bias=np.full(N, 0.1, np.float16)))
     s, vals = 12345, np.empty(B * S * d, np.float32)
-    for i in range(vals.size):          # the program's 64-bit LCG
+    for i in range(vals.size):          # the programs' 64-bit LCG
         s = (s * 6364136223846793005 + 1442695040888963407) & 0xFFFFFFFFFFFFFFFF
         vals[i] = np.float32(s >> 40) * np.float32(1.0 / 8388608.0) - np.float32(1.0)
     x = vals.astype(np.float16).reshape(B * S, d)
     ln = [np.ones(d, np.float16), np.zeros(d, np.float16)] * 2
     mask = np.zeros((S, S), np.float16)
-    enc = Encoder_tile(d, S, H, workspace(Encoder_tile, d, S, H, B), *build_linears(lins, B * S), *ln, mask, B)
     xd = dev(x)
-    same = host(enc.run(torch.empty_like(xd), xd))
-    assert np.array_equal(got, same)
-    want = orc.encoder_tile_layer(x, lins, ln, mask, S, H, B, None, 1.0)
-    check_close(got, want, what="C++ caller")
-
+    L = build_linears(lins, B * S)
+    if program == "tile_test":
+        enc = Encoder_tile(d, S, H, workspace(Encoder_tile, d, S, H, B), *L, *ln, mask, B)
+        same = host(enc.run(torch.empty_like(xd), xd))
+        want = orc.encoder_tile_layer(x, lins, ln, mask, S, H, B, None, 1.0)
+    elif program == "prune_test":
+        v_id = formats.gen_sparse_row_mat(d, sp, 3)
+        Wv, bv = np.full((v_id.size, d), 0.01, np.float16), np.full(v_id.size, 0.1, np.float16)
+        L[2] = Linear_row(d, d, B * S, Wv, v_id, v_id.size, bv, H)
+        enc = Encoder_prune(d, S, H, workspace(Encoder_prune, d, S, H, B), *L, *ln, mask, B)
+        same = host(enc.run(torch.empty_like(xd), xd))
+        tl = lambda j, inp, g=False: orc.tile_linear(inp, lins[j]["row_ptr"], lins[j]["row_offset"],
+                                                     lins[j]["data"], lins[j]["bias"], lins[j]["N"], gelu=g)
+        z = orc.prune_attention(tl(0, x), tl(1, x), orc.row_linear(x, Wv, bv), None, v_id,
+                                orc.head_ptr(v_id, H, d // H), mask, S, d, H, B)
+        h1 = orc.skip_layernorm(tl(3, z), x, ln[0], ln[1])
+        want = orc.skip_layernorm(tl(5, tl(4, h1, True)), h1, ln[2], ln[3])
+    else:
+        enc = Encoder_length(d, S, H, workspace(Encoder_length, d, S, H, B), *L, *ln, mask, B)
+        full = host(enc.run(torch.empty_like(xd), xd))
+        lens = np.array([max(S - 7 * b, 1) for b in range(B)], np.int32)
+        enc.set_seq_lens(lens)
+        same = np.concatenate([full, host(enc.run(torch.empty_like(xd), xd))])
+        want = np.concatenate([orc.encoder_tile_layer(x, lins, ln, mask, S, H, B, None, 1.0),
+                               orc.encoder_tile_layer(x, lins, ln, mask, S, H, B, lens, 1.0)])
+        for b in range(B):              # padding rows of the packed run are zero on the device
+            want[B * S + b * S + lens[b]:B * S + (b + 1) * S] = 0
+    assert got.shape == same.shape and np.array_equal(got, same)
+    check_close(got, want, what="C++ caller " + program)
