@@ -180,11 +180,24 @@ def test_encoder_attnaware_layer_config4_wiring(balanced):
     rows are zero (and, for FFN2, the dropped hidden units' columns).  balanced = False moves 12 kept
     columns from head 0 to head 1 (20 and 44 columns): the ragged pruned-attention kernel instead of the
     narrow-head one."""
+    attnaware_case(S=64, B=2, balanced=balanced, sample=[0, 1])
+
+
+def test_encoder_attnaware_layer_config4_full_size():
+    """the same layer at BASELINE config 4's size (batch 32 x seq 256).  Sequences do not interact, so the
+    oracle runs three of them as a batch of their own and the full launch must agree on their rows."""
+    attnaware_case(S=256, B=32, balanced=True, sample=[0, 17, 31])
+
+
+def attnaware_case(S, B, balanced, sample):
     from et_amd.encoder import Encoder_attnaware, Linear_row, Linear_tile
     r = rng(650)
-    d, H, dff, S, B = 768, 12, 3072, 64, 2
-    hd, T = d // H, B * S
-    x = randn_h(r, (T, d))
+    d, H, dff = 768, 12, 3072
+    hd = d // H
+    x_all = randn_h(r, (B * S, d))
+    rows = np.concatenate([np.arange(b * S, (b + 1) * S) for b in sample])
+    x, Bfull, B = x_all[rows], B, len(sample)   # the oracle's batch: the sampled sequences
+    T = B * S
     mask = randn_h(r, (S, S), 0.5)
     ln = [randn_h(r, (d,), 0.2) + np.float16(1), randn_h(r, (d,), 0.2), randn_h(r, (d,), 0.2) + np.float16(1), randn_h(r, (d,), 0.2)]
     W = {k: randn_h(r, shp, 0.03) for k, shp in dict(q=(d, d), k=(d, d), v=(d, d), o=(d, d), m1=(dff, d), m2=(d, dff)).items()}
@@ -235,6 +248,7 @@ def test_encoder_attnaware_layer_config4_wiring(balanced):
     vt = dict(N=d, K=d)
     vt["row_ptr"], vt["row_offset"] = orc.gen_sparse_tile_mat(d, d, 0.0, seed=1)
     vt["data"] = orc.tile_pack(W["v"], vt["row_ptr"], vt["row_offset"])
+    B, T = Bfull, Bfull * S                     # the device runs the whole batch
     Lq = Linear_row(d, d, T, W["q"][qk_id], qk_id, qk_id.size, bsz["q"][qk_id], H)
     Lk = Linear_row(d, d, T, W["k"][qk_id], qk_id, qk_id.size, bsz["k"][qk_id], H)
     Lv = Linear_tile(d, d, T, vt["row_offset"].size, vt["data"], vt["row_ptr"], vt["row_offset"], bsz["v"], False)
@@ -243,8 +257,8 @@ def test_encoder_attnaware_layer_config4_wiring(balanced):
     L2 = Linear_row(pad16(m1_id.size), d, T, W2c, m2_id, m2_id.size, bsz["m2"][m2_id], H)
     assert (Lq.nrow, Lo.nrow, L1.nrow, L2.nrow) == (384, 240, 928, 240)
     enc = Encoder_attnaware(d, S, H, workspace(Encoder_attnaware, d, S, H, B), Lq, Lk, Lv, Lo, L1, L2, *ln, mask, B)
-    xd = dev(x)
-    got = host(enc.run(torch.empty_like(xd), xd))
+    xd = dev(x_all)
+    got = host(enc.run(torch.empty_like(xd), xd))[rows]
     check_close(got, want, what="Encoder_attnaware")
     check_close(got, outd, what="Encoder_attnaware vs dense-with-zeroed-rows")
 
@@ -305,6 +319,43 @@ def test_encoder_stack_variable_length():
     for lins, ln in params:
         cur = orc.encoder_tile_layer(cur, lins, ln, None, S, H, B, None, 1.0)
     check_close(got_full, cur, what="stack full length")
+
+
+def test_encoder_stack_config5_full_size():
+    """BASELINE config 5 at its size: 12 BERT-base layers, 80 % tile-pruned, batch 64, lengths drawn from
+    32..512 and padded to 512.  Sequences do not interact, so the oracle runs three of them (the shortest,
+    a middle one, the longest) one at a time through the 12 layers; the packed run must agree on their
+    valid rows and leave their padding rows zero, and the padded run on the shortest one's 512 rows.
+    Tolerance for TWELVE layers: max-abs 4e-2, mean-rel 3e-3 (one layer's is 2e-2 / 1e-3)."""
+    from et_amd.encoder import Encoder_length, Encoder_stack
+    r = rng(810)
+    d, H, dff, S, B, NL = 768, 12, 3072, 512, 64, 12
+    lens = r.integers(32, 513, size=B).astype(np.int32)
+    layers, params = [], []
+    for i in range(NL):
+        lins, ln = make_layer(r, d, dff, 0.8, seed=1000 + 10 * i)
+        params.append((lins, ln))
+        layers.append(Encoder_length(d, S, H, workspace(Encoder_length, d, S, H, B), *build_linears(lins, B * S), *ln, None, B))
+    x = randn_h(r, (B * S, d))
+    stack = Encoder_stack(layers, d, S, B)
+    stack.set_seq_lens(lens)
+    xd = dev(x)
+    got = host(stack.run(torch.empty_like(xd), xd))
+    order = np.argsort(lens, kind="stable")
+    def oracle_seq(b, n):
+        cur = x[b * S:(b + 1) * S]
+        for lins, ln in params:
+            cur = orc.encoder_tile_layer(cur, lins, ln, None, S, H, 1, None if n == S else np.array([n], np.int32), 1.0)
+        return cur
+    for b in (order[0], order[B // 2], order[-1]):
+        want = oracle_seq(b, lens[b])
+        check_close(got[b * S:b * S + lens[b]], want[:lens[b]], max_abs=4e-2, mean_rel=3e-3, what=f"packed stack, seq {b} ({lens[b]} rows)")
+    for b in range(B):
+        assert (got[b * S + lens[b]:(b + 1) * S] == 0).all()
+    stack.set_seq_lens(None)
+    got_full = host(stack.run(torch.empty_like(xd), xd))
+    b = order[0]
+    check_close(got_full[b * S:(b + 1) * S], oracle_seq(b, S), max_abs=4e-2, mean_rel=3e-3, what="padded stack")
 
 
 def test_encoder_runs_inside_a_captured_hip_graph():
