@@ -62,6 +62,26 @@ def test_encoder_tile_layer(S, B, sp, ls, use_mask):
     assert np.array_equal(got2, got)
 
 
+def test_encoder_tile_layer_config3_full_size():
+    """BASELINE config 3 at its size (batch 16 x seq 512, 80 % tiles, zero additive mask - the benchmark's
+    workload): sequences do not interact, so the oracle runs two of them as a batch of their own and the
+    full launch must agree on their rows; in place gives the same bits."""
+    from et_amd.encoder import Encoder_tile
+    r = rng(560)
+    d, H, dff, S, B = 768, 12, 3072, 512, 16
+    lins, ln = make_layer(r, d, dff, 0.8, seed=905)
+    x = randn_h(r, (B * S, d))
+    mask = np.zeros((S, S), np.float16)
+    sample = [3, 15]
+    rows = np.concatenate([np.arange(b * S, (b + 1) * S) for b in sample])
+    want = orc.encoder_tile_layer(x[rows], lins, ln, mask, S, H, len(sample), None, 1.0)
+    enc = Encoder_tile(d, S, H, workspace(Encoder_tile, d, S, H, B), *build_linears(lins, B * S), *ln, mask, B)
+    xd = dev(x)
+    got = host(enc.run(torch.empty_like(xd), xd))
+    check_close(got[rows], want, what="Encoder_tile, config 3 full size")
+    assert np.array_equal(host(enc.run(xd, xd)), got)
+
+
 @pytest.mark.parametrize("d,H,dff,S,B,sp", [
     (1024, 16, 4096, 128, 8, 0.8),    # BERT-large widths: K = 1024 needs two panel chunks everywhere
     (1024, 16, 4096, 64, 1, 0.5),     # ... and on few rows

@@ -455,12 +455,14 @@ def test_row_linear_multi_one_launch(K):
         check_close(host(o), want, max_abs=8e-3, mean_rel=5e-4, what="row linears, few rows")
 
 
-def test_tile_linear_full_size_config2_rows_sample(K):
-    """config-2 shape (4096x768 -> 3072, 80 %): rows are independent, so a row sample pins the full-size launch"""
+@pytest.mark.parametrize("sp,ntile", [(0.8, 1843), (0.0, 9216), (0.5, 4608), (0.9, 921)])
+def test_tile_linear_full_size_config2_rows_sample(K, sp, ntile):
+    """config-2 shape (4096x768 -> 3072) at each sparsity of its sweep: rows are independent, so a row
+    sample pins the full-size launch"""
     r = rng(32)
     M, N, Kd = 4096, 3072, 768
-    lin = make_tile_linear(r, N, Kd, 0.8, seed=2024, std=0.02)
-    assert lin["row_offset"].size == 1843
+    lin = make_tile_linear(r, N, Kd, sp, seed=2024, std=0.02)
+    assert lin["row_offset"].size == ntile
     X = randn_h(r, (M, Kd))
     got = host(K.tile_spmm_add_bias(dev(X), dev(lin["row_ptr"]), dev(lin["row_offset"]), dev(lin["data"]), dev(lin["bias"]), N))
     rows = np.sort(r.choice(M, 192, replace=False))
