@@ -35,6 +35,14 @@ def _dp(t):
     return t.data_ptr()
 
 
+def _dp2(t, rows, cols, what):
+    """device pointer of a [>= rows x cols] half tensor.  The C ABI takes bare pointers and cannot know a
+    buffer's extent: an operand of the wrong shape is refused here, before a kernel reads or writes past it."""
+    if t.dim() != 2 or t.shape[0] < rows or t.shape[1] != cols:
+        raise ValueError(f"{what}: expected at least {rows} rows of {cols} columns, got {tuple(t.shape)}")
+    return _dp(t)
+
+
 class Linear_tile:
     """encoder/Linear.h:4-46"""
 
@@ -51,15 +59,18 @@ class Linear_tile:
     def run(self, x, out=None, rows=None):
         rows = x.shape[0] if rows is None else rows
         out = out if out is not None else torch.empty((x.shape[0], self.out_feat), dtype=torch.float16, device=x.device)
-        check(lib().et_linear_tile_run_rows(self._h, _dp(out), _dp(x), rows, _stream()))
+        check(lib().et_linear_tile_run_rows(self._h, _dp2(out, rows, self.out_feat, "Linear_tile.run out"),
+                                            _dp2(x, rows, self.in_feat, "Linear_tile.run x"), rows, _stream()))
         return out
 
     def run_ln(self, x, skip, gamma, beta, out=None, rows=None):
         """LayerNorm(half(linear(x)) + skip) * gamma + beta in one launch"""
         rows = x.shape[0] if rows is None else rows
         out = out if out is not None else torch.empty((x.shape[0], self.out_feat), dtype=torch.float16, device=x.device)
-        check(lib().et_linear_tile_run_rows_ln(self._h, _dp(out), _dp(x), _dp(skip), _dp(gamma), _dp(beta),
-                                               rows, _stream()))
+        check(lib().et_linear_tile_run_rows_ln(self._h, _dp2(out, rows, self.out_feat, "Linear_tile.run_ln out"),
+                                               _dp2(x, rows, self.in_feat, "Linear_tile.run_ln x"),
+                                               _dp2(skip, rows, self.out_feat, "Linear_tile.run_ln skip"),
+                                               _dp(gamma), _dp(beta), rows, _stream()))
         return out
 
     @staticmethod
@@ -69,8 +80,11 @@ class Linear_tile:
         None insists on the fused kernel."""
         rows = x.shape[0] if rows is None else rows
         out = out if out is not None else torch.empty((x.shape[0], second.out_feat), dtype=torch.float16, device=x.device)
-        check(lib().et_linear_tile_run_rows_ffn_ln(first._h, second._h, _dp(out), _dp(x),
-                                                   _dp(hidden) if hidden is not None else None, _dp(skip),
+        what = "Linear_tile.run_ffn_ln"
+        check(lib().et_linear_tile_run_rows_ffn_ln(first._h, second._h, _dp2(out, rows, second.out_feat, what + " out"),
+                                                   _dp2(x, rows, first.in_feat, what + " x"),
+                                                   _dp2(hidden, rows, first.out_feat, what + " hidden") if hidden is not None else None,
+                                                   _dp2(skip, rows, second.out_feat, what + " skip"),
                                                    _dp(gamma), _dp(beta), rows, _stream()))
         return out
 
@@ -85,9 +99,14 @@ class Linear_tile:
         LayerNorm.  `mid` / `hidden` are only used where the fused kernel does not apply; mid=None insists on it."""
         rows = attn.shape[0] if rows is None else rows
         out = out if out is not None else torch.empty((attn.shape[0], second.out_feat), dtype=torch.float16, device=attn.device)
-        opt = lambda t: _dp(t) if t is not None else None
-        check(lib().et_linear_tile_run_rows_tail(out_proj._h, first._h, second._h, _dp(out), _dp(attn), _dp(inp),
-                                                 opt(mid), opt(hidden), _dp(gamma1), _dp(beta1), _dp(gamma2),
+        what = "Linear_tile.run_tail"
+        opt = lambda t, cols, name: _dp2(t, rows, cols, what + name) if t is not None else None
+        check(lib().et_linear_tile_run_rows_tail(out_proj._h, first._h, second._h,
+                                                 _dp2(out, rows, second.out_feat, what + " out"),
+                                                 _dp2(attn, rows, out_proj.in_feat, what + " attn"),
+                                                 _dp2(inp, rows, out_proj.out_feat, what + " inp"),
+                                                 opt(mid, out_proj.out_feat, " mid"), opt(hidden, first.out_feat, " hidden"),
+                                                 _dp(gamma1), _dp(beta1), _dp(gamma2),
                                                  _dp(beta2), rows, _stream()))
         return out
 
@@ -133,8 +152,8 @@ class Linear_row:
 
     def run(self, x, out=None):
         out = out if out is not None else torch.empty((x.shape[0], self.nrow), dtype=torch.float16, device=x.device)
-        assert x.shape[0] == self.size
-        check(lib().et_linear_row_run(self._h, _dp(out), _dp(x), _stream()))
+        check(lib().et_linear_row_run(self._h, _dp2(out, self.size, self.nrow, "Linear_row.run out"),
+                                      _dp2(x, self.size, self.in_feat, "Linear_row.run x"), _stream()))
         return out
 
     def _release(self):
@@ -177,7 +196,9 @@ class _Encoder:
     def run(self, out, inp):
         """out, inp: [batch*seq_len, d_model] device tensors; out may be inp"""
         check(lib().et_encoder_set_stream(self._h, _stream()))
-        check(lib().et_encoder_run(self._h, _dp(out), _dp(inp)))
+        rows = self.batch * self.seq_len
+        check(lib().et_encoder_run(self._h, _dp2(out, rows, self.d_model, "Encoder.run out"),
+                                   _dp2(inp, rows, self.d_model, "Encoder.run inp")))
         return out
 
     def set_log2_scale(self, v):
@@ -245,7 +266,8 @@ class Encoder_stack:
     def run(self, out, inp):
         if self.act is None or self.act.device != inp.device:
             self.act = torch.empty(self.shape, dtype=torch.float16, device=inp.device)
-        check(lib().et_encoder_stack_run(self._h, _dp(out), _dp(inp), _dp(self.act), _stream()))
+        check(lib().et_encoder_stack_run(self._h, _dp2(out, *self.shape, "Encoder_stack.run out"),
+                                         _dp2(inp, *self.shape, "Encoder_stack.run inp"), _dp(self.act), _stream()))
         return out
 
     def __del__(self):

@@ -166,3 +166,16 @@ def test_class_headers_compile_with_a_plain_host_compiler(tmp_path):
     res = subprocess.run([gxx, "-std=c++17", "-Wall", "-fsyntax-only", "-I", root, str(tu)], capture_output=True, text=True)
     assert res.returncode == 0, res.stderr
 
+
+
+def test_python_binding_refuses_operands_of_the_wrong_shape():
+    """the C ABI takes bare pointers; the Python classes check every operand's shape before a launch, so a
+    swapped (x, out) pair or a short buffer is an error here and not a kernel writing past a buffer"""
+    import torch
+    from et_amd import encoder
+    ok = torch.empty((8, 16), dtype=torch.float16)
+    for rows, cols in ((8, 32), (9, 16)):                # wrong width, too few rows
+        with pytest.raises(ValueError):
+            encoder._dp2(ok, rows, cols, "operand")
+    with pytest.raises(ValueError):
+        encoder._dp2(ok.reshape(-1), 8, 16, "operand")   # not two-dimensional
