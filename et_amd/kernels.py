@@ -33,9 +33,24 @@ def _i32(t):
     return _p(t)
 
 
+def _want(t, what, *shape):
+    """The C ABI takes bare pointers and cannot know a buffer's extent: the extents that the other
+    arguments imply are checked here, before a kernel reads or writes past a tensor.  A single number
+    is an element count, several are the exact shape; None tensors (optional operands) pass."""
+    if t is None:
+        return
+    ok = t.numel() == shape[0] if len(shape) == 1 else tuple(t.shape) == tuple(shape)
+    if not ok:
+        raise ValueError(f"{what}: expected {shape[0] if len(shape) == 1 else tuple(shape)} "
+                         f"{'elements' if len(shape) == 1 else ''}, got {tuple(t.shape)}")
+
+
 def skip_layernorm(in_out, skip, gamma, beta):
     """in place on in_out[num x size]; kernels/kernels.h:3-5"""
     num, size = in_out.shape
+    _want(skip, "skip_layernorm skip", num, size)
+    _want(gamma, "skip_layernorm gamma", size)
+    _want(beta, "skip_layernorm beta", size)
     check(lib().et_skip_layernorm(_h(in_out), _h(skip), _h(gamma), _h(beta), num, size, _stream()))
     return in_out
 
@@ -44,6 +59,9 @@ def tile_spmm_add_bias(X, row_ptr, row_offset, data, bias, N, gelu=False, out=No
     """Y = X W^T + bias with W as tile_mat; kernels/kernels.h:13-20"""
     M, K = X.shape
     Y = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=X.device)
+    _want(Y, "tile_spmm_add_bias out", M, N)
+    _want(bias, "tile_spmm_add_bias bias", N)
+    _want(data, "tile_spmm_add_bias data", (0 if row_offset is None else row_offset.numel()) * 256)
     fn = lib().et_tile_spmm_add_bias_gelu if gelu else lib().et_tile_spmm_add_bias
     check(fn(_h(Y), _h(X), _i32(row_ptr), _i32(row_offset), _h(data), M, N, K, _h(bias), _stream()))
     return Y
@@ -54,6 +72,9 @@ def row_spmm_add_bias(X, weight, bias, out=None, gelu=False):
     M, K = X.shape
     N = weight.shape[0]
     Y = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=X.device)
+    _want(Y, "row_spmm_add_bias out", M, N)
+    _want(weight, "row_spmm_add_bias weight", N, K)
+    _want(bias, "row_spmm_add_bias bias", N)
     fn = lib().et_row_spmm_add_bias_gelu if gelu else lib().et_row_spmm_add_bias
     check(fn(_h(Y), _h(X), _h(weight), _h(bias), M, N, K, _stream()))
     return Y
@@ -75,6 +96,10 @@ def OTF_attention(Q, K, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2_sc
     """kernels/kernels.h:22-24 (+ batch, seq_lens, exponent base)"""
     d_model = Q.shape[1]
     Z = out if out is not None else torch.empty_like(Q)
+    for t, name in ((Q, "Q"), (K, "K"), (V, "V"), (Z, "out")):
+        _want(t, "OTF_attention " + name, batch * seq_len, d_model)
+    _want(mask, "OTF_attention mask", seq_len * seq_len)
+    _want(seq_lens, "OTF_attention seq_lens", batch)
     check(lib().et_OTF_attention(_h(Z), _h(Q), _h(K), _h(V), _h(mask), seq_len, d_model, nhead, batch,
                                  _i32(seq_lens), log2_scale, _stream()))
     return Z
@@ -84,6 +109,12 @@ def OTF_attention_qk_width(Q, K, V, mask, qk_width, seq_len, nhead, batch=1, seq
     """Q, K compact [rows x nhead*qk_width] (the same number of kept columns in every head); V full width"""
     d_model = V.shape[1]
     Z = out if out is not None else torch.empty_like(V)
+    for t, name in ((Q, "Q"), (K, "K")):
+        _want(t, "OTF_attention_qk_width " + name, batch * seq_len, nhead * qk_width)
+    for t, name in ((V, "V"), (Z, "out")):
+        _want(t, "OTF_attention_qk_width " + name, batch * seq_len, d_model)
+    _want(mask, "OTF_attention_qk_width mask", seq_len * seq_len)
+    _want(seq_lens, "OTF_attention_qk_width seq_lens", batch)
     check(lib().et_OTF_attention_qk_width(_h(Z), _h(Q), _h(K), _h(V), _h(mask), qk_width, seq_len, d_model, nhead,
                                           batch, _i32(seq_lens), log2_scale, _stream()))
     return Z
@@ -93,6 +124,9 @@ def OTF_attention_varlen(Q, K, V, mask, cu_seqlens, max_seq_len, nhead, log2_sca
     d_model = Q.shape[1]
     batch = cu_seqlens.numel() - 1
     Z = out if out is not None else torch.empty_like(Q)
+    for t, name in ((K, "K"), (V, "V"), (Z, "out")):
+        _want(t, "OTF_attention_varlen " + name, *Q.shape)
+    _want(mask, "OTF_attention_varlen mask", max_seq_len * max_seq_len)
     check(lib().et_OTF_attention_varlen(_h(Z), _h(Q), _h(K), _h(V), _h(mask), _i32(cu_seqlens), max_seq_len,
                                         d_model, nhead, batch, log2_scale, _stream()))
     return Z
@@ -103,6 +137,13 @@ def Prune_attention(Q, K, V, qk_head_ptr, v_col_id, v_head_ptr, mask, seq_len, d
     """kernels/kernels.h:26-30 (+ compact Q/K, batch, seq_lens, exponent base)"""
     rows = Q.shape[0]
     Z = out if out is not None else torch.empty((rows, d_model), dtype=torch.float16, device=Q.device)
+    _want(Z, "Prune_attention out", batch * seq_len, d_model)
+    for t, name in ((Q, "Q"), (K, "K"), (V, "V")):
+        if t.dim() != 2 or t.shape[0] != batch * seq_len:
+            raise ValueError(f"Prune_attention {name}: expected {batch * seq_len} rows, got {tuple(t.shape)}")
+    _want(K, "Prune_attention K", *Q.shape)
+    _want(mask, "Prune_attention mask", seq_len * seq_len)
+    _want(seq_lens, "Prune_attention seq_lens", batch)
     check(lib().et_Prune_attention(_h(Z), _h(Q), _h(K), _h(V), _i32(qk_head_ptr), Q.shape[1], _i32(v_col_id),
                                    _i32(v_head_ptr), V.shape[1], _h(mask), seq_len, d_model, nhead, batch,
                                    _i32(seq_lens), log2_scale, _stream()))
@@ -121,6 +162,11 @@ def sharedQK_attention(QK, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2
     """kernels/kernels.h:32-34"""
     d_model = V.shape[1]
     Z = out if out is not None else torch.empty_like(V)
+    _want(QK, "sharedQK_attention QK", batch * nhead * seq_len * seq_len)
+    for t, name in ((V, "V"), (Z, "out")):
+        _want(t, "sharedQK_attention " + name, batch * seq_len, d_model)
+    _want(mask, "sharedQK_attention mask", seq_len * seq_len)
+    _want(seq_lens, "sharedQK_attention seq_lens", batch)
     check(lib().et_sharedQK_attention(_h(Z), _h(QK), _h(V), _h(mask), seq_len, d_model, nhead, batch,
                                       _i32(seq_lens), log2_scale, _stream()))
     return Z
@@ -157,6 +203,10 @@ def scatter_skip_layernorm(compact, col_id, skip, gamma, beta, out=None):
     rows, ld = compact.shape
     width = skip.shape[1]
     out = torch.empty_like(skip) if out is None else out
+    _want(skip, "scatter_skip_layernorm skip", rows, width)
+    _want(out, "scatter_skip_layernorm out", rows, width)
+    _want(gamma, "scatter_skip_layernorm gamma", width)
+    _want(beta, "scatter_skip_layernorm beta", width)
     check(lib().et_scatter_skip_layernorm(_h(out), _h(compact), _i32(col_id), col_id.numel(), ld, _h(skip),
                                           _h(gamma), _h(beta), rows, width, _stream()))
     return out

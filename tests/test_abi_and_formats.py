@@ -179,3 +179,19 @@ def test_python_binding_refuses_operands_of_the_wrong_shape():
             encoder._dp2(ok, rows, cols, "operand")
     with pytest.raises(ValueError):
         encoder._dp2(ok.reshape(-1), 8, 16, "operand")   # not two-dimensional
+
+
+def test_kernel_wrappers_refuse_operands_of_the_wrong_extent():
+    """the same for the per-kernel wrappers: an extent that the other arguments imply is checked before
+    anything is launched (here on host tensors, which the check meets before it would ask for a device)"""
+    import torch
+    from et_amd import kernels
+    h = lambda *shape: torch.zeros(shape, dtype=torch.float16)
+    with pytest.raises(ValueError):     # out narrower than N
+        kernels.row_spmm_add_bias(h(8, 32), h(16, 32), h(16), out=h(8, 8))
+    with pytest.raises(ValueError):     # skip with fewer rows
+        kernels.skip_layernorm(h(8, 64), h(4, 64), h(64), h(64))
+    with pytest.raises(ValueError):     # K of another sequence length
+        kernels.OTF_attention(h(32, 64), h(16, 64), h(32, 64), None, 32, 1)
+    with pytest.raises(ValueError):     # mask of another sequence length
+        kernels.OTF_attention(h(32, 64), h(32, 64), h(32, 64), h(16, 16), 32, 1)

@@ -483,7 +483,7 @@ def test_tile_linear_argument_errors(K):
     lin = make_tile_linear(r, 32, 32, 0.0, seed=1)
     X = dev(randn_h(r, (16, 32)))
     with pytest.raises(EtError):   # N not a multiple of 16
-        K.tile_spmm_add_bias(X, dev(lin["row_ptr"]), dev(lin["row_offset"]), dev(lin["data"]), dev(lin["bias"]), 24)
+        K.tile_spmm_add_bias(X, dev(lin["row_ptr"]), dev(lin["row_offset"]), dev(lin["data"]), dev(lin["bias"][:24]), 24)
     with pytest.raises(EtError):   # misaligned X
         K.tile_spmm_add_bias(dev(randn_h(r, (17, 32))).view(-1)[1:1 + 16 * 32].view(16, 32), dev(lin["row_ptr"]),
                              dev(lin["row_offset"]), dev(lin["data"]), dev(lin["bias"]), 32)
