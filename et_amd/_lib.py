@@ -26,6 +26,7 @@ PROTOTYPES = {
     "et_row_spmm_add_bias_multi": (_i, [C.POINTER(_vp), _vp, C.POINTER(_vp), C.POINTER(_vp), _ip, _i, _i, _i, _vp]),
     "et_row_spmm_prefers_gemm": (_i, [_i, _i, _i]),
     "et_OTF_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _ip, _f, _vp]),
+    "et_OTF_attention_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _ip, _f, _vp]),
     "et_attention_mask_summary_bytes": (C.c_size_t, [_i]),
     "et_attention_mask_summary": (_i, [_vp, _i, _vp, _vp]),
     "et_attention_mask_summary_attach": (_i, [_vp, _i, _vp]),

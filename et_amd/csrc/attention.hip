@@ -846,8 +846,11 @@ static bool attach_mask_summary(AttnArgs &a) {
 }
 
 // qk_width: columns per head in Q and K (0 = head_dim)
+// given_summary: a summary of a.mask supplied by the caller of this function
+// (it then replaces the lookup among the attached ones)
 static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedqk,
-                              hipStream_t st, const char *who, int qk_width = 0) {
+                              hipStream_t st, const char *who, int qk_width = 0,
+                              const unsigned *given_summary = nullptr) {
     ET_REQUIRE(a.out && a.V, ET_ERR_INVALID_ARG, "%s: null pointer", who);
     ET_REQUIRE(sharedqk ? a.QK != nullptr : (a.Q && a.K), ET_ERR_INVALID_ARG, "%s: null pointer", who);
     ET_REQUIRE(a.seq_len > 0 && d_model > 0 && a.nhead > 0 && a.batch > 0, ET_ERR_INVALID_ARG,
@@ -864,7 +867,14 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
     }
     a.ldo = d_model;
     a.scale = head_scale(hd);
-    const bool no_mask = attach_mask_summary(a);
+    bool no_mask;
+    if (given_summary && a.mask) {
+        a.msum = given_summary;
+        a.msum_words = mask_summary_words(a.seq_len);
+        no_mask = false; // its bits are only known on the device
+    } else {
+        no_mask = attach_mask_summary(a);
+    }
     // 128 query rows per workgroup when that still fills the chip, else 64
     int variant = 0;
     {
@@ -925,6 +935,75 @@ extern "C" int et_OTF_attention(void *out, const void *Q, const void *K, const v
     a.log2_scale = log2_scale;
     return attention_dispatch(a, d_model, false, false, static_cast<hipStream_t>(stream),
                               "et_OTF_attention");
+}
+
+// ---- the entry point that allocates nothing --------------------------------
+// Its scratch memory is the summary of the mask (one bit per 16 query rows x 64
+// keys), which the other entry points keep in a buffer that the caller
+// allocates and attaches.  Every GPU holds its own copy of the array at its own
+// address: the address is looked up once per device and only that pointer is
+// ever handed to a kernel (the array's name is a host-side stand-in).
+namespace et {
+constexpr int NOALLOC_MAX_SEQ = 4096; // 64 key tiles: what the kernels' two summary words per row group cover
+constexpr int NOALLOC_WORDS = (NOALLOC_MAX_SEQ / 16) * 2;
+static __device__ __align__(256) unsigned scratch[NOALLOC_WORDS]; // 2 KiB
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static unsigned *g_scratch_ptr[NOALLOC_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+static int noalloc_scratch(unsigned **ptr) {
+    int dev = -1;
+    ET_HIP(hipGetDevice(&dev));
+    ET_REQUIRE(dev >= 0 && dev < NOALLOC_MAX_DEVICES, ET_ERR_UNSUPPORTED,
+               "et_OTF_attention_noalloc: device index %d beyond %d", dev, NOALLOC_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        ET_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        ET_REQUIRE(p != nullptr, ET_ERR_HIP, "et_OTF_attention_noalloc: no address for the scratch array");
+        g_scratch_ptr[dev] = static_cast<unsigned *>(p);
+    }
+    *ptr = g_scratch_ptr[dev];
+    return ET_OK;
+}
+} // namespace et
+
+extern "C" int et_OTF_attention_noalloc(void *out, const void *Q, const void *K, const void *V,
+                                        const void *mask, int seq_len, int d_model, int nhead,
+                                        int batch, const int *seq_lens, float log2_scale,
+                                        void *stream) {
+    using namespace et;
+    AttnArgs a = {};
+    a.out = static_cast<f16 *>(out);
+    a.Q = static_cast<const f16 *>(Q);
+    a.K = static_cast<const f16 *>(K);
+    a.V = static_cast<const f16 *>(V);
+    a.mask = static_cast<const f16 *>(mask);
+    a.seq_lens = seq_lens;
+    a.ldq = a.ldv = d_model;
+    a.seq_len = seq_len;
+    a.nhead = nhead;
+    a.batch = batch;
+    a.log2_scale = log2_scale;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (!mask) // nothing to summarise: no scratch memory is touched
+        return attention_dispatch(a, d_model, false, false, st, "et_OTF_attention_noalloc");
+    ET_REQUIRE(seq_len > 0, ET_ERR_INVALID_ARG, "et_OTF_attention_noalloc: seq_len=%d", seq_len);
+    ET_REQUIRE(seq_len <= NOALLOC_MAX_SEQ, ET_ERR_UNSUPPORTED,
+               "et_OTF_attention_noalloc: seq_len %d beyond the %d that the static scratch array covers",
+               seq_len, NOALLOC_MAX_SEQ);
+    unsigned *summary = nullptr;
+    const int rc = noalloc_scratch(&summary);
+    if (rc != ET_OK)
+        return rc;
+    // every word that the attention kernel reads for this seq_len is written
+    // here first, so what an earlier call left in the array does not matter
+    hipLaunchKernelGGL(mask_summary_kernel, dim3((seq_len + 15) / 16), dim3(64), 0, st, a.mask, seq_len,
+                       summary, mask_summary_words(seq_len));
+    const int rs = launch_status("et_OTF_attention_noalloc summary launch");
+    if (rs != ET_OK)
+        return rs;
+    return attention_dispatch(a, d_model, false, false, st, "et_OTF_attention_noalloc", 0, summary);
 }
 
 extern "C" int et_OTF_attention_qk_width(void *out, const void *Q, const void *K, const void *V,

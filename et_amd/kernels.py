@@ -105,6 +105,22 @@ def OTF_attention(Q, K, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2_sc
     return Z
 
 
+def OTF_attention_noalloc(Q, K, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2_scale=1.0, out=None):
+    """OTF_attention through the entry point that allocates nothing: the mask summary is computed into a
+    static device array of the library (seq_len <= 4096 with a mask).  `out` is required: this wrapper
+    allocates nothing either."""
+    if out is None:
+        raise ValueError("OTF_attention_noalloc: pass the output tensor")
+    d_model = Q.shape[1]
+    for t, name in ((Q, "Q"), (K, "K"), (V, "V"), (out, "out")):
+        _want(t, "OTF_attention_noalloc " + name, batch * seq_len, d_model)
+    _want(mask, "OTF_attention_noalloc mask", seq_len * seq_len)
+    _want(seq_lens, "OTF_attention_noalloc seq_lens", batch)
+    check(lib().et_OTF_attention_noalloc(_h(out), _h(Q), _h(K), _h(V), _h(mask), seq_len, d_model, nhead, batch,
+                                         _i32(seq_lens), log2_scale, _stream()))
+    return out
+
+
 def OTF_attention_qk_width(Q, K, V, mask, qk_width, seq_len, nhead, batch=1, seq_lens=None, log2_scale=1.0, out=None):
     """Q, K compact [rows x nhead*qk_width] (the same number of kept columns in every head); V full width"""
     d_model = V.shape[1]

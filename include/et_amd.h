@@ -117,6 +117,27 @@ size_t et_attention_mask_summary_bytes(int seq_len);
 int et_attention_mask_summary(const void *mask, int seq_len, void *summary, void *stream);
 int et_attention_mask_summary_attach(const void *mask, int seq_len, const void *summary);
 
+/* et_OTF_attention for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * It has no counterpart in the reference.  Same arguments and the same result,
+ * bit for bit, as et_OTF_attention; what differs is where the mask summary
+ * lives: this call computes it from `mask` on `stream` into a 2 KiB array
+ * that is part of the library's device image (one copy per GPU, held until the
+ * process ends) and hands it to the attention kernel, so all-zero mask tiles
+ * are skipped without any buffer of the caller's and without the attach
+ * registry.  It calls no hipMalloc, hipFree or other allocating routine.
+ * Limit: with a mask, seq_len <= 4096 (ET_ERR_UNSUPPORTED beyond).  All calls
+ * on one GPU share that array: calls that overlap on one GPU (different
+ * streams or host threads) race; calls in stream order do not, and every word
+ * a call reads it has written itself, so nothing needs clearing in between.
+ * The array's address is looked up on the first call on a device: make that
+ * call outside a graph capture. */
+int et_OTF_attention_noalloc(void *out, const void *Q, const void *K,
+                             const void *V, const void *mask, int seq_len,
+                             int d_model, int nhead, int batch,
+                             const int *seq_lens, float log2_scale,
+                             void *stream);
+
 /* et_OTF_attention with Q and K holding qk_width < head_dim columns per head,
  * the same number in every head (attention-aware pruning that keeps the heads
  * balanced): Q, K are [batch*seq_len x nhead*qk_width], head h at columns
