@@ -35,11 +35,22 @@ def _dp(t):
     return t.data_ptr()
 
 
+def _chk2(t, rows, cols, what):
+    if t.dim() != 2 or t.shape[0] < rows or t.shape[1] != cols:
+        raise ValueError(f"{what}: expected at least {rows} rows of {cols} columns, got {tuple(t.shape)}")
+
+
 def _dp2(t, rows, cols, what):
     """device pointer of a [>= rows x cols] half tensor.  The C ABI takes bare pointers and cannot know a
     buffer's extent: an operand of the wrong shape is refused here, before a kernel reads or writes past it."""
-    if t.dim() != 2 or t.shape[0] < rows or t.shape[1] != cols:
-        raise ValueError(f"{what}: expected at least {rows} rows of {cols} columns, got {tuple(t.shape)}")
+    _chk2(t, rows, cols, what)
+    return _dp(t)
+
+
+def _dpn(t, n, what):
+    """device pointer of a half vector of exactly n elements (LayerNorm parameters)"""
+    if t.numel() != n:
+        raise ValueError(f"{what}: expected {n} elements, got {tuple(t.shape)}")
     return _dp(t)
 
 
@@ -70,7 +81,8 @@ class Linear_tile:
         check(lib().et_linear_tile_run_rows_ln(self._h, _dp2(out, rows, self.out_feat, "Linear_tile.run_ln out"),
                                                _dp2(x, rows, self.in_feat, "Linear_tile.run_ln x"),
                                                _dp2(skip, rows, self.out_feat, "Linear_tile.run_ln skip"),
-                                               _dp(gamma), _dp(beta), rows, _stream()))
+                                               _dpn(gamma, self.out_feat, "Linear_tile.run_ln gamma"),
+                                               _dpn(beta, self.out_feat, "Linear_tile.run_ln beta"), rows, _stream()))
         return out
 
     @staticmethod
@@ -85,7 +97,8 @@ class Linear_tile:
                                                    _dp2(x, rows, first.in_feat, what + " x"),
                                                    _dp2(hidden, rows, first.out_feat, what + " hidden") if hidden is not None else None,
                                                    _dp2(skip, rows, second.out_feat, what + " skip"),
-                                                   _dp(gamma), _dp(beta), rows, _stream()))
+                                                   _dpn(gamma, second.out_feat, what + " gamma"),
+                                                   _dpn(beta, second.out_feat, what + " beta"), rows, _stream()))
         return out
 
     @staticmethod
@@ -106,8 +119,10 @@ class Linear_tile:
                                                  _dp2(attn, rows, out_proj.in_feat, what + " attn"),
                                                  _dp2(inp, rows, out_proj.out_feat, what + " inp"),
                                                  opt(mid, out_proj.out_feat, " mid"), opt(hidden, first.out_feat, " hidden"),
-                                                 _dp(gamma1), _dp(beta1), _dp(gamma2),
-                                                 _dp(beta2), rows, _stream()))
+                                                 _dpn(gamma1, out_proj.out_feat, what + " gamma1"),
+                                                 _dpn(beta1, out_proj.out_feat, what + " beta1"),
+                                                 _dpn(gamma2, second.out_feat, what + " gamma2"),
+                                                 _dpn(beta2, second.out_feat, what + " beta2"), rows, _stream()))
         return out
 
     @staticmethod
@@ -126,10 +141,20 @@ class Linear_tile:
 def run_multi(linears, x, outs=None):
     """several Linear_tile over the same input in one launch"""
     n = len(linears)
-    outs = outs or [torch.empty((x.shape[0], l.out_feat), dtype=torch.float16, device=x.device) for l in linears]
+    if x.dim() != 2:
+        raise ValueError(f"run_multi x: expected a matrix, got {tuple(x.shape)}")
+    rows = x.shape[0]
+    outs = outs or [torch.empty((rows, l.out_feat), dtype=torch.float16, device=x.device) for l in linears]
+    if len(outs) != n:
+        raise ValueError(f"run_multi: {n} linears but {len(outs)} outputs")
+    _chk2(x, rows, linears[0].in_feat, "run_multi x")
+    for i, (o, l) in enumerate(zip(outs, linears)):
+        if l.in_feat != linears[0].in_feat:
+            raise ValueError("run_multi: the linears must share in_feat")
+        _chk2(o, rows, l.out_feat, f"run_multi outs[{i}]")
     hs = (C.c_void_p * n)(*[l._h for l in linears])
     ys = (C.c_void_p * n)(*[_dp(o) for o in outs])
-    check(lib().et_linear_tile_run_multi(hs, ys, n, _dp(x), x.shape[0], _stream()))
+    check(lib().et_linear_tile_run_multi(hs, ys, n, _dp(x), rows, _stream()))
     return outs
 
 
@@ -152,8 +177,9 @@ class Linear_row:
 
     def run(self, x, out=None):
         out = out if out is not None else torch.empty((x.shape[0], self.nrow), dtype=torch.float16, device=x.device)
-        check(lib().et_linear_row_run(self._h, _dp2(out, self.size, self.nrow, "Linear_row.run out"),
-                                      _dp2(x, self.size, self.in_feat, "Linear_row.run x"), _stream()))
+        _chk2(out, self.size, self.nrow, "Linear_row.run out")
+        _chk2(x, self.size, self.in_feat, "Linear_row.run x")
+        check(lib().et_linear_row_run(self._h, _dp(out), _dp(x), _stream()))
         return out
 
     def _release(self):
@@ -208,8 +234,13 @@ class _Encoder:
         if lens is None:
             check(lib().et_encoder_set_seq_lens(self._h, None))
         else:
+            lens = _np(lens, np.int64)
+            if lens.size != self.batch:
+                raise ValueError(f"set_seq_lens: expected {self.batch} lengths, got {lens.size}")
+            if lens.size and (lens.min() < 0 or lens.max() > self.seq_len):
+                raise ValueError(f"set_seq_lens: lengths must lie in [0, {self.seq_len}], got "
+                                 f"[{lens.min()}, {lens.max()}]")
             lens = _np(lens, np.int32)
-            assert lens.size == self.batch
             check(lib().et_encoder_set_seq_lens(self._h, _hp(lens)))
 
     def __del__(self):

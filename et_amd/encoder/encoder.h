@@ -78,6 +78,11 @@ class Encoder_base {
     void set_log2_scale(float v) { log2_scale = v; }
     // HOST array of `batch` lengths in [0, seq_len]; nullptr clears them.
     void set_seq_lens(const int *host_lens) {
+        // a length outside [0, seq_len] would push the packed row offsets past
+        // the workspace units: refuse before anything changes or reaches the device
+        for (int b = 0; host_lens && b < batch; b++)
+            etRequire(host_lens[b] >= 0 && host_lens[b] <= seq_len,
+                      "set_seq_lens: every length must lie in [0, seq_len]");
         lens.clear();
         total_rows = batch * seq_len;
         if (!host_lens)

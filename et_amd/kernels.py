@@ -62,6 +62,8 @@ def tile_spmm_add_bias(X, row_ptr, row_offset, data, bias, N, gelu=False, out=No
     _want(Y, "tile_spmm_add_bias out", M, N)
     _want(bias, "tile_spmm_add_bias bias", N)
     _want(data, "tile_spmm_add_bias data", (0 if row_offset is None else row_offset.numel()) * 256)
+    if N % 16 == 0:  # (other widths are the C ABI's to refuse)
+        _want(row_ptr, "tile_spmm_add_bias row_ptr", N // 16 + 1)
     fn = lib().et_tile_spmm_add_bias_gelu if gelu else lib().et_tile_spmm_add_bias
     check(fn(_h(Y), _h(X), _i32(row_ptr), _i32(row_offset), _h(data), M, N, K, _h(bias), _stream()))
     return Y
@@ -85,6 +87,12 @@ def row_spmm_add_bias_multi(X, weights, biases):
     import ctypes as C
     M, K = X.shape
     n = len(weights)
+    if len(biases) != n:
+        raise ValueError(f"row_spmm_add_bias_multi: {n} weights but {len(biases)} biases")
+    for i, (w, b) in enumerate(zip(weights, biases)):
+        if w.dim() != 2 or w.shape[1] != K:
+            raise ValueError(f"row_spmm_add_bias_multi weights[{i}]: expected [N x {K}], got {tuple(w.shape)}")
+        _want(b, f"row_spmm_add_bias_multi biases[{i}]", w.shape[0])
     outs = [torch.empty((M, w.shape[0]), dtype=torch.float16, device=X.device) for w in weights]
     arr = lambda ts: (C.c_void_p * n)(*[_h(t) for t in ts])
     ns = (C.c_int * n)(*[w.shape[0] for w in weights])
@@ -139,6 +147,7 @@ def OTF_attention_qk_width(Q, K, V, mask, qk_width, seq_len, nhead, batch=1, seq
 def OTF_attention_varlen(Q, K, V, mask, cu_seqlens, max_seq_len, nhead, log2_scale=1.0, out=None):
     d_model = Q.shape[1]
     batch = cu_seqlens.numel() - 1
+    _check_cu(cu_seqlens, max_seq_len, Q.shape[0], "OTF_attention_varlen")
     Z = out if out is not None else torch.empty_like(Q)
     for t, name in ((K, "K"), (V, "V"), (Z, "out")):
         _want(t, "OTF_attention_varlen " + name, *Q.shape)
@@ -169,6 +178,8 @@ def Prune_attention(Q, K, V, qk_head_ptr, v_col_id, v_head_ptr, mask, seq_len, d
 def qk_scores(Q, K, seq_len, nhead, batch=1):
     """scaled Q K^T per head into [(b*nhead+h), S, S]; encoder/encoder.cu:126-130"""
     d_model = Q.shape[1]
+    _want(Q, "qk_scores Q", batch * seq_len, d_model)
+    _want(K, "qk_scores K", batch * seq_len, d_model)
     QK = torch.empty((batch * nhead, seq_len, seq_len), dtype=torch.float16, device=Q.device)
     check(lib().et_qk_scores(_h(QK), _h(Q), _h(K), seq_len, d_model, nhead, batch, _stream()))
     return QK
@@ -188,10 +199,25 @@ def sharedQK_attention(QK, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2
     return Z
 
 
+def _check_cu(cu_seqlens, seq_len, total_rows, what):
+    """the packed row offsets must start at 0, rise by at most seq_len per sequence and end at the packed
+    tensor's row count: the kernels trust them for every address (one small device-to-host copy)"""
+    cu = cu_seqlens.detach().cpu().numpy().astype("int64")
+    if cu.size < 1 or cu[0] != 0 or cu[-1] != total_rows:
+        raise ValueError(f"{what}: cu_seqlens must run from 0 to the {total_rows} packed rows, got "
+                         f"{cu[0] if cu.size else None}..{cu[-1] if cu.size else None}")
+    step = cu[1:] - cu[:-1]
+    if step.size and (step.min() < 0 or step.max() > seq_len):
+        raise ValueError(f"{what}: every sequence must hold 0..{seq_len} rows")
+
+
 def pack_rows(padded, cu_seqlens, seq_len, total_rows, order=None):
     """order (int32 device tensor, optional): packed sequence i is padded sequence order[i]."""
     width = padded.shape[1]
     batch = cu_seqlens.numel() - 1
+    _want(padded, "pack_rows padded", batch * seq_len, width)
+    _want(order, "pack_rows order", batch)
+    _check_cu(cu_seqlens, seq_len, total_rows, "pack_rows")
     packed = torch.empty((total_rows, width), dtype=torch.float16, device=padded.device)
     check(lib().et_pack_rows_ordered(_h(packed), _h(padded), _i32(cu_seqlens), _i32(order), batch, seq_len,
                                      width, _stream()))
@@ -201,6 +227,8 @@ def pack_rows(padded, cu_seqlens, seq_len, total_rows, order=None):
 def unpack_rows(packed, cu_seqlens, seq_len, order=None):
     width = packed.shape[1]
     batch = cu_seqlens.numel() - 1
+    _want(order, "unpack_rows order", batch)
+    _check_cu(cu_seqlens, seq_len, packed.shape[0], "unpack_rows")
     padded = torch.empty((batch * seq_len, width), dtype=torch.float16, device=packed.device)
     check(lib().et_unpack_rows_ordered(_h(padded), _h(packed), _i32(cu_seqlens), _i32(order), batch, seq_len,
                                        width, _stream()))
@@ -209,6 +237,8 @@ def unpack_rows(packed, cu_seqlens, seq_len, order=None):
 
 def scatter_cols(x, col_id, width):
     rows, ld = x.shape
+    if col_id.numel() > ld or col_id.numel() > width:
+        raise ValueError(f"scatter_cols: {col_id.numel()} column ids for a [{rows} x {ld}] input and width {width}")
     out = torch.empty((rows, width), dtype=torch.float16, device=x.device)
     check(lib().et_scatter_cols(_h(out), _h(x), _i32(col_id), rows, col_id.numel(), ld, width, _stream()))
     return out
@@ -223,6 +253,8 @@ def scatter_skip_layernorm(compact, col_id, skip, gamma, beta, out=None):
     _want(out, "scatter_skip_layernorm out", rows, width)
     _want(gamma, "scatter_skip_layernorm gamma", width)
     _want(beta, "scatter_skip_layernorm beta", width)
+    if col_id.numel() > ld or col_id.numel() > width:
+        raise ValueError(f"scatter_skip_layernorm: {col_id.numel()} column ids for a [{rows} x {ld}] input and width {width}")
     check(lib().et_scatter_skip_layernorm(_h(out), _h(compact), _i32(col_id), col_id.numel(), ld, _h(skip),
                                           _h(gamma), _h(beta), rows, width, _stream()))
     return out
@@ -238,4 +270,39 @@ def attention_mask_summary(mask, seq_len):
 
 
 def attention_mask_summary_attach(mask, seq_len, summary):
+    """Raw form of the registry call (entries are keyed on the mask's device address): prefer MaskSummary,
+    which ties the entry to the tensors' lifetime."""
     check(lib().et_attention_mask_summary_attach(_h(mask), seq_len, None if summary is None else _p(summary)))
+
+
+class MaskSummary:
+    """Owns the summary of an additive mask tensor and its registration with the attention launchers.
+
+    The registry is keyed on the mask's device address, so an entry must not outlive the mask it was
+    computed from: this object keeps the mask tensor alive while it is attached (its address cannot be
+    handed to another tensor meanwhile) and detaches when it is closed or collected.  After writing
+    into the mask in place, call refresh(): a stale summary would skip tiles that are no longer zero."""
+
+    def __init__(self, mask, seq_len):
+        _want(mask, "MaskSummary mask", seq_len * seq_len)
+        self.mask, self.seq_len = mask, seq_len
+        self.summary = None
+        self.refresh()
+
+    def refresh(self):
+        self.summary = attention_mask_summary(self.mask, self.seq_len)
+        attention_mask_summary_attach(self.mask, self.seq_len, self.summary)
+
+    def close(self):
+        if getattr(self, "summary", None) is not None:
+            attention_mask_summary_attach(self.mask, self.seq_len, None)
+            self.summary = None
+            self.mask = None
+
+    __del__ = close
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()

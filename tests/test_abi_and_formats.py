@@ -195,3 +195,57 @@ def test_kernel_wrappers_refuse_operands_of_the_wrong_extent():
         kernels.OTF_attention(h(32, 64), h(16, 64), h(32, 64), None, 32, 1)
     with pytest.raises(ValueError):     # mask of another sequence length
         kernels.OTF_attention(h(32, 64), h(32, 64), h(32, 64), h(16, 16), 32, 1)
+
+
+def test_more_wrappers_refuse_operands_of_the_wrong_extent():
+    """run_multi, the packed-row copies, the multi row linear and the raw tile launcher on host tensors: the
+    ValueError comes before any device pointer is asked for"""
+    import torch
+    from et_amd import encoder, kernels
+    h = lambda *shape: torch.zeros(shape, dtype=torch.float16)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32)
+
+    class Stub:                         # stands in for a Linear_tile / Linear_row handle: never reached
+        _h = None
+        in_feat, out_feat, size, nrow = 32, 48, 8, 48
+
+    with pytest.raises(ValueError):     # x of another width than in_feat
+        encoder.run_multi([Stub(), Stub()], h(8, 64), [h(8, 48), h(8, 48)])
+    with pytest.raises(ValueError):     # second output too narrow
+        encoder.run_multi([Stub(), Stub()], h(8, 32), [h(8, 48), h(8, 16)])
+    with pytest.raises(ValueError):     # fewer output rows than x has
+        encoder.run_multi([Stub()], h(8, 32), [h(4, 48)])
+    # the swap that once wrote 48-wide rows into a 32-wide tensor: Linear_row.run(x, out) with the two exchanged
+    lr = encoder.Linear_row.__new__(encoder.Linear_row)
+    lr.__dict__.update(_h=None, in_feat=32, out_feat=64, size=8, nrow=48)
+    with pytest.raises(ValueError):
+        encoder.Linear_row.run(lr, h(8, 48), out=h(8, 32))
+    with pytest.raises(ValueError):     # gamma of the wrong length
+        encoder._dpn(h(16), 48, "gamma")
+    with pytest.raises(ValueError):     # cu_seqlens ends beyond the packed rows
+        kernels.pack_rows(h(2 * 16, 8), i32([0, 10, 30]), 16, 26)
+    with pytest.raises(ValueError):     # a sequence longer than seq_len
+        kernels.pack_rows(h(2 * 16, 8), i32([0, 20, 26]), 16, 26)
+    with pytest.raises(ValueError):     # order of the wrong length
+        kernels.pack_rows(h(2 * 16, 8), i32([0, 10, 26]), 16, 26, order=i32([0, 1, 2]))
+    with pytest.raises(ValueError):     # packed tensor shorter than cu_seqlens says
+        kernels.unpack_rows(h(20, 8), i32([0, 10, 26]), 16)
+    with pytest.raises(ValueError):     # bias shorter than the weight's rows
+        kernels.row_spmm_add_bias_multi(h(8, 32), [h(16, 32), h(16, 32)], [h(16), h(8)])
+    with pytest.raises(ValueError):     # weight with another K
+        kernels.row_spmm_add_bias_multi(h(8, 32), [h(16, 64)], [h(16)])
+    with pytest.raises(ValueError):     # row_ptr must hold N/16 + 1 entries
+        kernels.tile_spmm_add_bias(h(8, 32), i32([0, 1]), i32([0]), h(256), h(32), 32)
+
+
+def test_seq_lens_outside_the_sequence_are_refused():
+    """a length above seq_len or below 0 would push the packed row offsets past the workspace: the Python
+    class refuses it before the call (the C++ class's own check needs an encoder object, hence a device:
+    tests/test_gpu_encoder.py covers its error code)"""
+    import numpy as np
+    from et_amd import encoder
+    enc = encoder.Encoder_length.__new__(encoder.Encoder_length)
+    enc.__dict__.update(_h=None, batch=3, seq_len=64)
+    for bad in ([64, 65, 1], [3, -1, 2], [1, 2]):
+        with pytest.raises(ValueError):
+            encoder._Encoder.set_seq_lens(enc, np.array(bad))

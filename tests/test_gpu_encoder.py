@@ -309,6 +309,16 @@ def test_encoder_length_paths():
         assert (got_l[b * S + lens[b]:(b + 1) * S] == 0).all()
     got_alias = host(enc.run(xd, xd))
     assert np.array_equal(got_alias, got_l)
+    # lengths outside [0, seq_len] are refused by the C++ class before anything is uploaded (the Python
+    # class has its own check in front, so the C entry point is called directly)
+    import ctypes as C
+    from et_amd import lib
+    for bad in ([256, 257, 1], [5, -1, 3]):
+        arr = (C.c_int * B)(*bad)
+        assert lib().et_encoder_set_seq_lens(enc._h, C.cast(arr, C.c_void_p)) < 0
+        assert b"seq_len" in lib().et_last_error()
+    got_after = host(enc.run(torch.empty_like(xd), dev(x)))     # the refused calls changed nothing
+    assert np.array_equal(got_after, got_l)
 
 
 def test_encoder_stack_variable_length():

@@ -475,6 +475,22 @@ def test_tile_linear_full_size_config2_rows_sample(K, sp, ntile):
     normal = np.abs(got) >= 2.0 ** -13
     assert np.array_equal(got2[normal], (got * np.float16(2))[normal])
     assert np.abs(got2.astype(np.float64) - 2 * got.astype(np.float64))[~normal].max() <= 2.0 ** -23
+    # the planned form of the same linear (Linear_tile::run: the 64-row resident kernel that the encoders
+    # and the benchmark run at this size), its index arrays from the product's own generator and packer
+    from et_amd import formats
+    from et_amd.encoder import Linear_tile
+    rp, ro = formats.gen_sparse_tile_mat(N, Kd, sp, 2024)
+    assert np.array_equal(rp, lin["row_ptr"]) and np.array_equal(ro, lin["row_offset"])
+    data = formats.tile_pack(lin["W"], rp, ro)
+    assert np.array_equal(data, lin["data"])
+    bias = randn_h(r, (N,), 0.1)
+    want_b = orc.tile_linear(X[rows], rp, ro, data, bias, N, f64=True)
+    planned = host(Linear_tile(Kd, N, M, ro.size, data, rp, ro, bias).run(dev(X)))
+    check_close(planned[rows], want_b, max_abs=2e-3, mean_rel=5e-4, what="config-2 sample, planned")
+    if sp in (0.8, 0.0):
+        want_g = orc.tile_linear(X[rows], rp, ro, data, bias, N, gelu=True, f64=True)
+        planned_g = host(Linear_tile(Kd, N, M, ro.size, data, rp, ro, bias, True).run(dev(X)))
+        check_close(planned_g[rows], want_g, max_abs=2e-3, mean_rel=5e-4, what="config-2 sample, planned + GELU")
 
 
 def test_tile_linear_argument_errors(K):
@@ -584,6 +600,42 @@ def test_attention_mask_summary(K, S):
         assert np.array_equal(plain, fast)
         want = orc.otf_attention(Q, Kk, V, m, S, H, B, None, 1.0, f64=True)
         check_close(fast, want, max_abs=5e-3, mean_rel=1e-3, what="attention with mask summary")
+
+
+def test_mask_summary_object_does_not_outlive_its_mask(K):
+    """the summary registry is keyed on the mask's address: a MaskSummary holds its mask while attached
+    and detaches when it goes, so another mask that the allocator puts at the same address is not
+    treated with the old summary"""
+    r = rng(46)
+    S, H, d = 256, 4, 256
+    Q, Kk, V = (randn_h(r, (S, d)) for _ in range(3))
+    zeros = torch.zeros((S, S), dtype=torch.float16, device="cuda")
+    addr = zeros.data_ptr()
+    ms = K.MaskSummary(zeros, S)           # all-zero: the launchers take the no-mask kernel for this address
+    no_mask = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), zeros, S, H))
+    del zeros                              # the object still holds the tensor: the address stays taken
+    other = torch.empty((S, S), dtype=torch.float16, device="cuda")
+    assert other.data_ptr() != addr
+    del ms, other                          # detaches, then frees
+    mask = randn_h(r, (S, S), 2.0)
+    md = torch.empty((S, S), dtype=torch.float16, device="cuda")
+    md.copy_(torch.from_numpy(mask))
+    if md.data_ptr() != addr:
+        pytest.skip("the allocator did not hand the address out again")
+    got = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), md, S, H))
+    want = orc.otf_attention(Q, Kk, V, mask, S, H, 1, None, 1.0, f64=True)
+    check_close(got, want, max_abs=5e-3, mean_rel=1e-3, what="attention with a mask at a reused address")
+    assert not np.array_equal(got, no_mask)
+    # in-place update of an attached mask: refresh() brings the summary up to date
+    with K.MaskSummary(md, S) as ms2:
+        md.zero_()
+        md[5, 200] = -4.0
+        ms2.refresh()
+        got2 = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), md, S, H))
+    m2 = np.zeros((S, S), np.float16)
+    m2[5, 200] = -4.0
+    check_close(got2, orc.otf_attention(Q, Kk, V, m2, S, H, 1, None, 1.0, f64=True), max_abs=5e-3, mean_rel=1e-3,
+                what="attention after an in-place mask update")
 
 
 @pytest.mark.parametrize("S,H,d,B,lens", [(2048, 12, 768, 1, [1500]), (4160, 2, 128, 2, [4160, 4097])])
