@@ -50,10 +50,10 @@ PROTOTYPES = {
     "et_prune_row_mat": (_i, [_vp, _i, _i, _f, _ip]),
     "et_tile_mat_save": (_i, [C.c_char_p, _i, _i, _i, _ip, _ip, _vp, _vp]),
     "et_tile_mat_peek": (_i, [C.c_char_p, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
-    "et_tile_mat_load": (_i, [C.c_char_p, _ip, _ip, _vp, _vp]),
+    "et_tile_mat_load": (_i, [C.c_char_p, _i, _i, _i, _ip, _ip, _vp, _vp]),
     "et_row_mat_save": (_i, [C.c_char_p, _i, _i, _i, _ip, _vp, _vp]),
     "et_row_mat_peek": (_i, [C.c_char_p, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
-    "et_row_mat_load": (_i, [C.c_char_p, _ip, _vp, _vp]),
+    "et_row_mat_load": (_i, [C.c_char_p, _i, _i, _i, _ip, _vp, _vp]),
     "et_gen_sparse_tile_mat": (_i, [_i, _i, _f, _u64, _ip, _ip]),
     "et_gen_sparse_row_mat": (_i, [_i, _f, _u64, _ip]),
     "et_gen_head_balanced_rows": (_i, [_i, _i, _i, _u64, _ip]),

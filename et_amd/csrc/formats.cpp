@@ -335,6 +335,11 @@ int read_header(FILE *f, const char *magic, ContainerHeader *h, const char *path
         et::set_error("%s: %s is not a version-1 container of this kind", who, path);
         return ET_ERR_FORMAT;
     }
+    for (char c : h->reserved) // written as zero; anything else is damage (the checksum covers the payload only)
+        if (c != 0) {
+            et::set_error("%s: %s has a damaged header", who, path);
+            return ET_ERR_FORMAT;
+        }
     return ET_OK;
 }
 
@@ -379,7 +384,11 @@ int load_container(const char *path, const char *magic, PartsFn parts_of, const 
         uint64_t total = 0, sum = 0xcbf29ce484222325ull;
         for (const Part &p : parts)
             total += p.bytes;
-        if (total != h.payload_bytes) {
+        if (parts.empty()) {
+            et::set_error("%s: %s holds in_feat=%d out_feat=%d count=%d, not what the caller sized its arrays for", who,
+                          path, h.in_feat, h.out_feat, h.count);
+            rc = ET_ERR_FORMAT;
+        } else if (total != h.payload_bytes) {
             et::set_error("%s: %s: payload size does not match its header", who, path);
             rc = ET_ERR_FORMAT;
         }
@@ -426,7 +435,8 @@ extern "C" int et_tile_mat_peek(const char *path, int *in_feat, int *out_feat, i
     return peek_container(path, TILE_MAGIC, in_feat, out_feat, ntile, "et_tile_mat_peek");
 }
 
-extern "C" int et_tile_mat_load(const char *path, int *row_ptr, int *row_offset, void *data, void *bias) {
+extern "C" int et_tile_mat_load(const char *path, int expect_in_feat, int expect_out_feat, int expect_ntile,
+                                int *row_ptr, int *row_offset, void *data, void *bias) {
     if (!row_ptr || !row_offset || !data || !bias) {
         et::set_error("et_tile_mat_load: null pointer");
         return ET_ERR_INVALID_ARG;
@@ -436,6 +446,10 @@ extern "C" int et_tile_mat_load(const char *path, int *row_ptr, int *row_offset,
         path, TILE_MAGIC,
         [&](const ContainerHeader &h) {
             in_feat = h.in_feat, out_feat = h.out_feat, ntile = h.count;
+            // the caller sized its arrays from an earlier peek: a file that has changed since, or
+            // arrays meant for another file, must not be written past
+            if (h.in_feat != expect_in_feat || h.out_feat != expect_out_feat || h.count != expect_ntile)
+                return std::vector<Part>{};
             return std::vector<Part>{{nullptr, row_ptr, sizeof(int) * (size_t)(h.out_feat / 16 + 1)},
                                      {nullptr, row_offset, sizeof(int) * (size_t)h.count},
                                      {nullptr, data, 512 * (size_t)h.count},
@@ -475,7 +489,8 @@ extern "C" int et_row_mat_peek(const char *path, int *in_feat, int *out_feat, in
     return peek_container(path, ROW_MAGIC, in_feat, out_feat, nrow, "et_row_mat_peek");
 }
 
-extern "C" int et_row_mat_load(const char *path, int *row_id, void *weight, void *bias) {
+extern "C" int et_row_mat_load(const char *path, int expect_in_feat, int expect_out_feat, int expect_nrow,
+                               int *row_id, void *weight, void *bias) {
     if (!row_id || !weight || !bias) {
         et::set_error("et_row_mat_load: null pointer");
         return ET_ERR_INVALID_ARG;
@@ -485,6 +500,8 @@ extern "C" int et_row_mat_load(const char *path, int *row_id, void *weight, void
         path, ROW_MAGIC,
         [&](const ContainerHeader &h) {
             out_feat = h.out_feat, nrow = h.count;
+            if (h.in_feat != expect_in_feat || h.out_feat != expect_out_feat || h.count != expect_nrow)
+                return std::vector<Part>{};
             return std::vector<Part>{{nullptr, row_id, sizeof(int) * (size_t)h.count},
                                      {nullptr, weight, 2 * (size_t)h.count * h.in_feat},
                                      {nullptr, bias, 2 * (size_t)h.out_feat}};

@@ -103,7 +103,7 @@ const char *et_strerror(int code) {
 }
 
 const char *et_last_error(void) { return et::g_err; }
-int et_abi_version(void) { return 1; }
+int et_abi_version(void) { return 2; } // 2: the container loaders take the expected sizes
 
 int et_malloc(void **ptr, size_t bytes) {
     ET_REQUIRE(ptr, ET_ERR_INVALID_ARG, "et_malloc: null out pointer");

@@ -286,25 +286,6 @@ __device__ __forceinline__ void tl_preload(const f16 *data, const int *poff, uns
         tl_load_pair(data, poff, min(q0 + i, qlast), lane_w, hi, w[i], o[i]);
 }
 
-#ifdef TL_STAGETRACE
-// profiling builds only: lane 0 of a traced wave stamps (cycle counter << 8 |
-// code) into an LDS buffer at every stage
-struct TlTracer {
-    unsigned long long *buf;
-    int n, cap;
-};
-__device__ unsigned long long *g_stage_trace = nullptr;
-__device__ __forceinline__ void tl_stamp(TlTracer &t, unsigned lane_w, unsigned code) {
-    if (t.buf && t.n < t.cap) {
-        if (lane_w == 0)
-            t.buf[t.n] = ((unsigned long long)__builtin_readcyclecounter() << 8) | code;
-        t.n++;
-    }
-}
-#define TL_STAMP(code_) tl_stamp(*trc_, lane_w, code_)
-#else
-#define TL_STAMP(code_)
-#endif
 
 // bvec: lane j holds the first pair of block-row j, lane NB the end of the
 // last one (read back with v_readlane)
@@ -313,18 +294,9 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
                                           const int *poff, unsigned lane_w, unsigned hi, int q0,
                                           int qend, int qlast, int bvec, f16x8 (&w)[TL_DEPTH],
                                           int (&o)[TL_DEPTH], Flush &&flush
-#ifdef TL_STAGETRACE
-                                          , TlTracer *trc_ = nullptr
-#endif
 ) {
-#ifdef TL_STAGETRACE
-    TlTracer dummy_{nullptr, 0, 0};
-    if (!trc_)
-        trc_ = &dummy_;
-#endif
     if (q0 >= qend)
         return;
-    TL_STAMP(3);
     __builtin_amdgcn_s_setprio(TL_PRIO);
     f32x4 cur0 = f32x4{0.f, 0.f, 0.f, 0.f}, cur1 = f32x4{0.f, 0.f, 0.f, 0.f};
     int j = 0;
@@ -352,7 +324,6 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
         // keep the reads above the MFMAs: left alone, the scheduler sinks them
         // to the end of the stage and every stage then waits out the LDS latency
         __builtin_amdgcn_sched_barrier(0);
-        TL_STAMP(1);
         cur0 = mfma16x16x32(w[S], xa[P], cur0);
         cur1 = mfma16x16x32(w[S], xb[P], cur1);
         // pair q + I + TL_DEPTH; the last stages of a stream request nothing:
@@ -361,7 +332,6 @@ __device__ __forceinline__ void tl_stream(const char *xlane, int xrow16, const f
         if (decltype(always)::value || q + I + TL_DEPTH < qend)
             tl_load_pair_at(wp + I * 1024, op + I * 8, lane_lo, lane_lw, w[S], o[S]);
         if (q + I + 1 == bend) { // block-row j is complete
-            TL_STAMP(2);
             __builtin_amdgcn_s_setprio(0);
             flush(j, cur0, cur1);
             __builtin_amdgcn_s_setprio(TL_PRIO);
@@ -396,18 +366,9 @@ __device__ __forceinline__ void tl_stream64(const char *xlane, int xrow16, const
                                           const int *poff, unsigned lane_w, unsigned hi, int q0,
                                           int qend, int qlast, int bvec, f16x8 (&w)[TL_DEPTH],
                                           int (&o)[TL_DEPTH], Flush &&flush
-#ifdef TL_STAGETRACE
-                                          , TlTracer *trc_ = nullptr
-#endif
 ) {
-#ifdef TL_STAGETRACE
-    TlTracer dummy_{nullptr, 0, 0};
-    if (!trc_)
-        trc_ = &dummy_;
-#endif
     if (q0 >= qend)
         return;
-    TL_STAMP(3);
     f32x4 cur0 = f32x4{0.f, 0.f, 0.f, 0.f}, cur1 = cur0, cur2 = cur0, cur3 = cur0;
     int j = 0;
     int bend = __builtin_amdgcn_readlane(bvec, 1);
@@ -438,7 +399,6 @@ __device__ __forceinline__ void tl_stream64(const char *xlane, int xrow16, const
         // keep the reads above the MFMAs: left alone, the scheduler sinks them
         // to the end of the stage and every stage then waits out the LDS latency
         __builtin_amdgcn_sched_barrier(0);
-        TL_STAMP(1);
         cur0 = mfma16x16x32(w[S], xa[P], cur0);
         cur1 = mfma16x16x32(w[S], xb[P], cur1);
         cur2 = mfma16x16x32(w[S], xc[P], cur2);
@@ -449,7 +409,6 @@ __device__ __forceinline__ void tl_stream64(const char *xlane, int xrow16, const
         if (decltype(always)::value || q + I + TL_DEPTH < qend)
             tl_load_pair_at(wp + I * 1024, op + I * 8, lane_lo, lane_lw, w[S], o[S]);
         if (q + I + 1 == bend) { // block-row j is complete
-            TL_STAMP(2);
             flush(j, cur0, cur1, cur2, cur3);
             cur0 = cur1 = cur2 = cur3 = f32x4{0.f, 0.f, 0.f, 0.f};
             j++;
@@ -627,10 +586,6 @@ __device__ __forceinline__ void tl_ln_rows_at(const TlLnOperands<NB, NW, NLW> &o
 // boundary (a scalar compare per pair) it is added into that block-row's
 // static accumulator.
 // ---------------------------------------------------------------------------
-#ifdef TL_TRACE
-__device__ unsigned long long *g_trace = nullptr; // per wave: start, panel, compute, epilogue ticks, HW ids
-#define TL_TICK() __builtin_readcyclecounter()
-#endif
 
 template <int NB, bool GELU, int NW, bool LN>
 __global__ void __launch_bounds__(NW * 64) tile_linear_plan_kernel(const TlArgs a) {
@@ -658,10 +613,6 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_plan_kernel(const TlArgs 
     f16 *const stage0 = xs + TL_BM * x.ldx;
     f16 *const stage = stage0 + x.wave * tl_wave_stage_halves<NB>();
     const int per_rp = a.ncg * a.nlin;
-#ifdef TL_TRACE
-    const unsigned long long tt0 = TL_TICK();
-    unsigned long long tpanel = 0, tcomp = 0, tepi = 0, tlast = tt0, tgap = 0;
-#endif
 
     // X panel staging: global -> LDS directly (global_load_lds_dwordx4: lane L
     // of the issuing wave writes 16 bytes at  base + 16*L, the source address is
@@ -718,10 +669,6 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_plan_kernel(const TlArgs 
         const unsigned lane_w = hi * 256 + x.c16 * 16 + x.khalf8; // lane's halves inside a 1 KB tile pair
 
         for (int c = 0; c < a.nchunk; c++) {
-#ifdef TL_TRACE
-            const unsigned long long ta = TL_TICK();
-            tgap += ta - tlast;
-#endif
             // pair-index boundaries of the wave's block-rows: lane j holds the end
             // of block-row j (read back with v_readlane)
             const int bidx = c * nbr + min(x.bn0 + min(lane, NB), nbr);
@@ -747,21 +694,10 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_plan_kernel(const TlArgs 
             f16x8 w[TL_DEPTH];
             int o[TL_DEPTH];
             tl_preload(data, poff, lane_w, hi, q0, qlast, w, o);
-#ifdef TL_TRACE
-            const unsigned long long tb = TL_TICK();
-            tpanel += tb - ta;
-#endif
             tl_stream<NB>(xlane, xrow16, data, poff, lane_w, hi, q0, qend, qlast, bvec, w, o,
                           [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); });
-#ifdef TL_TRACE
-            tlast = TL_TICK();
-            tcomp += tlast - tb;
-#endif
         }
         panel_rp = a.nchunk > 1 ? -1 : rp;
-#ifdef TL_TRACE
-        const unsigned long long te = TL_TICK();
-#endif
         tl_epilogue_wave<NB, GELU, !LN>(a, x, stage, Yp, N, nbr, acc, b4);
         if constexpr (LN) {
             TlLnOperands<NB, NW, NW> lnop;
@@ -770,21 +706,8 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_plan_kernel(const TlArgs 
             tl_ln_rows(lnop, a, stage0, x.wave, lane, x.m0, Yp, N);
             lds_used = true; // (the next item's panel load starts with a barrier)
         }
-#ifdef TL_TRACE
-        tlast = TL_TICK();
-        tepi += tlast - te;
-#endif
     }
 #undef TL_PANEL_LOAD
-#ifdef TL_TRACE
-    if (g_trace && lane == 0) {
-        unsigned hwid, xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        unsigned long long *t = g_trace + ((size_t)blockIdx.x * NW + x.wave) * 8;
-        t[0] = tt0; t[1] = tpanel; t[2] = tcomp; t[3] = tepi; t[4] = TL_TICK(); t[5] = hwid; t[6] = xcc; t[7] = tgap;
-    }
-#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -932,10 +855,6 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
         const bool lw = cw && t.lin + 1 == a.nlin;
         return tl_item(t.rp + (lw ? 1 : 0), lw ? 0 : t.lin + (cw ? 1 : 0), cw ? 0 : t.cg + 1);
     };
-#ifdef TL_TRACE
-    const unsigned long long tt0 = TL_TICK();
-    unsigned long long tpanel = 0, tcomp = 0, tepi = 0, tgap = 0, tlast = tt0;
-#endif
     const int per_rp = a.ncg * a.nlin;
     const int rp0 = it0 / per_rp, rest0 = it0 - rp0 * per_rp;
     TlItem cur = tl_item(rp0, rest0 / a.ncg, rest0 % a.ncg);
@@ -950,10 +869,6 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
     f16x8 w[TL_DEPTH];
     int o[TL_DEPTH];
     TL_PRELOAD(cur, bvec)
-#ifdef TL_TRACE
-    tlast = TL_TICK();
-    tpanel = tlast - tt0;
-#endif
 
     for (int it = it0;; it++) {
         const bool has_next = it + 1 < it1;
@@ -962,10 +877,6 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
         f16x4 b4n[NB];
         TL_BIAS(b4n, nxt)
 
-#ifdef TL_TRACE
-        const unsigned long long ta = TL_TICK();
-        tgap += ta - tlast;
-#endif
         // a finished block-row goes straight to the wave's staging tile
         // bias of block-row j as a 0/1-masked sum (exact); a chain of selects
         // over b4[] would be turned into an indexed load and put the array into
@@ -990,10 +901,6 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
                                 tl_stage_tile<GELU>(stage_lane + 32 * lds + j * 16, lds, c2, c3, bj);
                             });
         }
-#ifdef TL_TRACE
-        const unsigned long long tb = TL_TICK();
-        tcomp += tb - ta;
-#endif
         // block-rows without any tile: bias only
 #pragma unroll
         for (int k = 0; k < NB; k++)
@@ -1032,10 +939,6 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
                 }
             }
         }
-#ifdef TL_TRACE
-        tlast = TL_TICK();
-        tepi += tlast - tb;
-#endif
         if (!has_next)
             break;
         if (!same_panel) {
@@ -1052,15 +955,6 @@ __global__ void __launch_bounds__(NW * 64) tile_linear_resident_kernel(const TlA
 #undef TL_PRELOAD
 #undef TL_PANEL
 #undef TL_BIAS
-#ifdef TL_TRACE
-    if (g_trace && lane == 0) {
-        unsigned hwid, xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        unsigned long long *t = g_trace + ((size_t)blockIdx.x * NW + wave) * 8;
-        t[0] = tt0; t[1] = tpanel; t[2] = tcomp; t[3] = tepi; t[4] = TL_TICK(); t[5] = hwid; t[6] = xcc; t[7] = tgap;
-    }
-#endif
 #undef TL_BVEC
 #undef TL_KARG
 }
@@ -1109,10 +1003,6 @@ __global__ void __launch_bounds__(TL_CTHREADS) tile_linear_chunked_ln_kernel(con
     f16 *const Yp = a.Y[0];
     const int N = a.N[0];
     const int nbr = N >> 4;
-#ifdef TL_TRACE
-    const unsigned long long tt0 = TL_TICK();
-    unsigned long long tpanel = 0, tcomp = 0, tepi = 0, tgap = 0, tlast = tt0;
-#endif
 
     if (x.wave == TL_CWAVES) {
         // ---- the fetching wave ----
@@ -1136,17 +1026,8 @@ __global__ void __launch_bounds__(TL_CTHREADS) tile_linear_chunked_ln_kernel(con
             TL_FETCH(1)
         tl_barrier_lds(); // chunk 0 is in LDS
         for (int c = 1; c < a.nchunk; c++) {
-#ifdef TL_TRACE
-            tlast = TL_TICK();
-#endif
             __builtin_amdgcn_s_waitcnt(0x0F70); // chunk c has landed
-#ifdef TL_TRACE
-            { const unsigned long long t = TL_TICK(); tpanel += t - tlast; tlast = t; }
-#endif
             tl_barrier_lds();                   // ... and every wave has left chunk c-1
-#ifdef TL_TRACE
-            tgap += TL_TICK() - tlast;
-#endif
             if (c + 1 < a.nchunk)
                 TL_FETCH(c + 1)
         }
@@ -1185,42 +1066,19 @@ __global__ void __launch_bounds__(TL_CTHREADS) tile_linear_chunked_ln_kernel(con
             const int cn = min(c + 1, a.nchunk - 1);
             const int bvec_n = cptr[cn * nbr + min(x.bn0 + min(lane, NB), nbr)] >> 1;
             const int bcur = bvec;
-#ifdef TL_TRACE
-            tlast = TL_TICK();
-#endif
             tl_barrier_lds();
-#ifdef TL_TRACE
-            const unsigned long long tb = TL_TICK();
-            tgap += tb - tlast;
-#endif
 
             tl_stream<NB>(xlane, xrow16, data, poff, lane_w, hi, q0, qend, qlast, bcur, w, o,
                           [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); });
-#ifdef TL_TRACE
-            tcomp += TL_TICK() - tb;
-#endif
             bvec = bvec_n;
         }
         f16 *stage = stage0 + x.wave * tl_wave_stage_halves<NB>();
         tl_epilogue_wave<NB, false, false>(a, x, stage, Yp, N, nbr, acc, b4);
     }
-#ifdef TL_TRACE
-    tlast = TL_TICK();
-#endif
     TlLnOperands<NB, TL_CWAVES, TL_CWAVES + 1> lnop;
     tl_ln_fetch(lnop, a, x.wave, lane, x.m0, N);
     __syncthreads(); // every computing wave's part of the rows is staged
     tl_ln_rows(lnop, a, stage0, x.wave, lane, x.m0, Yp, N);
-#ifdef TL_TRACE
-    tepi = TL_TICK() - tlast;
-    if (g_trace && lane == 0) {
-        unsigned hwid, xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        unsigned long long *t = g_trace + ((size_t)blockIdx.x * 16 + x.wave) * 8;
-        t[0] = tt0; t[1] = tpanel; t[2] = tcomp; t[3] = tepi; t[4] = TL_TICK(); t[5] = hwid; t[6] = xcc; t[7] = tgap;
-    }
-#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -1259,10 +1117,17 @@ __device__ __forceinline__ void tl_signal(unsigned *ctr, int lane) {
     if (lane == 0)
         __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
+// The wait is bounded (about 4 million polls, tens of milliseconds): should a
+// wave ever fail to signal, the kernel ends with a wrong result instead of
+// hanging the GPU.  Every launch site checks on the host that the phase count
+// fits the counters (tile_launch_ffn).
 __device__ __forceinline__ void tl_wait_count(unsigned *ctr, unsigned target) {
-    while ((unsigned)__builtin_amdgcn_readfirstlane(
-               (int)__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) < target)
+    for (int spin = 0; spin < (1 << 22); spin++) {
+        if ((unsigned)__builtin_amdgcn_readfirstlane(
+                (int)__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) >= target)
+            break;
         __builtin_amdgcn_s_sleep(1);
+    }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
@@ -1297,15 +1162,6 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
     // event counters behind the hidden buffers: [p] first linear of phase p
     // done, [TL_FFN_MAX_PHASES + p] second linear of phase p done
     unsigned *const ctr = reinterpret_cast<unsigned *>(hs + 2 * hbuf);
-#ifdef TL_STAGETRACE
-    TlTracer trc{nullptr, 0, 192};
-    if (rp == 0 && x.wave < 8)
-        trc.buf = reinterpret_cast<unsigned long long *>(ctr + 2 * TL_FFN_MAX_PHASES) + x.wave * 192;
-    TlTracer *const trc_ = &trc;
-#define TL_TRC_ARG , &trc
-#else
-#define TL_TRC_ARG
-#endif
     const int N1 = a.N[L1], N2 = a.N[L2], nbr1 = N1 >> 4, nbr2 = N2 >> 4;
     const int hbr = a.KC >> 4; // hidden block-rows per phase
     const unsigned lane_w = hi * 256 + c16 * 16 + x.khalf8;
@@ -1372,7 +1228,7 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
                           _Pragma("unroll") for (int k = 0; k < NB; k++)                          \
                               bj += b1_[k] * ((j == k) ? (f16)1 : (f16)0);                        \
                           tl_stage_tile<true>(hlane + j * 16, ldh, c0, c1, bj);                   \
-                      } TL_TRC_ARG);                                                              \
+                      });                                                              \
         /* block-rows of this phase without any tile: bias only */                                \
         const int lim1 = min(((p_) + 1) * hbr, nbr1);                                             \
         _Pragma("unroll") for (int k = 0; k < NB; k++)                                            \
@@ -1427,7 +1283,7 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
             const int q0_ = __builtin_amdgcn_readfirstlane(bvecO), qe_ = __builtin_amdgcn_readlane(bvecO, NB);
             tl_stream<NB>(xlane1, xrow1, a.data[0], a.row_offset[0], lane_w, hi, q0_, qe_, max(qe_ - 1, q0_),
                           bvecO, wB, oB,
-                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); } TL_TRC_ARG);
+                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); });
         }
         TL_FFN_PRELOAD(data1, poff1, bvecF, wA, oA)
         TlLnOperands<NB, NW, NW> lnop1; // (requested here: their latency runs under the wait for the other waves)
@@ -1457,10 +1313,8 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
         const int fq = p + 1 - behind; // the first-linear phase this wave runs before S(p)
         if (fq >= 1 && fq < a.nchunk) {
             const int bvecF2 = TL_FFN_BVEC1(min(fq + 1, a.nchunk - 1)); // (scalar loads, used after the stream)
-            TL_STAMP(5);
             if (fq >= 2) // F(fq) overwrites the buffer that S(fq-2) read
                 tl_wait_count(ctr + TL_FFN_MAX_PHASES + fq - 2, NW);
-            TL_STAMP(6);
             TL_FFN_FIRST(fq, bvecFn, b1n, wB, oB)
             bvecFn = bvecF2;
             if (fq + 1 < a.nchunk) { // F(fq+1), a stream (or two) ahead
@@ -1468,15 +1322,13 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
                 TL_FFN_BIAS1(b1n, fq + 1)
             }
         }
-        TL_STAMP(7);
         tl_wait_count(ctr + p, NW); // hidden buffer p & 1 is complete
-        TL_STAMP(8);
         {
             const char *const xlane2 =
                 reinterpret_cast<const char *>(hs + (p & 1) * hbuf + c16 * ldh + x.khalf8);
             const int q0_ = __builtin_amdgcn_readfirstlane(bvecS), qe_ = __builtin_amdgcn_readlane(bvecS, NB);
             tl_stream<NB>(xlane2, xrow2, data2, poff2, lane_w, hi, q0_, qe_, max(qe_ - 1, q0_), bvecS, wA, oA,
-                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); } TL_TRC_ARG);
+                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); });
             tl_signal(ctr + TL_FFN_MAX_PHASES + p, lane);
         }
         bvecS = bvecSn;
@@ -1507,14 +1359,6 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
                                        acc, b2);
     __syncthreads(); // every wave's part of the rows is staged
     tl_ln_rows(lnop, a, stage0, wave, lane, x.m0, a.Y[L2], N2);
-#ifdef TL_STAGETRACE
-    TL_STAMP(9);
-    __syncthreads();
-    if (rp == 0 && g_stage_trace)
-        for (int i = threadIdx.x; i < 8 * 192; i += blockDim.x)
-            g_stage_trace[i] = reinterpret_cast<unsigned long long *>(ctr + 2 * TL_FFN_MAX_PHASES)[i];
-#endif
-#undef TL_TRC_ARG
 }
 
 // ---------------------------------------------------------------------------
@@ -1831,9 +1675,6 @@ static int g_tile_fuse_ffn = 2; // et_tuning_set("tile_fuse_ffn"): 1 feed-forwar
 static size_t ffn_lds_bytes(int K1, int KC2) {
     const size_t ldx = K1 + ((K1 & 31) ? 0 : TL_PAD), ldh = KC2 + ((KC2 & 31) ? 0 : TL_PAD);
     size_t panels = (size_t)TL_BM * (ldx + 2 * ldh) * sizeof(f16) + 2 * TL_FFN_MAX_PHASES * sizeof(unsigned);
-#ifdef TL_STAGETRACE
-    panels += 8 * 192 * 8;
-#endif
     const size_t staging = (size_t)TL_FFN_WAVES * TL_BM * (16 * 3 + 8) * sizeof(f16);
     return std::max(panels, staging);
 }
@@ -1843,6 +1684,9 @@ static size_t ffn_lds_bytes(int K1, int KC2) {
 static int tile_launch_ffn(const TlProblem *pO, const TlProblem &p1, const TlProblem &p2, const f16 *X,
                            int M, int K1, int KC2, int nchunk2, const f16 *skip, const f16 *gamma,
                            const f16 *beta, const f16 *gamma2, const f16 *beta2, hipStream_t st) {
+    // the kernel's LDS event counters cover TL_FFN_MAX_PHASES phases: every launch passes through here
+    ET_REQUIRE(nchunk2 >= 1 && nchunk2 <= TL_FFN_MAX_PHASES, ET_ERR_UNSUPPORTED,
+               "fused feed-forward: %d phases, the kernel covers %d", nchunk2, TL_FFN_MAX_PHASES);
     TlArgs a;
     memset(&a, 0, sizeof(a));
     const TlProblem *ps[3] = {pO ? pO : &p1, pO ? &p1 : &p2, &p2};
@@ -2683,15 +2527,3 @@ extern "C" int et_tile_plan_run(const et_tile_plan *plan, void *Y, const void *X
                        plan->nchunk, gelu != 0, TL_PLAN, static_cast<hipStream_t>(stream));
 }
 
-#ifdef TL_STAGETRACE
-extern "C" int et_debug_stage_trace(void *buf) {
-    return hipMemcpyToSymbol(HIP_SYMBOL(et::g_stage_trace), &buf, sizeof(buf)) == hipSuccess ? 0 : -1;
-}
-#endif
-#ifdef TL_TRACE
-// profiling builds only: per-wave phase tick counters are written to `buf`
-// (8 x u64 per wave, indexed by hardware workgroup id)
-extern "C" int et_debug_trace(void *buf) {
-    return hipMemcpyToSymbol(HIP_SYMBOL(et::g_trace), &buf, sizeof(buf)) == hipSuccess ? 0 : -1;
-}
-#endif

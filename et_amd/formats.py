@@ -100,7 +100,8 @@ def tile_mat_load(path):
     row_offset = np.zeros(max(nt, 1), np.int32)
     data = np.zeros(max(nt, 1) * 256, np.float16)
     bias = np.zeros(out_feat, np.float16)
-    check(lib().et_tile_mat_load(str(path).encode(), _ptr(row_ptr), _ptr(row_offset), _ptr(data), _ptr(bias)))
+    check(lib().et_tile_mat_load(str(path).encode(), in_feat, out_feat, nt, _ptr(row_ptr), _ptr(row_offset), _ptr(data),
+                                 _ptr(bias)))
     return dict(in_feat=in_feat, out_feat=out_feat, row_ptr=row_ptr, row_offset=row_offset[:nt].copy(),
                 data=data[:nt * 256].copy(), bias=bias)
 
@@ -123,5 +124,5 @@ def row_mat_load(path):
     row_id = np.zeros(max(n, 1), np.int32)
     weight = np.zeros((max(n, 1), in_feat), np.float16)
     bias = np.zeros(out_feat, np.float16)
-    check(lib().et_row_mat_load(str(path).encode(), _ptr(row_id), _ptr(weight), _ptr(bias)))
+    check(lib().et_row_mat_load(str(path).encode(), in_feat, out_feat, n, _ptr(row_id), _ptr(weight), _ptr(bias)))
     return dict(in_feat=in_feat, out_feat=out_feat, row_id=row_id[:n].copy(), weight=weight[:n].copy(), bias=bias)

@@ -305,18 +305,22 @@ int et_prune_row_mat(const void *W, int N, int K, float sparsity, int *row_id);
  * bytes, FNV-1a 64 of the payload) followed by
  *   tile_mat: row_ptr[out_feat/16+1], row_offset[ntile], data[ntile*256], bias[out_feat]
  *   row_mat : row_id[nrow], weight[nrow x in_feat] (compact rows), bias[out_feat]
- * _peek reads the sizes so that the caller can allocate; _load verifies size,
- * checksum and the format's invariants (ET_ERR_FORMAT) and fills the arrays. */
+ * _peek reads the sizes so that the caller can allocate; _load is told the
+ * sizes that the arrays were allocated for, refuses a file whose header says
+ * otherwise before it writes anything (the file may have changed since the
+ * peek), verifies size, checksum and the format's invariants (ET_ERR_FORMAT)
+ * and fills the arrays. */
 int et_tile_mat_save(const char *path, int in_feat, int out_feat, int ntile,
                      const int *row_ptr, const int *row_offset, const void *data,
                      const void *bias);
 int et_tile_mat_peek(const char *path, int *in_feat, int *out_feat, int *ntile);
-int et_tile_mat_load(const char *path, int *row_ptr, int *row_offset, void *data,
-                     void *bias);
+int et_tile_mat_load(const char *path, int in_feat, int out_feat, int ntile,
+                     int *row_ptr, int *row_offset, void *data, void *bias);
 int et_row_mat_save(const char *path, int in_feat, int out_feat, int nrow,
                     const int *row_id, const void *weight, const void *bias);
 int et_row_mat_peek(const char *path, int *in_feat, int *out_feat, int *nrow);
-int et_row_mat_load(const char *path, int *row_id, void *weight, void *bias);
+int et_row_mat_load(const char *path, int in_feat, int out_feat, int nrow,
+                    int *row_id, void *weight, void *bias);
 
 /* 0 if (row_ptr,row_offset) is a well-formed tile_mat of W[N x K]
  * (the asserts of test/tile_mat.cu:31-33 plus range/alignment/duplicates). */

@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
     assert not missing, missing
     # and the Python binding covers the same set
     assert set(_lib.PROTOTYPES) == set(syms)
-    assert _lib.lib().et_abi_version() == 1
+    assert _lib.lib().et_abi_version() == 2
 
 
 @pytest.mark.parametrize("N,K,sp", [(768, 768, 0.8), (3072, 768, 0.5), (768, 3072, 0.9), (64, 96, 0.33), (16, 16, 0.0), (32, 32, 1.0)])
@@ -148,6 +148,14 @@ def test_pruned_weight_containers_round_trip_and_reject_damage(tmp_path):
     with pytest.raises(EtError) as e:
         formats.tile_mat_load(tmp_path / "missing")
     assert e.value.code == -6
+    # arrays sized for another file (or a file that changed after the peek): refused before anything is written
+    from et_amd._lib import lib
+    guard = np.full(8, 7, np.int32)
+    rc = lib().et_tile_mat_load(str(p).encode(), K, N - 16, 3, guard.ctypes.data, guard.ctypes.data, guard.ctypes.data,
+                                guard.ctypes.data)
+    assert rc == -5 and (guard == 7).all()
+    rc = lib().et_row_mat_load(str(q).encode(), K, N, ids.size - 1, guard.ctypes.data, guard.ctypes.data, guard.ctypes.data)
+    assert rc == -5 and (guard == 7).all()
     with pytest.raises(EtError):                                      # unsorted row ids are refused on save
         formats.row_mat_save(tmp_path / "x", K, N, ids[::-1], W[ids], bias)
 
