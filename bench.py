@@ -33,14 +33,43 @@ MFMA_F16_PEAK_TF = 2500.0   # MI355X dense fp16 MFMA, published
 
 D, H, DFF = 768, 12, 3072
 
-# HBM bytes per launch (fetch + write, MiB) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the
-# default workload and scaled by the 64 MiB copy kernel launched below; commands and raw figures are in
-# profiles/encoder_layer_b16_s512_hbm_traffic.txt.  Only valid for batch 16 x seq 512 at 80 % sparsity.
-MEASURED_TRAFFIC_MIB = {
-    "tile_linear qkv (3 x 768->768, one launch)": 17.95 + 36.01,
-    "attention (on-the-fly)": 36.08 + 12.00,
-    "layer tail: o + skip + LayerNorm + feed-forward (gelu) + skip + LayerNorm, fused": 43.44 + 14.00,
+# HBM bytes per launch come from profiles/encoder_layer_b16_s512_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE, scaled by the 64 MiB copy kernel launched below).  The summary records a fingerprint of the kernel
+# sources it was measured on; when the sources have changed since, `traffic` is null rather than a stale figure.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "encoder_layer_b16_s512_hbm_traffic.txt")
+KERNEL_SOURCES = ("tile_linear.hip", "attention.hip", "skip_layernorm.hip", "common.h")
+TRAFFIC_KERNELS = {  # bench line -> kernel name prefix in the profile summary
+    "tile_linear qkv (3 x 768->768, one launch)": "et::tile_linear_resident_kernel",
+    "attention (on-the-fly)": "et::attention_kernel",
+    "layer tail: o + skip + LayerNorm + feed-forward (gelu) + skip + LayerNorm, fused": "et::tile_ffn_fused_kernel",
 }
+
+
+def kernel_source_fingerprint():
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "et_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic_mib():
+    """{kernel prefix: fetch + write MiB per launch} from the profile summary, or {} when it is stale or absent"""
+    import re
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return {}
+    m = re.search(r"kernel sources fingerprint:\s*([0-9a-f]+)", text)
+    if not m or m.group(1) != kernel_source_fingerprint():
+        return {}
+    out = {}
+    for line in text.splitlines():
+        m = re.match(r"(\S.*?)\s+n=\s*\d+\s+fetch avg\s+([0-9.]+) MiB\s+write avg\s+([0-9.]+) MiB", line)
+        if m:
+            out[m.group(1).split("<")[0]] = float(m.group(2)) + float(m.group(3))
+    return out
 
 
 def tile_bytes(T, N, K, ntile):
@@ -51,10 +80,20 @@ def tile_flops(T, ntile):
     return 512 * ntile * T
 
 
+def product_tile_linear(r, N, K, sparsity, seed, std=0.02):
+    """dense W ~ N(0, std) -> seeded tile_mat through the library's own generator and packer
+    (et_gen_sparse_tile_mat / et_tile_pack); same dictionary as tests/helpers.make_tile_linear"""
+    from et_amd import formats
+    from helpers import randn_h
+    W = randn_h(r, (N, K), std)
+    row_ptr, row_offset = formats.gen_sparse_tile_mat(N, K, sparsity, seed)
+    return dict(W=W, row_ptr=row_ptr, row_offset=row_offset, data=formats.tile_pack(W, row_ptr, row_offset),
+                bias=np.zeros(N, np.float16), N=N, K=K)
+
+
 def build_layer(orc, r, sparsity, seed):
-    from helpers import make_tile_linear, randn_h
     shapes = [(D, D)] * 4 + [(DFF, D), (D, DFF)]
-    lins = [make_tile_linear(r, n, k, sparsity, seed=seed + j, std=0.02) for j, (n, k) in enumerate(shapes)]
+    lins = [product_tile_linear(r, n, k, sparsity, seed=seed + j) for j, (n, k) in enumerate(shapes)]
     ln = [np.ones(D, np.float16), np.zeros(D, np.float16), np.ones(D, np.float16), np.zeros(D, np.float16)]
     return lins, ln
 
@@ -185,8 +224,9 @@ def main():
                      "TFLOPs": round(flops / us / 1e6, 1), "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TF, 4),
                      "bound": bound})
     default_cfg = (B, S, args.sparsity) == (16, 512, 0.8)
+    traffic = measured_traffic_mib() if default_cfg else {}
     for k in kern:
-        mib = MEASURED_TRAFFIC_MIB.get(k["kernel"]) if default_cfg else None
+        mib = traffic.get(TRAFFIC_KERNELS.get(k["kernel"], ""))
         k["traffic_MB"] = None if mib is None else round(mib * 1.048576, 2)
     dom = max(kern, key=lambda k: k["us"])
     if dom["bound"] == "hbm":
@@ -200,15 +240,20 @@ def main():
     layer_flops = sum(k["GFLOP"] for k in kern)
     total_us = sum(k["us"] for k in kern)
 
-    # ---- parity spot check of the timed configuration (rows of the first sequence)
-    got = out[:S].float().cpu().numpy()
-    want = orc.encoder_tile_layer(x_h[:S], lins, ln, mask_h, S, H, 1, None, 1.0).astype(np.float32)
+    # ---- parity spot check of the timed configuration: three sequences from across the batch (sequences do
+    # not interact, so the oracle runs them as a batch of their own)
+    sample = sorted({0, B // 2, B - 1})
+    srows = np.concatenate([np.arange(b * S, (b + 1) * S) for b in sample])
+    got = out.float().cpu().numpy()[srows]
+    want = orc.encoder_tile_layer(x_h[srows], lins, ln, mask_h, S, H, len(sample), None, 1.0).astype(np.float32)
     max_abs = float(np.abs(got - want).max())
     mean_rel = float(np.abs(got - want).mean() / np.abs(want).mean())
 
-    # ---- CPU baseline: the fp32 host-loop oracle on a bounded sample of the same workload
-    cpu = None
+    # ---- CPU baseline: the fp32 host-loop oracle on a bounded sample of the same workload, with all host
+    # threads and with one
+    cpu = cpu1 = None
     if not args.no_cpu:
+        import ctypes
         cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
         orc.encoder_tile_layer(x_h[:S], lins, ln, mask_h, S, H, 1, None, 1.0)  # warm
         passes, t0 = 0, time.perf_counter()
@@ -227,6 +272,23 @@ def main():
         cpu = {"value": round(passes * B / dt, 3), "unit": "seqs/s", "cores": cores, "cpu_model": model, "kind": "port",
                "sample": f"{passes} passes over all {B} sequences (seq {S}) through the fp32 host-loop oracle layer, {dt:.1f} s",
                "ms_per_seq": round(dt / (passes * B) * 1e3, 2)}
+        # one thread: single sequences of the same workload for about 8 s (the oracle's loops are OpenMP;
+        # the thread count is set through the OpenMP runtime that the oracle library has loaded)
+        try:
+            gomp = ctypes.CDLL("libgomp.so.1")
+            gomp.omp_set_num_threads(1)
+            n1, t0 = 0, time.perf_counter()
+            while n1 < B:
+                orc.encoder_tile_layer(x_h[n1 * S:(n1 + 1) * S], lins, ln, mask_h, S, H, 1, None, 1.0)
+                n1 += 1
+                dt1 = time.perf_counter() - t0
+                if dt1 >= 8.0:
+                    break
+            gomp.omp_set_num_threads(cores)
+            cpu1 = {"value": round(n1 / dt1, 3), "unit": "seqs/s", "cores": 1, "cpu_model": model, "kind": "port",
+                    "sample": f"{n1} single sequences (seq {S}) through the same oracle layer with one thread, {dt1:.1f} s"}
+        except OSError:
+            cpu1 = None
 
     extras = {}
     if args.extras:
@@ -244,18 +306,75 @@ def main():
         "layer_GFLOP_surviving": round(layer_flops, 2),
         "layer_mfma_frac": round(layer_flops / (ms_per_step * 1e3) * 1e3 / MFMA_F16_PEAK_TF, 4),  # GFLOP/us = PFLOP/s
         "sum_kernel_us": round(total_us, 1),
-        "parity_vs_oracle": {"max_abs": round(max_abs, 5), "mean_rel": round(mean_rel, 6), "rows": S},
-        "roofline": roof, "kernels": kern, "cpu_baseline": cpu,
+        "parity_vs_oracle": {"max_abs": round(max_abs, 5), "mean_rel": round(mean_rel, 6), "rows": int(srows.size),
+                             "sequences": sample},
+        "roofline": roof, "kernels": kern, "cpu_baseline": cpu, "cpu_baseline_1thread": cpu1,
     }
+    res.update(second_targets(torch, K, dev, enc, out, x, B, S, mask_h, lins, ln))
     if extras:
         res["extras"] = extras
     print(json.dumps(res))
 
 
+def event_time(torch, fn, reps=100, warm=10):
+    for _ in range(warm):
+        fn()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps * 1e3  # us
+
+
+def second_targets(torch, K, dev, enc, out, x, B, S, mask_h, lins, ln):
+    """Figures that belong in the default line next to the headline: the stand-alone skip + LayerNorm on
+    operands beyond the 256 MB last-level cache (an HBM figure, not a cache figure), BASELINE config 1
+    (dense layer, batch 1 x seq 128) and the headline layer with a padding mask instead of the all-zero one."""
+    from et_amd.encoder import Encoder_tile, Linear_tile
+    from helpers import randn_h, rng
+    res = {}
+    rows = 131072
+    gam = torch.ones(D, dtype=torch.float16, device=dev)
+    bet = torch.zeros(D, dtype=torch.float16, device=dev)
+    a_ = torch.randn((rows, D), device=dev).to(torch.float16)
+    s_ = torch.randn((rows, D), device=dev).to(torch.float16)
+    us = event_time(torch, lambda: K.skip_layernorm(a_, s_, gam, bet), reps=30, warm=3)
+    nbytes = 6.0 * rows * D + 4 * D
+    res["skip_layernorm"] = {"rows": rows, "width": D, "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                             "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                             "operand_MB": round(4.0 * rows * D / 1e6, 1)}
+    del a_, s_
+    # config 1: dense layer, batch 1 x seq 128
+    r = rng(8)
+    S1 = 128
+    lins1, ln1 = build_layer(None, r, 0.0, seed=50)
+    x1 = torch.from_numpy(randn_h(r, (S1, D))).to(dev)
+    ws1 = torch.empty(Encoder_tile.buffer_size(D, S1, H, 1) // 2, dtype=torch.float16, device=dev)
+    L1 = [Linear_tile(l["K"], l["N"], S1, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], j == 4)
+          for j, l in enumerate(lins1)]
+    enc1 = Encoder_tile(D, S1, H, ws1, *L1, *ln1, np.zeros((S1, S1), np.float16), 1)
+    o1 = torch.empty_like(x1)
+    res["config1_us"] = round(event_time(torch, lambda: enc1.run(o1, x1)), 2)
+    # the headline layer with a padding mask (the last 64 keys masked out): the attention launch then runs
+    # the form that reads and adds mask tiles, which the all-zero mask of the headline skips
+    pm = np.zeros((S, S), np.float16)
+    pm[:, S - 64:] = -30000.0
+    T = B * S
+    Lp = [Linear_tile(l["K"], l["N"], T, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], j == 4)
+          for j, l in enumerate(lins)]
+    wsp = torch.empty(Encoder_tile.buffer_size(D, S, H, B) // 2, dtype=torch.float16, device=dev)
+    encp = Encoder_tile(D, S, H, wsp, *Lp, *ln, pm, B)
+    res["latency_us_padding_mask"] = round(event_time(torch, lambda: encp.run(out, x), reps=50), 1)
+    return res
+
+
 def run_extras(torch, orc, K, dev):
     """Other BASELINE configurations, timed with HIP events (reported, not the headline)."""
     from et_amd.encoder import Encoder_tile, Linear_tile
-    from helpers import make_tile_linear, randn_h, rng
+    from helpers import randn_h, rng
     out = {}
 
     def timeit(fn, reps=100, warm=10):
@@ -290,7 +409,7 @@ def run_extras(torch, orc, K, dev):
     Y = torch.empty((M, N), dtype=torch.float16, device=dev)
     sweep = []
     for sp in (0.0, 0.5, 0.8, 0.9):
-        lin = make_tile_linear(r, N, Kd, sp, seed=11, std=0.02)
+        lin = product_tile_linear(r, N, Kd, sp, seed=11)
         nt = lin["row_offset"].size
         lt = Linear_tile(Kd, N, M, nt, lin["data"], lin["row_ptr"], lin["row_offset"], lin["bias"])
         us = timeit(lambda: lt.run(X, out=Y))
@@ -377,7 +496,7 @@ def run_extras(torch, orc, K, dev):
     o_id, m1_id, m2_id = (orc.gen_sparse_row_mat(n, 0.7, seed=s) for n, s in ((D, 12), (DFF, 13), (D, 14)))
     rw = lambda n, k: randn_h(r, (n, k), 0.02)
     zb = lambda n: np.zeros(n, np.float16)
-    vt = make_tile_linear(r, D, D, 0.0, seed=15, std=0.02)
+    vt = product_tile_linear(r, D, D, 0.0, seed=15)
     Lq, Lk = (Linear_row(D, D, T, rw(qk_id.size, D), qk_id, qk_id.size, zb(qk_id.size), H) for _ in range(2))
     Lv = Linear_tile(D, D, T, vt["row_offset"].size, vt["data"], vt["row_ptr"], vt["row_offset"], vt["bias"])
     Lo = Linear_row(D, D, T, rw(o_id.size, D), o_id, o_id.size, zb(o_id.size), H)
