@@ -301,23 +301,61 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
         // column) it fetches; lanes that land in the row padding fetch the
         // row's first bytes.  Rows at or beyond len re-read the last valid row
         // (their scores are masked to -inf / their P is 0).
+        // For a tile whose 64 keys all exist, a lane's source is "tile base + an
+        // offset that never changes": the offsets are worked out once (byte
+        // offsets in 32 bits, relative to the first row of the tile in K or V)
+        // and an instruction then costs no address arithmetic in the vector ALU -
+        // it was a quarter of the loop's vector instructions.
+        constexpr int DMA_ROWBK = LDK * 2, DMA_ROWBV = LDVN * 2; // LDS bytes per row
+        constexpr int DMA_NK = (DMA && !SHAREDQK) ? AT_KT * DMA_ROWBK / 1024 : 0;
+        constexpr int DMA_NV = DMA ? AT_KT * DMA_ROWBV / 1024 : 0;
+        constexpr int DMA_NTOT = DMA_NK + DMA_NV;
+        constexpr int DMA_PW = DMA ? (DMA_NTOT + AT_WAVES - 1) / AT_WAVES : 1; // instructions per wave
+        unsigned dma_off[DMA_PW];
+        if (DMA) {
+#pragma unroll
+            for (int j = 0; j < DMA_PW; j++) {
+                const int i = j * AT_WAVES + wave;
+                const bool isv = i >= DMA_NK;
+                const int ii = isv ? i - DMA_NK : i;
+                const int p = ii * 1024 + lane * 16;
+                const int rowb = isv ? DMA_ROWBV : DMA_ROWBK;
+                const int row = p / rowb, cb = p - row * rowb;
+                const int col = cb < (isv ? HD : HDK) * 2 ? (cb >> 1) : 0;
+                dma_off[j] = (unsigned)((row * (isv ? a.ldv : a.ldq) + col) * 2);
+            }
+        }
         auto dma_tile = [&](int kb, int buf) {
-            constexpr int ROWBK = LDK * 2, ROWBV = LDVN * 2; // LDS bytes per row
-            constexpr int NINSTK = SHAREDQK ? 0 : AT_KT * ROWBK / 1024, NINSTV = AT_KT * ROWBV / 1024;
-            static_assert(AT_KT * ROWBK % 1024 == 0 && AT_KT * ROWBV % 1024 == 0,
+            static_assert(!DMA || (AT_KT * DMA_ROWBK % 1024 == 0 && AT_KT * DMA_ROWBV % 1024 == 0),
                           "a tile is a whole number of DMA instructions");
-            constexpr int NTOT = NINSTK + NINSTV;
             f16 *ks = smem + buf * (KBUF + VBUF);
             f16 *vs = ks + KBUF;
+            if (PLAIN || kb + AT_KT <= len) { // (wave-uniform; always so in the plain form)
+                const char *kbase = reinterpret_cast<const char *>(a.K + (size_t)(row0 + kb) * a.ldq + qc0);
+                const char *vbase = reinterpret_cast<const char *>(a.V + (size_t)(row0 + kb) * a.ldv + vc0);
 #pragma unroll
-            for (int i0 = 0; i0 < NTOT; i0 += AT_WAVES) {
+                for (int j = 0; j < DMA_PW; j++) {
+                    const int i = j * AT_WAVES + wave;
+                    if (DMA_NTOT % AT_WAVES != 0 && i >= DMA_NTOT)
+                        break;
+                    const bool isv = i >= DMA_NK;
+                    const int ii = isv ? i - DMA_NK : i;
+                    // (kept opaque in place: otherwise the offsets are folded into 64-bit vector
+                    // addresses again, one 64-bit add per instruction and tile)
+                    asm("" : "+v"(dma_off[j]));
+                    load_lds16((isv ? vbase : kbase) + dma_off[j], (isv ? vs : ks) + ii * 512);
+                }
+                return;
+            }
+#pragma unroll
+            for (int i0 = 0; i0 < DMA_NTOT; i0 += AT_WAVES) {
                 const int i = i0 + wave;
-                if (NTOT % AT_WAVES != 0 && i >= NTOT)
+                if (DMA_NTOT % AT_WAVES != 0 && i >= DMA_NTOT)
                     break;
-                const bool isv = i >= NINSTK;
-                const int ii = isv ? i - NINSTK : i;
+                const bool isv = i >= DMA_NK;
+                const int ii = isv ? i - DMA_NK : i;
                 const int p = ii * 1024 + lane * 16;
-                const int rowb = isv ? ROWBV : ROWBK;
+                const int rowb = isv ? DMA_ROWBV : DMA_ROWBK;
                 const int row = p / rowb, cb = p - row * rowb;
                 const int rr = min(kb + row, len - 1);
                 const int col = cb < (isv ? HD : HDK) * 2 ? (cb >> 1) : 0;
