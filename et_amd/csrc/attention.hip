@@ -108,14 +108,22 @@ __device__ __forceinline__ float xor_max_16_32(float v) {
 // the same number of kept columns in every head: Q and K are compact
 // [rows x nhead*HDK], head h at columns h*HDK, and the scores contract over
 // HDK; V and the output keep HD columns per head.
-template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK, bool PLAIN = false, int HDK = HD>
+// VWIN (pruned variant with dense Q/K and compact V whose row pitch is a
+// multiple of 8): K and V are staged by DMA like the unpruned kernel.  A head's
+// compact value columns [c0, c1) start at an arbitrary column, which DMA cannot
+// address (16-byte pieces), so the tile holds the 16-byte-aligned WINDOW of 80
+// columns that begins at c0 rounded down to 8; the product runs over the
+// window's 16-column subtiles that reach into [c0, c1) (at most five), and the
+// columns of the window that belong to neighbouring heads are never written.
+template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK, bool PLAIN = false, int HDK = HD, bool VWIN = false>
 __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attention_kernel(const AttnArgs a) {
-    static_assert(!PLAIN || (!PRUNED && !SHAREDQK), "the plain form exists for the on-the-fly kernel only");
+    static_assert(!PLAIN || ((!PRUNED || VWIN) && !SHAREDQK), "the plain form exists for the DMA-staged kernels only");
     static_assert(HDK == HD || (!PRUNED && !SHAREDQK && HDK % 32 == 0), "narrow Q/K heads: on-the-fly kernel only");
+    static_assert(!VWIN || (PRUNED && HD == 64), "the value-window form exists for the pruned kernel with 64-wide heads");
     constexpr int AT_THREADS = NW * 64; // NW waves, each owning 16*QS query rows
     constexpr int AT_WAVES = NW;
     constexpr int DK = HDK / 32;   // k-steps of Q K^T
-    constexpr int DV = HD / 16;    // 16-wide column subtiles of the output
+    constexpr int DV = VWIN ? 5 : HD / 16; // 16-wide column subtiles of the output (of the 80-column window)
     // LDS row strides.  K rows are read with ds_read_b128 by 16 lanes at a
     // time: a stride of 32 (mod 64) bytes is conflict-free (measured); V^T rows
     // are read with ds_read_b64, for which an odd multiple of 16 bytes is.
@@ -127,8 +135,9 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
     // natural [key][d] layout, K and V alike; the transposed V^T fragments the
     // second contraction needs are then produced by the LDS transpose read
     // (ds_read_b64_tr_b16).  The pruned variant gathers ragged column sets and
-    // keeps the register path, which transposes V while storing it.
-    constexpr bool DMA = !PRUNED;
+    // keeps the register path, which transposes V while storing it - except in
+    // its value-window form (VWIN), which is DMA-staged as well.
+    constexpr bool DMA = !PRUNED || VWIN;
     constexpr int LDVN = HD + 16; // V row stride in the natural layout (as LDK)
     constexpr int KBUF = AT_KT * LDK, VBUF = DMA ? AT_KT * LDVN : HD * LDV;
     constexpr int SM_KV = 2 * (KBUF + VBUF); // double-buffered key/value tiles
@@ -176,6 +185,13 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
             nv = min(a.v_head_ptr[h + 1] - vc0, HD);
         }
     }
+    // value window: vskip columns of a neighbouring head in front of the head's own nv
+    int vskip = 0;
+    if (VWIN) {
+        vskip = vc0 & 7;
+        vc0 -= vskip;
+        nv += vskip; // columns of the window up to the head's last one
+    }
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -197,7 +213,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 f16x8 v = zero8;
                 if (!SHAREDQK && q < len) {
                     const f16 *qrow = a.Q + (size_t)(row0 + q) * a.ldq + qc0;
-                    if (PRUNED)
+                    if (PRUNED && !VWIN)
                         v = load8_guard(qrow, s * 32 + g4 * 8, nqk);
                     else
                         v = *reinterpret_cast<const f16x8 *>(qrow + s * 32 + g4 * 8);
@@ -321,7 +337,9 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 const int p = ii * 1024 + lane * 16;
                 const int rowb = isv ? DMA_ROWBV : DMA_ROWBK;
                 const int row = p / rowb, cb = p - row * rowb;
-                const int col = cb < (isv ? HD : HDK) * 2 ? (cb >> 1) : 0;
+                int col = cb < (isv ? HD : HDK) * 2 ? (cb >> 1) : 0;
+                if (VWIN && isv) // all 80 columns of a window row are data; pieces past the row pitch re-read its last one
+                    col = min(cb >> 1, a.ldv - 8 - vc0);
                 dma_off[j] = (unsigned)((row * (isv ? a.ldv : a.ldq) + col) * 2);
             }
         }
@@ -358,7 +376,9 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 const int rowb = isv ? DMA_ROWBV : DMA_ROWBK;
                 const int row = p / rowb, cb = p - row * rowb;
                 const int rr = min(kb + row, len - 1);
-                const int col = cb < (isv ? HD : HDK) * 2 ? (cb >> 1) : 0;
+                int col = cb < (isv ? HD : HDK) * 2 ? (cb >> 1) : 0;
+                if (VWIN && isv)
+                    col = min(cb >> 1, a.ldv - 8 - vc0);
                 const f16 *src = isv ? a.V + (size_t)(row0 + rr) * a.ldv + vc0 + col
                                      : a.K + (size_t)(row0 + rr) * a.ldq + qc0 + col;
                 load_lds16(src, (isv ? vs : ks) + ii * 512);
@@ -370,6 +390,15 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
         const int nt = (len + AT_KT - 1) / AT_KT;
         // all of this wave's query rows valid?  (wave-uniform)
         const bool wave_rows_ok = q0 + (wave + 1) * QS * 16 <= len;
+        // value window: the output column (within the head) of every window column, -1 for the columns of
+        // other heads; kept behind the tile buffers for the epilogue
+        int *wcol = reinterpret_cast<int *>(at_smem + SM * 2);
+        if (VWIN && tid < DV * 16) {
+            int c = -1;
+            if (tid >= vskip && tid < nv)
+                c = (a.v_col_id ? a.v_col_id[vc0 + tid] : vc0 + tid) - h * HD;
+            wcol[tid] = (c >= 0 && c < HD) ? c : -1;
+        }
         if (DMA) {
             dma_tile(0, 0);
             __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
@@ -693,7 +722,14 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
 #pragma unroll
                 for (int r = 0; r < 4; r++)
                     o[r] = (f16)(ot[d][qs][r] * inv);
-                if (PRUNED) {
+                if (VWIN) {
+                    typedef int i32x4 __attribute__((ext_vector_type(4)));
+                    const i32x4 c4 = *reinterpret_cast<const i32x4 *>(wcol + d * 16 + g4 * 4);
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (c4[r] >= 0)
+                            os[ql * LDO + c4[r]] = o[r];
+                } else if (PRUNED) {
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
                         const int j = d * 16 + g4 * 4 + r;
@@ -776,17 +812,17 @@ qk_scores_kernel(f16 *__restrict__ QK, const f16 *__restrict__ Q, const f16 *__r
 }
 
 // LDS bytes of one workgroup (mirrors the constants inside the kernel)
-template <int HD, int QS, int NW, bool PRUNED, int HDK = HD> constexpr size_t attn_lds_bytes() {
+template <int HD, int QS, int NW, bool PRUNED, int HDK = HD, bool VWIN = false> constexpr size_t attn_lds_bytes() {
     // (must agree with the kernel's KBUF / VBUF)
-    constexpr int KV = 2 * (AT_KT * (HDK + 16) + (PRUNED ? HD * (AT_KT + 8) : AT_KT * (HD + 16)));
+    constexpr int KV = 2 * (AT_KT * (HDK + 16) + ((PRUNED && !VWIN) ? HD * (AT_KT + 8) : AT_KT * (HD + 16)));
     constexpr int O = NW * 16 * QS * (HD + 8);
-    return sizeof(f16) * (size_t)(KV > O ? KV : O);
+    return sizeof(f16) * (size_t)(KV > O ? KV : O) + (VWIN ? 5 * 16 * sizeof(int) : 0); // (+ the window's column table)
 }
 
-template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK, bool PLAIN = false, int HDK = HD>
+template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK, bool PLAIN = false, int HDK = HD, bool VWIN = false>
 static void attn_launch_one(const AttnArgs &a, hipStream_t st) {
-    constexpr size_t lds = attn_lds_bytes<HD, QS, NW, PRUNED, HDK>();
-    auto kern = attention_kernel<HD, QS, NW, PRUNED, SHAREDQK, PLAIN, HDK>;
+    constexpr size_t lds = attn_lds_bytes<HD, QS, NW, PRUNED, HDK, VWIN>();
+    auto kern = attention_kernel<HD, QS, NW, PRUNED, SHAREDQK, PLAIN, HDK, VWIN>;
     if (lds > 64 * 1024) { // above the default dynamic-LDS limit: opt in once per kernel
         static bool done = false;
         if (!done) {
@@ -821,6 +857,7 @@ static void attn_launch_variant(int variant, bool plain, const AttnArgs &a, hipS
 }
 
 static int g_attn_variant = -1; // et_tuning_set("attn_variant"): -1 = automatic
+static int g_attn_vwin = 1;     // et_tuning_set("attn_vwin"): 0 = pruned attention always stages through registers
 
 static float head_scale(int hd) {
     // half(sqrt(1/head_dim)), kernels/attention.cu:126
@@ -944,6 +981,21 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
         attn_launch_variant<64, false, false, 32>(variant, plain, a, st);
         return launch_status(who);
     }
+    // dense Q/K with compact V (the reference's pruned wiring): DMA-staged value windows
+    if (pruned && hd == 64 && !a.qk_head_ptr && a.v_head_ptr && a.ldq % 8 == 0 && a.ldv % 8 == 0 && a.ldv >= 8 &&
+        g_attn_vwin) {
+        if (variant == 0 && plain)
+            attn_launch_one<64, 2, 4, true, false, true, 64, true>(a, st);
+        else if (variant == 0)
+            attn_launch_one<64, 2, 4, true, false, false, 64, true>(a, st);
+        else if (variant == 1)
+            attn_launch_one<64, 1, 8, true, false, false, 64, true>(a, st);
+        else if (plain)
+            attn_launch_one<64, 1, 4, true, false, true, 64, true>(a, st);
+        else
+            attn_launch_one<64, 1, 4, true, false, false, 64, true>(a, st);
+        return launch_status(who);
+    }
     ET_ATTN_CASE(32)
     ET_ATTN_CASE(64)
     ET_ATTN_CASE(128)
@@ -952,6 +1004,7 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
 }
 
 void set_attn_variant(int v) { g_attn_variant = v; }
+void set_attn_vwin(int v) { g_attn_vwin = v; }
 
 } // namespace et
 

@@ -700,6 +700,42 @@ def test_prune_attention(K):
 
 
 @pytest.mark.parametrize("S,B,with_mask,with_lens", [(160, 2, True, True), (256, 3, False, False),
+                                                     (128, 20, False, False), (77, 1, False, True),
+                                                     (512, 11, False, False), (512, 11, True, True)])
+def test_prune_attention_value_windows(K, S, B, with_mask, with_lens):
+    """dense Q/K with compact V whose row pitch is a multiple of 8 (the reference's wiring, encoder/encoder.cu:76-79):
+    V is staged by DMA as aligned 80-column windows.  Heads that start at any column mod 8, a head that keeps all
+    64 columns behind an odd start (5 subtiles), a head that keeps none; == the oracle, and bit for bit == the
+    register-staged kernel (same products in the same order)"""
+    from et_amd._lib import lib
+    r = rng(49 + S)
+    H, d = 12, 768
+    hd = d // H
+    Q, Kk, V = (randn_h(r, (B * S, d)) for _ in range(3))
+    mask = randn_h(r, (S, S), 0.3) if with_mask else None
+    lens = r.integers(1, S + 1, size=B).astype(np.int32) if with_lens else None
+    keep = [3, 64, 0, 17, 8, 1, 64, 33, 64, 5, 21, 64]       # columns kept per head
+    v_id = np.concatenate([h * hd + np.sort(r.choice(hd, k, replace=False)) for h, k in enumerate(keep)]).astype(np.int32)
+    v_hp = orc.head_ptr(v_id, H, hd)
+    ld = (v_id.size + 7) // 8 * 8
+    Vc = np.zeros((B * S, ld), np.float16)
+    Vc[:, :v_id.size] = V[:, v_id]
+    md, lensd = (None if mask is None else dev(mask)), (None if lens is None else dev(lens))
+    want = orc.prune_attention(Q, Kk, np.ascontiguousarray(Vc[:, :v_id.size]), None, v_id, v_hp, mask, S, d, H, B, lens, f64=True)
+    got = host(K.Prune_attention(dev(Q), dev(Kk), dev(Vc), None, dev(v_id), dev(v_hp), md, S, d, H, B, lensd))
+    try:
+        lib().et_tuning_set(b"attn_vwin", 0)
+        regs = host(K.Prune_attention(dev(Q), dev(Kk), dev(Vc), None, dev(v_id), dev(v_hp), md, S, d, H, B, lensd))
+    finally:
+        lib().et_tuning_set(b"attn_vwin", 1)
+    assert np.array_equal(got, regs)
+    valid = np.ones(B * S, bool) if lens is None else np.concatenate([np.arange(S) < n for n in lens])
+    check_close(got[valid], want[valid], max_abs=5e-3, mean_rel=1e-3, what="pruned attention, value windows")
+    assert (got[~valid] == 0).all()
+    assert (got[:, np.setdiff1d(np.arange(d), v_id)] == 0).all()
+
+
+@pytest.mark.parametrize("S,B,with_mask,with_lens", [(160, 2, True, True), (256, 3, False, False),
                                                      (512, 2, True, False), (77, 1, False, True)])
 def test_otf_attention_narrow_qk_heads(K, S, B, with_mask, with_lens):
     """every head keeps 32 of its 64 Q/K columns: the on-the-fly kernel on compact Q/K
