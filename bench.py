@@ -108,11 +108,18 @@ def main():
     ap.add_argument("--sparsity", type=float, default=0.8)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--extras", action="store_true", help="also time the other BASELINE configurations")
+    ap.add_argument("--micro", action="store_true",
+                    help="only run the delivery-path microbenchmarks (LDS reads, weight stream, MFMA / vector-ALU "
+                         "co-execution) and print their figures")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures ONE GPU (the path needs no collectives; it shards by "
               "batch). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+
+    if args.micro:
+        print(json.dumps(run_micro()))
+        return
 
     import torch
     import oracle.et_oracle as orc          # checker / CPU baseline only
@@ -314,6 +321,46 @@ def main():
     if extras:
         res["extras"] = extras
     print(json.dumps(res))
+
+
+def run_micro():
+    """Delivery-path microbenchmarks (et_microbench).  Rates are per CU; "clk" figures use the clock that the
+    MFMA-only loop implies (a v_mfma_f32_16x16x32_f16 occupies its SIMD's matrix unit for 16 cycles)."""
+    import ctypes as C
+    from et_amd._lib import check, lib
+
+    def mb(what, p0, p1):
+        sec, units = C.c_double(), C.c_double()
+        check(lib().et_microbench(what, p0, p1, C.byref(sec), C.byref(units)))
+        return sec.value, units.value
+
+    res = {}
+    t_m, n_m = mb(2, 0, 4)                       # one MFMA wave per SIMD
+    clk_ghz = n_m * 16 / t_m / 1e9               # 16 cycles per MFMA
+    res["clock_GHz_from_mfma_loop"] = round(clk_ghz, 3)
+    lds = {}
+    for stride, name in ((0, "linear"), (1568, "x_panel_stride_1568"), (160, "k_tile_stride_160"), (1552, "stride_1552"),
+                         (1536, "stride_1536")):
+        t, b = mb(0, stride, 16)
+        lds[name] = {"GBps_per_CU": round(b / t / 1e9, 1), "bytes_per_clk_per_CU": round(b / t / 1e9 / clk_ghz, 1)}
+    res["lds_ds_read_b128"] = lds
+    ws = {}
+    for waves in (4, 8, 16):
+        t, b = mb(1, 0, waves)
+        ws[f"{waves}_waves"] = {"GBps_per_CU": round(b / t / 1e9, 1), "bytes_per_clk_per_CU": round(b / t / 1e9 / clk_ghz, 1)}
+    res["weight_stream_1KB_requests_from_L2"] = ws
+    co = {}
+    t_v, _ = mb(2, 1, 4)
+    t_x, _ = mb(2, 2, 4)
+    t_s, _ = mb(2, 3, 8)
+    co["mfma_only_1_wave_per_simd_ms"] = round(t_m * 1e3, 4)
+    co["fma_only_1_wave_per_simd_ms"] = round(t_v * 1e3, 4)
+    co["alternating_in_one_wave_ms"] = round(t_x * 1e3, 4)
+    co["mfma_wave_and_fma_wave_on_one_simd_ms"] = round(t_s * 1e3, 4)
+    co["same_wave_overlap"] = round(1.0 - (t_x - max(t_m, t_v)) / min(t_m, t_v), 3)   # 1 = fully hidden, 0 = added
+    co["two_wave_overlap"] = round(1.0 - (t_s - max(t_m, t_v)) / min(t_m, t_v), 3)
+    res["mfma_valu_coexecution"] = co
+    return res
 
 
 def event_time(torch, fn, reps=100, warm=10):

@@ -108,6 +108,7 @@ PROTOTYPES = {
     "et_stream_synchronize": (_i, [_vp]),
     "et_device_synchronize": (_i, []),
     "et_device_cu_count": (_i, []),
+    "et_microbench": (_i, [_i, _i, _i, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "et_tuning_set": (_i, [C.c_char_p, _i]),
 }
 

@@ -421,6 +421,21 @@ int et_device_synchronize(void);
  * Not thread-safe; results never depend on these beyond fp32 summation
  * order. */
 int et_tuning_set(const char *key, int value);
+/* Microbenchmarks of the delivery paths that bound the kernels (no counterpart
+ * in the reference; they allocate and synchronise, so not for hot paths).
+ *   what 0: LDS fragment reads (ds_read_b128); p0 = row stride in bytes of the
+ *           16-row x 64-byte fragment pattern (0: 64 x 16 consecutive bytes),
+ *           p1 = waves per CU.  units = bytes read per CU.
+ *   what 1: the weight stream: one-kilobyte global_load_dwordx4 requests, four
+ *           in flight per wave, from 2 MiB that stay in L2; p1 = waves per CU.
+ *           units = bytes requested per CU.
+ *   what 2: matrix unit and vector ALU: p0 = 0 every wave issues MFMAs only,
+ *           1 v_fma_f32 only (four per MFMA of mode 0), 2 both, strictly
+ *           alternating in every wave, 3 four waves MFMAs and four waves (on
+ *           the same SIMDs) the FMAs; p1 = waves per CU (modes 0-2).
+ *           units = v_mfma_f32_16x16x32_f16 per MFMA-issuing wave.
+ * seconds = duration of one launch on every CU of the device. */
+int et_microbench(int what, int p0, int p1, double *seconds, double *units_per_cu);
 /* number of compute units of the current device (0 if none) */
 int et_device_cu_count(void);
 
