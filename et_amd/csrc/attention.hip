@@ -486,8 +486,19 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
         auto tile_body = [&](int kb, const f16 *ks, const f16 *vt, const bool FAST, const bool MASKED) {
             // MASKED: this tile's mask values are in mk
             __builtin_amdgcn_s_setprio(AT_PRIO);
-            // ---- scores, transposed: st[ksub][qs][r] = S[q = c16][key = 16 ksub + 4 g4 + r]
+            // ---- scores, transposed: st[ksub][qs][r] = S[q = c16][key = 16 ksub + 4 g4 + r],
+            // MINUS the row's running maximum: the matrix unit starts from -m
+            // instead of zero, which costs nothing there and saves the vector
+            // ALU one subtraction per score
             f32x4 st[4][QS];
+            float m_ref[QS];
+#pragma unroll
+            for (int qs = 0; qs < QS; qs++)
+                m_ref[qs] = (m_run[qs] == -INFINITY) ? 0.f : m_run[qs];
+            f32x4 nm4[QS];
+#pragma unroll
+            for (int qs = 0; qs < QS; qs++)
+                nm4[qs] = f32x4{-m_ref[qs], -m_ref[qs], -m_ref[qs], -m_ref[qs]};
             if (!SHAREDQK) {
                 // K fragments are read one 16-key subtile ahead of the MFMAs that
                 // use them (two subtiles' worth of registers instead of four)
@@ -505,13 +516,10 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                     }
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int qs = 0; qs < QS; qs++)
-                        st[ksub][qs] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
                     for (int s = 0; s < DK; s++)
 #pragma unroll
-                        for (int qs = 0; qs < QS; qs++)
-                            st[ksub][qs] = mfma16x16x32(kfr[ksub & 1][s], qf[qs][s], st[ksub][qs]);
+                        for (int qs = 0; qs < QS; qs++) // (the first step reads -m as its C operand: no copies)
+                            st[ksub][qs] = mfma16x16x32(kfr[ksub & 1][s], qf[qs][s], s == 0 ? nm4[qs] : st[ksub][qs]);
                 }
             } else {
 #pragma unroll
@@ -533,7 +541,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                                 if (key + r < len)
                                     v[r] = (float)src[r];
                         }
-                        st[ksub][qs] = v;
+                        st[ksub][qs] = v - m_ref[qs];
                     }
                 }
             }
@@ -579,34 +587,44 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                             if (kb + ksub * 16 + g4 * 4 + r >= len)
                                 st[ksub][qs][r] = -INFINITY;
                 }
+                // the lane's part of the row maximum (of s - m_ref); the row's other three
+                // parts only matter when some row of the wave has to raise its maximum
                 float mx = -INFINITY;
 #pragma unroll
                 for (int ksub = 0; ksub < 4; ksub++) {
                     mx = fmaxf(fmaxf(mx, st[ksub][qs][0]), st[ksub][qs][1]);
                     mx = fmaxf(fmaxf(mx, st[ksub][qs][2]), st[ksub][qs][3]);
                 }
-                mx = xor_max_16_32(mx);
-                const bool up = (mx - m_run[qs]) * ls > 8.0f; // also true for the first valid tile (m_run = -inf)
-                if (__builtin_amdgcn_ballot_w64(up) != 0) {
-                    const float m_new = up ? mx : m_run[qs];
+                // (a row without a maximum yet, m_run = -inf, takes its first finite one)
+                const bool up_lane = (m_run[qs] == -INFINITY) ? (mx > -INFINITY) : (mx * ls > 8.0f);
+                if (__builtin_amdgcn_ballot_w64(up_lane) != 0) {
+                    mx = xor_max_16_32(mx);
+                    const bool up = (m_run[qs] == -INFINITY) ? (mx > -INFINITY) : (mx * ls > 8.0f);
+                    const float m_new = up ? mx + m_ref[qs] : m_run[qs];
                     const float m_fin = (m_new == -INFINITY) ? 0.f : m_new;
                     const float alpha = __builtin_amdgcn_exp2f((m_run[qs] - m_fin) * ls); // 1 where unchanged
+                    const float shift = m_fin - m_ref[qs];                                // 0 where unchanged
                     m_run[qs] = m_new;
                     l_acc[qs] *= alpha;
 #pragma unroll
                     for (int d = 0; d < DV; d++)
                         ot[d][qs] *= alpha;
+#pragma unroll
+                    for (int ksub = 0; ksub < 4; ksub++)
+                        st[ksub][qs] -= shift;
                 }
-                const float msc = ((m_run[qs] == -INFINITY) ? 0.f : m_run[qs]) * ls;
+                if (ls != 1.0f) { // (wave-uniform; base-2 softmax needs no multiplication at all)
+#pragma unroll
+                    for (int ksub = 0; ksub < 4; ksub++)
+                        st[ksub][qs] *= ls;
+                }
                 f16x2 ph[8];
 #pragma unroll
                 for (int ksub = 0; ksub < 4; ksub++)
 #pragma unroll
                     for (int r2 = 0; r2 < 2; r2++) {
-                        float p0 = __builtin_fmaf(st[ksub][qs][2 * r2], ls, -msc);
-                        float p1 = __builtin_fmaf(st[ksub][qs][2 * r2 + 1], ls, -msc);
-                        p0 = __builtin_amdgcn_exp2f(p0);
-                        p1 = __builtin_amdgcn_exp2f(p1);
+                        const float p0 = __builtin_amdgcn_exp2f(st[ksub][qs][2 * r2]);
+                        const float p1 = __builtin_amdgcn_exp2f(st[ksub][qs][2 * r2 + 1]);
                         typedef float f32x2 __attribute__((ext_vector_type(2)));
                         ph[ksub * 2 + r2] = __builtin_convertvector(f32x2{p0, p1}, f16x2);
                     }
