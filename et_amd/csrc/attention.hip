@@ -115,8 +115,9 @@ __device__ __forceinline__ float xor_max_16_32(float v) {
 // columns that begins at c0 rounded down to 8; the product runs over the
 // window's 16-column subtiles that reach into [c0, c1) (at most five), and the
 // columns of the window that belong to neighbouring heads are never written.
+// One workgroup's work: the NW*16*QS query rows of block qb of (sequence b, head h).
 template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK, bool PLAIN = false, int HDK = HD, bool VWIN = false>
-__global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attention_kernel(const AttnArgs a) {
+__device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, const int h, const int qb) {
     static_assert(!PLAIN || ((!PRUNED || VWIN) && !SHAREDQK), "the plain form exists for the DMA-staged kernels only");
     static_assert(HDK == HD || (!PRUNED && !SHAREDQK && HDK % 32 == 0), "narrow Q/K heads: on-the-fly kernel only");
     static_assert(!VWIN || (PRUNED && HD == 64), "the value-window form exists for the pruned kernel with 64-wide heads");
@@ -147,17 +148,7 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
     f16 *smem = reinterpret_cast<f16 *>(at_smem);
     static_assert(SM * 2 <= 160 * 1024, "LDS budget");
 
-    // Workgroup ids go round-robin over the 8 XCDs.  XCD x works on the
-    // (batch, head) pairs x, x+8, x+16, ... in that order, all query blocks of a
-    // pair together (they share its K and V in that XCD's L2): with sequences of
-    // different lengths every XCD gets an even mix, and pairs keep their order.
-    const int xcd = blockIdx.x & 7, rest = blockIdx.x >> 3; // rest < per_xcd = ceil(pairs / 8) * nqb
-    const int qb = rest % a.nqb;
-    const int bh = (rest / a.nqb) * 8 + xcd;
-    if (bh >= a.nhead * a.batch)
-        return;
-    const int h = bh % a.nhead;
-    const int b = bh / a.nhead;
+    const int bh = b * a.nhead + h;
 
     int row0, len, rows_alloc; // first row, valid rows, rows that exist for this sequence
     if (a.cu_seqlens) {
@@ -785,6 +776,81 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
     }
 }
 
+template <int HD, int QS, int NW, bool PRUNED, bool SHAREDQK, bool PLAIN = false, int HDK = HD, bool VWIN = false>
+__global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attention_kernel(const AttnArgs a) {
+    // Workgroup ids go round-robin over the 8 XCDs.  XCD x works on the
+    // (batch, head) pairs x, x+8, x+16, ... in that order, all query blocks of a
+    // pair together (they share its K and V in that XCD's L2): with sequences of
+    // different lengths every XCD gets an even mix, and pairs keep their order.
+    const int xcd = blockIdx.x & 7, rest = blockIdx.x >> 3; // rest < per_xcd = ceil(pairs / 8) * nqb
+    const int qb = rest % a.nqb;
+    const int bh = (rest / a.nqb) * 8 + xcd;
+    if (bh >= a.nhead * a.batch)
+        return;
+    attention_block<HD, QS, NW, PRUNED, SHAREDQK, PLAIN, HDK, VWIN>(a, bh / a.nhead, bh % a.nhead, qb);
+}
+
+// Packed sequences of different lengths (cu_seqlens): a grid of one workgroup per
+// (sequence, head, query block of the LONGEST sequence) is mostly workgroups that
+// find nothing to do, and dispatching those costs as much as the work of a batch
+// of short sequences.  Here the grid is what the chip holds at once and every
+// workgroup walks its share of the blocks that exist: XCD x owns the (sequence,
+// head) pairs x, x+8, ... as above, their query blocks in order form that XCD's
+// list, and workgroup k of the W on the XCD takes blocks k, k+W, k+2W, ... .
+// A block's position in the list is found from the running block count per
+// sequence, which every wave keeps in registers (lane l: sequences l, l+64, ...;
+// at most 64*AT_PX sequences).
+constexpr int AT_PX = 4;
+template <int HD, int QS, int NW>
+__global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attention_packed_kernel(const AttnArgs a) {
+    constexpr int QB = NW * 16 * QS;
+    const int lane = threadIdx.x & 63;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, W = gridDim.x >> 3;
+    int px[AT_PX], nbv[AT_PX]; // blocks before sequence (l + 64 r) in this XCD's list; its query blocks
+    int run = 0;
+#pragma unroll
+    for (int r = 0; r < AT_PX; r++) {
+        const int s = lane + 64 * r;
+        int nb = 0, v = 0;
+        if (s < a.batch) {
+            const int len = min(max(a.cu_seqlens[s + 1] - a.cu_seqlens[s], 0), a.seq_len);
+            nb = (len + QB - 1) / QB;
+            const int h0 = (xcd - s * a.nhead) & 7; // first head of the sequence whose pair lands on this XCD
+            v = h0 < a.nhead ? nb * ((a.nhead - h0 + 7) >> 3) : 0;
+        }
+        int inc = v; // inclusive scan over the 64 lanes
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int t = __shfl_up(inc, d, 64);
+            inc += lane >= d ? t : 0;
+        }
+        px[r] = s < a.batch ? run + inc - v : 0x7fffffff;
+        nbv[r] = nb;
+        run += __shfl(inc, 63, 64);
+    }
+    run = __builtin_amdgcn_readfirstlane(run);
+    for (int i = slot; i < run; i += W) {
+        // the sequence: the last one whose first block is at or before i (the counts never decrease, and a
+        // sequence without blocks on this XCD shares its successor's count and is passed over)
+        int cnt = 0;
+#pragma unroll
+        for (int r = 0; r < AT_PX; r++)
+            cnt += __builtin_popcountll(__builtin_amdgcn_ballot_w64(px[r] <= i));
+        const int b = cnt - 1; // (cnt >= 1: the first sequence's count is 0)
+        int first = 0, nb = 1;
+#pragma unroll
+        for (int r = 0; r < AT_PX; r++)
+            if ((b >> 6) == r) {
+                first = __builtin_amdgcn_readlane(px[r], b & 63);
+                nb = __builtin_amdgcn_readlane(nbv[r], b & 63);
+            }
+        const int rem = i - first;
+        const int h = ((xcd - b * a.nhead) & 7) + 8 * (rem / nb);
+        attention_block<HD, QS, NW, false, false, false, HD, false>(a, b, h, rem % nb);
+        __syncthreads(); // the block's output staging in LDS is read before the next block's tiles land there
+    }
+}
+
 // scaled Q K^T written to memory, [(b*nhead+h)][q][k]; one wave per 16 queries
 // x 64 keys, transposed product so a lane owns 4 consecutive keys of one query.
 template <int HD>
@@ -852,6 +918,26 @@ static void attn_launch_one(const AttnArgs &a, hipStream_t st) {
     hipLaunchKernelGGL(kern, dim3(a.per_xcd * 8), dim3(NW * 64), lds, st, a);
 }
 
+// packed sequences: as many workgroups (4 waves x 16 query rows) as the chip holds at once, or fewer
+template <int HD>
+static void attn_launch_packed(const AttnArgs &a, hipStream_t st) {
+    // (32 query rows per wave need 207 registers here, two waves per SIMD: 63 us against 48 us on a batch of
+    // 64 sequences of 32..512 rows)
+    constexpr size_t lds = attn_lds_bytes<HD, 1, 4, false>();
+    auto kern = attention_packed_kernel<HD, 1, 4>;
+    if (lds > 64 * 1024) {
+        static bool done = false;
+        if (!done) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            done = true;
+        }
+    }
+    const long resident = (long)std::max(et_device_cu_count(), 1) * (HD <= 64 ? 4 : 2);
+    const long wgs = std::min<long>(resident, a.total);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((wgs + 7) / 8 * 8)), dim3(256), lds, st, a);
+}
+
 // variant 0: 4 waves x 32 query rows; 1: 8 waves x 16 rows; 2: 4 waves x 16 rows
 template <int HD, bool PRUNED, bool SHAREDQK, int HDK = HD>
 static void attn_launch_variant(int variant, bool plain, const AttnArgs &a, hipStream_t st) {
@@ -875,6 +961,7 @@ static void attn_launch_variant(int variant, bool plain, const AttnArgs &a, hipS
 }
 
 static int g_attn_variant = -1; // et_tuning_set("attn_variant"): -1 = automatic
+static int g_attn_packed = 1;   // et_tuning_set("attn_packed"): 0 = packed sequences run one workgroup per possible query block
 static int g_attn_vwin = 1;     // et_tuning_set("attn_vwin"): 0 = pruned attention always stages through registers
 
 static float head_scale(int hd) {
@@ -999,6 +1086,16 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
         attn_launch_variant<64, false, false, 32>(variant, plain, a, st);
         return launch_status(who);
     }
+    // packed sequences: the grid the chip holds, every workgroup walks its share of the query blocks that exist
+    if (a.cu_seqlens && !pruned && !sharedqk && variant == 2 && a.batch <= 64 * AT_PX && g_attn_packed) {
+        if (hd == 32)
+            attn_launch_packed<32>(a, st);
+        else if (hd == 64)
+            attn_launch_packed<64>(a, st);
+        else
+            attn_launch_packed<128>(a, st);
+        return launch_status(who);
+    }
     // dense Q/K with compact V (the reference's pruned wiring): DMA-staged value windows
     if (pruned && hd == 64 && !a.qk_head_ptr && a.v_head_ptr && a.ldq % 8 == 0 && a.ldv % 8 == 0 && a.ldv >= 8 &&
         g_attn_vwin) {
@@ -1023,6 +1120,7 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
 
 void set_attn_variant(int v) { g_attn_variant = v; }
 void set_attn_vwin(int v) { g_attn_vwin = v; }
+void set_attn_packed(int v) { g_attn_packed = v; }
 
 } // namespace et
 

@@ -43,6 +43,7 @@ namespace et {
 
 void set_attn_variant(int v);
 void set_attn_vwin(int v);
+void set_attn_packed(int v);
 void set_ln_rows(int v);
 
 constexpr int TL_THREADS = 512;
@@ -2076,6 +2077,10 @@ extern "C" int et_tuning_set(const char *key, int value) {
     }
     if (key && !strcmp(key, "ln_rows")) {
         et::set_ln_rows(value);
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "attn_packed")) {
+        et::set_attn_packed(value);
         return ET_OK;
     }
     if (key && !strcmp(key, "attn_vwin")) {

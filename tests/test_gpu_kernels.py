@@ -677,6 +677,40 @@ def test_otf_attention_varlen_equals_padded(K):
     check_close(packed, want[sel], max_abs=5e-3, mean_rel=1e-3, what="varlen attention")
 
 
+@pytest.mark.parametrize("S,H,d,lens", [
+    (256, 12, 768, [256, 31, 130, 64, 0, 200, 1]),                  # one sequence without rows
+    (128, 2, 128, [128, 5, 0, 0, 77, 64, 65, 128, 3, 90]),          # fewer heads than XCDs: sequences without a
+                                                                    # head on some XCD
+    (96, 4, 256, list(range(96, 96 - 70, -1))),                     # more than 64 sequences (two count registers)
+    (64, 2, 128, [64 - (i % 50) for i in range(300)]),              # more than the walked form takes: one
+                                                                    # workgroup per possible block
+])
+def test_otf_attention_varlen_walks_existing_blocks(K, S, H, d, lens):
+    """packed sequences: workgroups that walk the existing query blocks == one workgroup per possible block (the
+    same block code, bit for bit) == the oracle on the padded batch"""
+    from et_amd._lib import lib
+    r = rng(50 + S + H)
+    lens = np.array(lens, np.int32)
+    B = lens.size
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    Q, Kk, V = (randn_h(r, (T, d)) for _ in range(3))
+    mask = randn_h(r, (S, S), 0.5)
+    args = (dev(Q), dev(Kk), dev(V), dev(mask), dev(cu), S, H, 1.0)
+    walked = host(K.OTF_attention_varlen(*args))
+    try:
+        lib().et_tuning_set(b"attn_packed", 0)
+        grid = host(K.OTF_attention_varlen(*args))
+    finally:
+        lib().et_tuning_set(b"attn_packed", 1)
+    assert np.array_equal(walked, grid)
+    Qp, Kp, Vp = (np.zeros((B * S, d), np.float16) for _ in range(3))
+    sel = np.concatenate([np.arange(b * S, b * S + lens[b]) for b in range(B)]).astype(np.int64)
+    Qp[sel], Kp[sel], Vp[sel] = Q, Kk, V
+    want = orc.otf_attention(Qp, Kp, Vp, mask, S, H, B, lens, 1.0, f64=True)
+    check_close(walked, want[sel], max_abs=5e-3, mean_rel=1e-3, what="varlen attention, walked blocks")
+
+
 def test_prune_attention(K):
     r = rng(43)
     S, H, d, B = 160, 12, 768, 2
