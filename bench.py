@@ -38,10 +38,10 @@ D, H, DFF = 768, 12, 3072
 # sources it was measured on; when the sources have changed since, `traffic` is null rather than a stale figure.
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "encoder_layer_b16_s512_hbm_traffic.txt")
 KERNEL_SOURCES = ("tile_linear.hip", "attention.hip", "skip_layernorm.hip", "common.h")
-TRAFFIC_KERNELS = {  # bench line -> kernel name prefix in the profile summary
-    "tile_linear qkv (3 x 768->768, one launch)": "et::tile_linear_resident_kernel",
-    "attention (on-the-fly)": "et::attention_kernel",
-    "layer tail: o + skip + LayerNorm + feed-forward (gelu) + skip + LayerNorm, fused": "et::tile_ffn_fused_kernel",
+TRAFFIC_KERNELS = {  # bench line -> kernel instance in the profile summary (the default workload's launches)
+    "tile_linear qkv (3 x 768->768, one launch)": "et::tile_linear_resident_kernel<2, false, 12, false, 64>",
+    "attention (on-the-fly)": "et::attention_kernel<64, 2, 4, false, false, true, 64, false>",
+    "layer tail: o + skip + LayerNorm + feed-forward (gelu) + skip + LayerNorm, fused": "et::tile_ffn_fused_kernel<3, true>",
 }
 
 
@@ -55,7 +55,7 @@ def kernel_source_fingerprint():
 
 
 def measured_traffic_mib():
-    """{kernel prefix: fetch + write MiB per launch} from the profile summary, or {} when it is stale or absent"""
+    """{kernel instance: fetch + write MiB per launch} from the profile summary, or {} when it is stale or absent"""
     import re
     try:
         text = open(TRAFFIC_PROFILE).read()
@@ -68,7 +68,7 @@ def measured_traffic_mib():
     for line in text.splitlines():
         m = re.match(r"(\S.*?)\s+n=\s*\d+\s+fetch avg\s+([0-9.]+) MiB\s+write avg\s+([0-9.]+) MiB", line)
         if m:
-            out[m.group(1).split("<")[0]] = float(m.group(2)) + float(m.group(3))
+            out[m.group(1)] = float(m.group(2)) + float(m.group(3))
     return out
 
 
