@@ -845,7 +845,9 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
                 nb = __builtin_amdgcn_readlane(nbv[r], b & 63);
             }
         const int rem = i - first;
-        const int h = ((xcd - b * a.nhead) & 7) + 8 * (rem / nb);
+        const int h = ((xcd - b * a.nhead) & 7) + 8 * (rem / max(nb, 1));
+        if (nb <= 0 || rem < 0 || b >= a.batch || h >= a.nhead)
+            continue; // (cannot happen with consistent counts; never index past the operands)
         attention_block<HD, QS, NW, false, false, false, HD, false>(a, b, h, rem % nb);
         __syncthreads(); // the block's output staging in LDS is read before the next block's tiles land there
     }
