@@ -87,6 +87,7 @@ def test_argument_errors_return_codes_without_a_device():
     assert l.et_OTF_attention(p, p, p, p, None, 128, 96, 2, 1, None, 1.0, None) == -3   # head_dim 48 unsupported
     assert b"head_dim" in l.et_last_error()
     assert l.et_strerror(-3) == b"unsupported shape"
+    assert l.et_microbench(0, 1568, 16, None, None) == -1                               # no result pointers
     with pytest.raises(_lib.EtError):
         formats.gen_sparse_tile_mat(100, 64, 0.5, 1)     # nrow not a multiple of 16
     with pytest.raises(_lib.EtError):

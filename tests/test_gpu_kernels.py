@@ -906,3 +906,26 @@ def test_launchers_with_no_rows_touch_nothing_and_bad_arguments_fail_cleanly(K):
     assert (sentinel == 7).all()
     assert L.et_last_error().decode() != ""
 
+
+
+# ------------------------------------------------------------ machine rates
+def test_microbenchmarks_report_plausible_rates():
+    """et_microbench runs its three kernels and returns rates of the right order (not a performance assertion:
+    the bounds are a factor of several around what an MI355X measures)"""
+    import ctypes as C
+    from et_amd._lib import lib, check
+    sec, units = C.c_double(), C.c_double()
+    def rate(what, p0, p1):
+        check(lib().et_microbench(what, p0, p1, C.byref(sec), C.byref(units)))
+        assert sec.value > 0 and units.value > 0
+        return units.value / sec.value
+    mfma_per_s = rate(2, 0, 4)                  # MFMAs per second and wave: 16 clk each
+    clock = mfma_per_s * 16
+    assert 0.8e9 < clock < 3.0e9
+    lds = rate(0, 1568, 16) / clock             # bytes per clock and CU
+    assert 100 < lds < 300
+    assert rate(0, 1536, 16) / clock < 0.5 * lds    # a row stride of a multiple of 256 bytes conflicts
+    stream = rate(1, 0, 16) / clock
+    assert 20 < stream < 140
+    with pytest.raises(Exception):
+        check(lib().et_microbench(7, 0, 0, C.byref(sec), C.byref(units)))
