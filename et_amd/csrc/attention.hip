@@ -430,8 +430,32 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
         // requested one tile ahead (right after the previous tile consumed
         // its own) so the L2 latency is covered by a whole tile of work.
         f16x4 mk[QS][4];
+        // Whole mask rows of a tile are 128 bytes, one cache line.  Where rows are 16-byte aligned a full tile's
+        // values come as two 16-byte loads per lane that together read each of the 16 lines once (lane (row, g)
+        // takes keys 16g .. 16g+15); the score layout wants keys 16k + 4g .. +3 for k = 0..3, i.e. the 4 x 4
+        // transpose of the 8-byte pieces across the row's four lanes, done with row swaps when the values are
+        // consumed (mk_blocked says that it is still due).  Four 8-byte loads per lane, the direct form, touch
+        // every line four times from four requests: with twelve waves per CU the lines do not survive in L1
+        // between them, and a dense mask then costs more L2 traffic than K and V together.
+        const bool mask_vec16 = mask_vec && ((a.seq_len & 7) == 0) && ((reinterpret_cast<uintptr_t>(a.mask) & 15u) == 0);
+        bool mk_blocked = false;
         auto load_mask = [&](int kb, auto fast_c) {
             constexpr bool FAST = decltype(fast_c)::value;
+            mk_blocked = FAST && mask_vec16;
+            if (FAST && mask_vec16) {
+#pragma unroll
+                for (int qs = 0; qs < QS; qs++) {
+                    const int q = q0 + (wave * QS + qs) * 16 + c16;
+                    const f16 *mrow = a.mask + (size_t)q * a.seq_len + kb + g4 * 16;
+                    const f16x8 l0 = *reinterpret_cast<const f16x8 *>(mrow);
+                    const f16x8 l1 = *reinterpret_cast<const f16x8 *>(mrow + 8);
+                    mk[qs][0] = f16x4{l0[0], l0[1], l0[2], l0[3]};
+                    mk[qs][1] = f16x4{l0[4], l0[5], l0[6], l0[7]};
+                    mk[qs][2] = f16x4{l1[0], l1[1], l1[2], l1[3]};
+                    mk[qs][3] = f16x4{l1[4], l1[5], l1[6], l1[7]};
+                }
+                return;
+            }
 #pragma unroll
             for (int qs = 0; qs < QS; qs++) {
                 const int q = q0 + (wave * QS + qs) * 16 + c16;
@@ -543,6 +567,30 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
             // more than 8 binades (P then stays <= 256, exact enough in half),
             // so after the first tiles the accumulator rescale is skipped.
             f16x8 pf[QS][2];
+            if (MASKED && mk_blocked) { // 4 x 4 transpose of the pieces over the row's four lanes
+#pragma unroll
+                for (int qs = 0; qs < QS; qs++) {
+                    typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+                    u32x2 pc[4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        pc[j] = __builtin_bit_cast(u32x2, mk[qs][j]);
+#pragma unroll
+                    for (int d = 0; d < 2; d++) {
+                        auto s01 = __builtin_amdgcn_permlane16_swap(pc[0][d], pc[1][d], false, false);
+                        auto s23 = __builtin_amdgcn_permlane16_swap(pc[2][d], pc[3][d], false, false);
+                        auto t02 = __builtin_amdgcn_permlane32_swap(s01[0], s23[0], false, false);
+                        auto t13 = __builtin_amdgcn_permlane32_swap(s01[1], s23[1], false, false);
+                        pc[0][d] = t02[0];
+                        pc[2][d] = t02[1];
+                        pc[1][d] = t13[0];
+                        pc[3][d] = t13[1];
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        mk[qs][j] = __builtin_bit_cast(f16x4, pc[j]);
+                }
+            }
             if (MASKED) {
                 // (the multiplier is exactly 1.0 but opaque to the optimiser,
                 // which would otherwise turn the fused form back into a
