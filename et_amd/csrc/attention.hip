@@ -94,6 +94,30 @@ __device__ __forceinline__ float xor_max_16_32(float v) {
     return __builtin_bit_cast(float, z0);
 }
 
+// 4 x 4 transpose of 8-byte pieces over the four lanes l, l+16, l+32, l+48: on entry piece j of the lane in
+// row g (g = lane / 16) is element (g, j), on return it is element (j, g).  Two row-swap steps per dword.
+__device__ __forceinline__ void transpose_pieces_4x4(f16x4 (&p)[4]) {
+    typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+    u32x2 pc[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        pc[j] = __builtin_bit_cast(u32x2, p[j]);
+#pragma unroll
+    for (int d = 0; d < 2; d++) {
+        auto s01 = __builtin_amdgcn_permlane16_swap(pc[0][d], pc[1][d], false, false);
+        auto s23 = __builtin_amdgcn_permlane16_swap(pc[2][d], pc[3][d], false, false);
+        auto t02 = __builtin_amdgcn_permlane32_swap(s01[0], s23[0], false, false);
+        auto t13 = __builtin_amdgcn_permlane32_swap(s01[1], s23[1], false, false);
+        pc[0][d] = t02[0];
+        pc[2][d] = t02[1];
+        pc[1][d] = t13[0];
+        pc[3][d] = t13[1];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        p[j] = __builtin_bit_cast(f16x4, pc[j]);
+}
+
 // PLAIN: the launcher has established that there is no mask (or an all-zero
 // one), every sequence has full length and seq_len is a multiple of the
 // workgroup's query rows - no guards, no mask bookkeeping.
@@ -228,6 +252,7 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
                               ((reinterpret_cast<uintptr_t>(a.mask) & 7u) == 0);
         const bool qk_vec = SHAREDQK && ((a.seq_len & 3) == 0) &&
                             ((reinterpret_cast<uintptr_t>(a.QK) & 7u) == 0);
+        const bool qk_vec16 = qk_vec && ((a.seq_len & 7) == 0) && ((reinterpret_cast<uintptr_t>(a.QK) & 15u) == 0);
         const float ls = a.log2_scale;
 
         // ---- key/value tile staging: global -> registers -> LDS.  The
@@ -536,6 +561,21 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
                         for (int qs = 0; qs < QS; qs++) // (the first step reads -m as its C operand: no copies)
                             st[ksub][qs] = mfma16x16x32(kfr[ksub & 1][s], qf[qs][s], s == 0 ? nm4[qs] : st[ksub][qs]);
                 }
+            } else if (FAST && qk_vec16) {
+                // stored scores of a full tile: line-wise like the mask (128 bytes per query row and tile)
+#pragma unroll
+                for (int qs = 0; qs < QS; qs++) {
+                    const int q = q0 + (wave * QS + qs) * 16 + c16;
+                    const f16 *src = a.QK + ((size_t)bh * a.seq_len + q) * a.seq_len + kb + g4 * 16;
+                    const f16x8 l0 = *reinterpret_cast<const f16x8 *>(src);
+                    const f16x8 l1 = *reinterpret_cast<const f16x8 *>(src + 8);
+                    f16x4 pc[4] = {f16x4{l0[0], l0[1], l0[2], l0[3]}, f16x4{l0[4], l0[5], l0[6], l0[7]},
+                                   f16x4{l1[0], l1[1], l1[2], l1[3]}, f16x4{l1[4], l1[5], l1[6], l1[7]}};
+                    transpose_pieces_4x4(pc);
+#pragma unroll
+                    for (int ksub = 0; ksub < 4; ksub++)
+                        st[ksub][qs] = __builtin_convertvector(pc[ksub], f32x4) - m_ref[qs];
+                }
             } else {
 #pragma unroll
                 for (int qs = 0; qs < QS; qs++) {
@@ -567,29 +607,10 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
             // more than 8 binades (P then stays <= 256, exact enough in half),
             // so after the first tiles the accumulator rescale is skipped.
             f16x8 pf[QS][2];
-            if (MASKED && mk_blocked) { // 4 x 4 transpose of the pieces over the row's four lanes
+            if (MASKED && mk_blocked) { // the line-wise loads hold key blocks per lane: into the score layout
 #pragma unroll
-                for (int qs = 0; qs < QS; qs++) {
-                    typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-                    u32x2 pc[4];
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        pc[j] = __builtin_bit_cast(u32x2, mk[qs][j]);
-#pragma unroll
-                    for (int d = 0; d < 2; d++) {
-                        auto s01 = __builtin_amdgcn_permlane16_swap(pc[0][d], pc[1][d], false, false);
-                        auto s23 = __builtin_amdgcn_permlane16_swap(pc[2][d], pc[3][d], false, false);
-                        auto t02 = __builtin_amdgcn_permlane32_swap(s01[0], s23[0], false, false);
-                        auto t13 = __builtin_amdgcn_permlane32_swap(s01[1], s23[1], false, false);
-                        pc[0][d] = t02[0];
-                        pc[2][d] = t02[1];
-                        pc[1][d] = t13[0];
-                        pc[3][d] = t13[1];
-                    }
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        mk[qs][j] = __builtin_bit_cast(f16x4, pc[j]);
-                }
+                for (int qs = 0; qs < QS; qs++)
+                    transpose_pieces_4x4(mk[qs]);
             }
             if (MASKED) {
                 // (the multiplier is exactly 1.0 but opaque to the optimiser,
@@ -901,8 +922,12 @@ __global__ void __launch_bounds__(NW * 64, (QS == 1 && HD <= 64) ? 4 : 2) attent
     }
 }
 
-// scaled Q K^T written to memory, [(b*nhead+h)][q][k]; one wave per 16 queries
-// x 64 keys, transposed product so a lane owns 4 consecutive keys of one query.
+// scaled Q K^T written to memory, [(b*nhead+h)][q][k]; one wave per 64 queries x 64 keys (the K fragments are
+// fetched once and used for four tiles of 16 queries), transposed product so a lane owns 4 consecutive keys of
+// one query.  A query's 64 scores of the tile are 128 bytes, one cache line: the lane's four 8-byte pieces are
+// transposed over the query's four lanes so that every lane stores 32 contiguous bytes and the four of them the
+// whole line (element-wise 2-byte stores of the same values took 129 us for batch 16 x seq 512, six times the
+// time of writing 100 MB).
 template <int HD>
 __global__ void __launch_bounds__(256)
 qk_scores_kernel(f16 *__restrict__ QK, const f16 *__restrict__ Q, const f16 *__restrict__ K,
@@ -911,36 +936,60 @@ qk_scores_kernel(f16 *__restrict__ QK, const f16 *__restrict__ Q, const f16 *__r
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63, c16 = lane & 15, g4 = lane >> 4;
     const int bh = blockIdx.z, h = bh % nhead, b = bh / nhead;
-    const int q0 = blockIdx.y * 16;
+    const int qb0 = blockIdx.y * 64;
     const int k0 = (blockIdx.x * 4 + wave) * 64;
     if (k0 >= seq_len)
         return;
     const size_t row0 = (size_t)b * seq_len;
-    const int q = q0 + c16;
-    f16x8 qf[DK];
-#pragma unroll
-    for (int s = 0; s < DK; s++) {
-        qf[s] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        if (q < seq_len)
-            qf[s] = *reinterpret_cast<const f16x8 *>(Q + (row0 + q) * d_model + h * HD + s * 32 + g4 * 8);
-    }
+    f16x8 kf[4][DK];
 #pragma unroll
     for (int ksub = 0; ksub < 4; ksub++) {
         const int key = k0 + ksub * 16 + c16;
-        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < DK; s++) {
-            f16x8 kf = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            kf[ksub][s] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
             if (key < seq_len)
-                kf = *reinterpret_cast<const f16x8 *>(K + (row0 + key) * d_model + h * HD + s * 32 + g4 * 8);
-            acc = mfma16x16x32(kf, qf[s], acc);
+                kf[ksub][s] = *reinterpret_cast<const f16x8 *>(K + (row0 + key) * d_model + h * HD + s * 32 + g4 * 8);
         }
-        if (q < seq_len) {
-            f16 *dst = QK + ((size_t)bh * seq_len + q) * seq_len + k0 + ksub * 16 + g4 * 4;
+    }
+    // whole lines: all 64 keys exist and rows start on 16-byte boundaries (wave-uniform)
+    const bool lines = k0 + 64 <= seq_len && (seq_len & 7) == 0 && (reinterpret_cast<uintptr_t>(QK) & 15u) == 0;
+    for (int qt = 0; qt < 4; qt++) {
+        if (qb0 + qt * 16 >= seq_len)
+            break;
+        const int q = qb0 + qt * 16 + c16;
+        f16x8 qf[DK];
 #pragma unroll
-            for (int r = 0; r < 4; r++)
-                if (k0 + ksub * 16 + g4 * 4 + r < seq_len)
-                    dst[r] = (f16)(acc[r] * scale);
+        for (int s = 0; s < DK; s++) {
+            qf[s] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (q < seq_len)
+                qf[s] = *reinterpret_cast<const f16x8 *>(Q + (row0 + q) * d_model + h * HD + s * 32 + g4 * 8);
+        }
+        f16x4 pc[4]; // piece ksub: keys k0 + 16 ksub + 4 g4 .. + 3 of query q
+#pragma unroll
+        for (int ksub = 0; ksub < 4; ksub++) {
+            f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < DK; s++)
+                acc = mfma16x16x32(kf[ksub][s], qf[s], acc);
+            pc[ksub] = __builtin_convertvector(acc * scale, f16x4);
+        }
+        f16 *qrow = QK + ((size_t)bh * seq_len + q) * seq_len + k0;
+        if (lines) {
+            transpose_pieces_4x4(pc); // piece j: keys k0 + 16 g4 + 4 j .. + 3
+            if (q < seq_len) {
+                *reinterpret_cast<f16x8 *>(qrow + g4 * 16) =
+                    f16x8{pc[0][0], pc[0][1], pc[0][2], pc[0][3], pc[1][0], pc[1][1], pc[1][2], pc[1][3]};
+                *reinterpret_cast<f16x8 *>(qrow + g4 * 16 + 8) =
+                    f16x8{pc[2][0], pc[2][1], pc[2][2], pc[2][3], pc[3][0], pc[3][1], pc[3][2], pc[3][3]};
+            }
+        } else if (q < seq_len) {
+#pragma unroll
+            for (int ksub = 0; ksub < 4; ksub++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (k0 + ksub * 16 + g4 * 4 + r < seq_len)
+                        qrow[ksub * 16 + g4 * 4 + r] = pc[ksub][r];
         }
     }
 }
@@ -1369,7 +1418,7 @@ extern "C" int et_qk_scores(void *QK, const void *Q, const void *K, int seq_len,
                "et_qk_scores: Q/K must be 16-byte aligned");
     // scale = half(1/sqrt(head_dim)), encoder/encoder.cu:113
     const float scale = (float)(f16)(1.0f / sqrtf((float)hd));
-    const dim3 grid((seq_len + 255) / 256, (seq_len + 15) / 16, batch * nhead), block(256);
+    const dim3 grid((seq_len + 255) / 256, (seq_len + 63) / 64, batch * nhead), block(256);
     hipStream_t st = static_cast<hipStream_t>(stream);
     f16 *o = static_cast<f16 *>(QK);
     const f16 *q = static_cast<const f16 *>(Q), *k = static_cast<const f16 *>(K);
