@@ -637,6 +637,10 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
                         load_mask(kb + AT_KT, no_t{});
                 }
             }
+            // the lane's part of each row maximum (of s - m_ref); the row's other three
+            // parts only matter when some row of the wave has to raise its maximum
+            float pmx[QS];
+            bool live = false;
 #pragma unroll
             for (int qs = 0; qs < QS; qs++) {
                 if (!FAST) {
@@ -647,14 +651,25 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
                             if (kb + ksub * 16 + g4 * 4 + r >= len)
                                 st[ksub][qs][r] = -INFINITY;
                 }
-                // the lane's part of the row maximum (of s - m_ref); the row's other three
-                // parts only matter when some row of the wave has to raise its maximum
                 float mx = -INFINITY;
 #pragma unroll
                 for (int ksub = 0; ksub < 4; ksub++) {
                     mx = fmaxf(fmaxf(mx, st[ksub][qs][0]), st[ksub][qs][1]);
                     mx = fmaxf(fmaxf(mx, st[ksub][qs][2]), st[ksub][qs][3]);
                 }
+                pmx[qs] = mx;
+                // does this tile add anything to the row?  Not if every score is 160 binades or more under a
+                // maximum the row already has: every exp2 is then exactly zero in fp32 (so is P, and the sums
+                // and the output do not change).
+                live = live || m_run[qs] == -INFINITY || !(mx * ls < -160.0f);
+            }
+            // A tile that is dead for every row of the wave - the keys behind a padding mask - ends here: no
+            // exponentials, no second product (wave-uniform; same bits as going through with P = 0).
+            if (!PLAIN && __builtin_amdgcn_ballot_w64(live) == 0)
+                return;
+#pragma unroll
+            for (int qs = 0; qs < QS; qs++) {
+                float mx = pmx[qs];
                 // (a row without a maximum yet, m_run = -inf, takes its first finite one)
                 const bool up_lane = (m_run[qs] == -INFINITY) ? (mx > -INFINITY) : (mx * ls > 8.0f);
                 if (__builtin_amdgcn_ballot_w64(up_lane) != 0) {

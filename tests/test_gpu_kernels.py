@@ -711,6 +711,33 @@ def test_otf_attention_varlen_walks_existing_blocks(K, S, H, d, lens):
     check_close(walked, want[sel], max_abs=5e-3, mean_rel=1e-3, what="varlen attention, walked blocks")
 
 
+@pytest.mark.parametrize("S,keep,value", [(512, 300, -30000.0), (512, 64, -65504.0), (256, 200, -1000.0), (192, 1, -30000.0)])
+def test_otf_attention_padding_mask_with_dead_tiles(K, S, keep, value):
+    """a padding mask that blanks the keys from `keep` on: key tiles that lie wholly behind it add nothing (every
+    exp2 is exactly zero) and the kernel passes over them; == the oracle, with and without a mask summary, and the
+    blanked keys' V rows have no influence at all"""
+    r = rng(60 + S + keep)
+    H, d, B = 12, 768, 2
+    Q, Kk, V = (randn_h(r, (B * S, d)) for _ in range(3))
+    mask = np.zeros((S, S), np.float16)
+    mask[:, keep:] = value
+    want = orc.otf_attention(Q, Kk, V, mask, S, H, B, None, 1.0, f64=True)
+    md = dev(mask)
+    got = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), md, S, H, B, None, 1.0))
+    check_close(got, want, max_abs=5e-3, mean_rel=1e-3, what="attention, padding mask")
+    summ = K.attention_mask_summary(md, S)
+    K.attention_mask_summary_attach(md, S, summ)
+    try:
+        fast = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), md, S, H, B, None, 1.0))
+    finally:
+        K.attention_mask_summary_attach(md, S, None)
+    assert np.array_equal(got, fast)
+    if value <= -30000.0:
+        V2 = V.copy()
+        V2.reshape(B, S, d)[:, keep:] = randn_h(r, (B, S - keep, d), 7.0)
+        assert np.array_equal(host(K.OTF_attention(dev(Q), dev(Kk), dev(V2), md, S, H, B, None, 1.0)), got)
+
+
 def test_prune_attention(K):
     r = rng(43)
     S, H, d, B = 160, 12, 768, 2
