@@ -418,6 +418,14 @@ int et_device_synchronize(void);
  *   "ln_rows"         rows per wave of et_skip_layernorm (1, 2, 4)
  *   "attn_variant"    0: 4 waves x 32 query rows, 1: 8 waves x 16 rows,
  *                     2: 4 waves x 16 rows; -1 automatic
+ *   "attn_vwin"       0: et_Prune_attention always stages K and V through
+ *                     registers; 1 (default): dense Q/K with a compact V whose
+ *                     pitch is a multiple of 8 take the DMA-staged kernel
+ *   "attn_packed"     0: et_OTF_attention_varlen launches one workgroup per
+ *                     possible query block; 1 (default): workgroups walk the
+ *                     blocks that exist (up to 256 sequences)
+ *   "tile_tail_min_panels"  row panels below which the layer tail runs step
+ *                     by step when the caller gave it buffers (default 72)
  * Not thread-safe; results never depend on these beyond fp32 summation
  * order. */
 int et_tuning_set(const char *key, int value);
