@@ -415,6 +415,19 @@ def second_targets(torch, K, dev, enc, out, x, B, S, mask_h, lins, ln):
     wsp = torch.empty(Encoder_tile.buffer_size(D, S, H, B) // 2, dtype=torch.float16, device=dev)
     encp = Encoder_tile(D, S, H, wsp, *Lp, *ln, pm, B)
     res["latency_us_padding_mask"] = round(event_time(torch, lambda: encp.run(out, x), reps=50), 1)
+    # the headline layer replayed from a HIP graph of twenty runs (Encoder_tile::run only launches kernels, so a
+    # caller can capture it: a 12-layer model is such a graph); replays repeated with eager work in between
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        enc.run(out, x)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for _ in range(20):
+            enc.run(out, x)
+    res["latency_us_hip_graph_of_20"] = round(event_time(torch, graph.replay, reps=10, warm=2) / 20, 1)
     return res
 
 
