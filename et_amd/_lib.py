@@ -44,6 +44,10 @@ PROTOTYPES = {
     "et_tile_plan_ffn_fusable": (_i, [_vp, _vp]),
     "et_tile_plan_run_tail": (_i, [_vp] * 12 + [_i, _vp]),
     "et_tile_plan_tail_fusable": (_i, [_vp, _vp, _vp]),
+    "et_tile_plan_run_tail_ws": (_i, [_vp] * 12 + [_i, _vp, _sz, _vp]),
+    "et_tile_plan_tail_prepare": (_i, [_vp, _vp, _vp]),
+    "et_tile_plan_tail_ws_bytes": (_sz, [_vp, _vp, _vp, _i]),
+    "et_tail_ws_bytes_for": (_sz, [_i, _i]),
     "et_tile_plan_run_multi": (_i, [C.POINTER(_vp), C.POINTER(_vp), _i, _vp, _i, _vp]),
     "et_tile_plan_query": (_i, [_vp, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
     "et_prune_tile_mat": (_i, [_vp, _i, _i, _f, _ip, _ip]),
@@ -76,6 +80,9 @@ PROTOTYPES = {
     "et_linear_tile_ffn_fusable": (_i, [_vp, _vp]),
     "et_linear_tile_run_rows_tail": (_i, [_vp] * 12 + [_i, _vp]),
     "et_linear_tile_tail_fusable": (_i, [_vp, _vp, _vp]),
+    "et_linear_tile_run_rows_tail_ws": (_i, [_vp] * 12 + [_i, _vp, _sz, _vp]),
+    "et_linear_tile_tail_prepare": (_i, [_vp, _vp, _vp]),
+    "et_linear_tile_tail_ws_bytes": (_sz, [_vp, _vp, _vp, _i]),
     "et_linear_tile_run_multi": (_i, [C.POINTER(_vp), C.POINTER(_vp), _i, _vp, _i, _vp]),
     "et_linear_row_create": (_i, [C.POINTER(_vp), _i, _i, _i, _vp, _ip, _i, _vp, _i]),
     "et_linear_row_set_gelu": (_i, [_vp, _i]),

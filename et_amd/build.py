@@ -9,7 +9,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libet_amd.so")
 
-SOURCES = ["runtime.hip", "formats.cpp", "skip_layernorm.hip", "tile_linear.hip", "dense_gemm.hip", "attention.hip", "microbench.hip",
+SOURCES = ["runtime.hip", "formats.cpp", "skip_layernorm.hip", "tile_linear.hip", "tile_tail.hip", "dense_gemm.hip", "attention.hip", "microbench.hip",
            "encoder_capi.cpp"]
 
 # packed fp32 ops stay off: some of their forms have produced wrong results on

@@ -203,8 +203,14 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
     // value window: vskip columns of a neighbouring head in front of the head's own nv
     int vskip = 0;
     if (VWIN) {
-        vskip = vc0 & 7;
-        vc0 -= vskip;
+        // The window starts at the head's first column rounded down to 8, and never
+        // beyond ldv - 8: a head that keeps no columns and sits at the very end
+        // (v_head_ptr[h] == ldv) would otherwise start its window behind the row,
+        // and the clamp of the staging offsets below (ldv - 8 - vc0) would go
+        // negative.  The launcher guarantees ldv >= 8.
+        const int w0 = min(vc0 & ~7, a.ldv - 8);
+        vskip = vc0 - w0;
+        vc0 = w0;
         nv += vskip; // columns of the window up to the head's last one
     }
 

@@ -120,6 +120,36 @@ int et_linear_tile_run_rows_tail(const et_linear_tile *out_proj, const et_linear
                                    stream);
     });
 }
+int et_linear_tile_run_rows_tail_ws(const et_linear_tile *out_proj, const et_linear_tile *first,
+                                    const et_linear_tile *second, void *out, const void *attn, const void *input,
+                                    void *mid, void *hidden, const void *gamma1, const void *beta1,
+                                    const void *gamma2, const void *beta2, int rows, void *ws, size_t ws_bytes,
+                                    void *stream) {
+    if (!out_proj || !first || !second) {
+        et::set_error("et_linear_tile_run_rows_tail_ws: null handle");
+        return ET_ERR_INVALID_ARG;
+    }
+    return guarded([&] {
+        Linear_tile::run_rows_tail(out_proj->impl, first->impl, second->impl, H(out), H(attn),
+                                   static_cast<const half *>(input), H(mid), H(hidden),
+                                   static_cast<const half *>(gamma1), static_cast<const half *>(beta1),
+                                   static_cast<const half *>(gamma2), static_cast<const half *>(beta2), rows,
+                                   stream, ws, ws_bytes);
+    });
+}
+int et_linear_tile_tail_prepare(const et_linear_tile *out_proj, const et_linear_tile *first,
+                                const et_linear_tile *second) {
+    if (!out_proj || !first || !second) {
+        et::set_error("et_linear_tile_tail_prepare: null handle");
+        return ET_ERR_INVALID_ARG;
+    }
+    return guarded([&] { Linear_tile::tail_prepare(out_proj->impl, first->impl, second->impl); });
+}
+size_t et_linear_tile_tail_ws_bytes(const et_linear_tile *out_proj, const et_linear_tile *first,
+                                    const et_linear_tile *second, int rows) {
+    return out_proj && first && second ? Linear_tile::tail_ws_bytes(out_proj->impl, first->impl, second->impl, rows)
+                                       : 0;
+}
 int et_linear_tile_tail_fusable(const et_linear_tile *out_proj, const et_linear_tile *first,
                                 const et_linear_tile *second) {
     return out_proj && first && second && Linear_tile::tail_fusable(out_proj->impl, first->impl, second->impl)

@@ -1,6 +1,6 @@
 // Error reporting, device-memory plumbing and the small data-movement kernels
 // of the sequence-length-aware path.
-#include "common.h"
+#include "tile_plan.h"
 
 #include <algorithm>
 #include <cstdarg>
@@ -20,6 +20,46 @@ void set_error(const char *fmt, ...) {
 int hip_fail(hipError_t e, const char *what) {
     set_error("%s: %s", what, hipGetErrorString(e));
     return ET_ERR_HIP;
+}
+
+// The wait-status word: pinned host memory that the device sees, allocated
+// once per process (by the first plan that is created, never inside a run).
+static int *g_status_host = nullptr, *g_status_dev = nullptr;
+static bool g_status_tried = false;
+static void status_init() {
+    if (g_status_tried)
+        return;
+    g_status_tried = true;
+    void *h = nullptr, *d = nullptr;
+    if (hipHostMalloc(&h, 64, hipHostMallocMapped) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    memset(h, 0, 64);
+    if (hipHostGetDevicePointer(&d, h, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipHostFree(h);
+        return;
+    }
+    g_status_host = static_cast<int *>(h);
+    g_status_dev = static_cast<int *>(d);
+}
+int *wait_status_device() {
+    status_init();
+    return g_status_dev;
+}
+volatile int *wait_status_host() {
+    status_init();
+    return g_status_host;
+}
+int check_wait_status(const char *who) {
+    volatile int *h = wait_status_host();
+    if (h && *h != 0) {
+        *h = 0;
+        set_error("%s: an earlier launch gave up a bounded wait inside a workgroup; its result was wrong", who);
+        return ET_ERR_HIP;
+    }
+    return ET_OK;
 }
 
 // one workgroup per (sequence, position), 16-byte copies

@@ -30,7 +30,7 @@
 // chunks + LayerNorm, double-buffered panels with a fetching wave),
 // tile_ffn_fused_kernel (feed-forward block / whole layer tail in one launch,
 // hidden activations in LDS), tile_linear_generic_kernel (raw and dense input).
-#include "common.h"
+#include "tile_plan.h"
 
 #include <algorithm>
 #include <type_traits>
@@ -45,6 +45,9 @@ void set_attn_variant(int v);
 void set_attn_vwin(int v);
 void set_attn_packed(int v);
 void set_ln_rows(int v);
+void set_tail_pair(int v);
+void set_tail_spin(int v);
+int tail_spin();
 
 constexpr int TL_THREADS = 512;
 constexpr int TL_WAVES = 8;
@@ -2029,6 +2032,8 @@ static int raw_tile_linear(void *Y, const void *X, const int *row_ptr, const int
 
 } // namespace et
 
+static int g_tail_pair_min_wgs = 0; // et_tuning_set("tile_tail_pair_min_wgs"): 0 = three quarters of the CUs
+
 extern "C" int et_tuning_set(const char *key, int value) {
     if (key && !strcmp(key, "tile_splitk_k1")) {
         et::g_tile_splitk_k1 = value;
@@ -2052,6 +2057,18 @@ extern "C" int et_tuning_set(const char *key, int value) {
     }
     if (key && !strcmp(key, "tile_bm64")) {
         et::g_tile_bm64 = value;
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "tile_tail_pair_min_wgs")) {
+        g_tail_pair_min_wgs = value;
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "tile_tail_pair")) {
+        et::set_tail_pair(value);
+        return ET_OK;
+    }
+    if (key && !strcmp(key, "tile_wait_spin")) {
+        et::set_tail_spin(value);
         return ET_OK;
     }
     if (key && !strcmp(key, "tile_fuse_ffn")) {
@@ -2187,14 +2204,6 @@ extern "C" int et_row_spmm_add_bias_gelu(void *out, const void *in, const void *
 // ---------------------------------------------------------------------------
 // plans
 // ---------------------------------------------------------------------------
-struct et_tile_plan {
-    int in_feat, out_feat, ntile, KC, nchunk;
-    et::f16 *d_data;
-    int *d_cptr;
-    int *d_row_offset;
-    et::f16 *d_bias;
-};
-
 extern "C" int et_tile_plan_create(et_tile_plan **plan, int in_feat, int out_feat, int ntile,
                                    const void *data, const int *row_ptr,
                                    const int *row_offset, const void *bias) {
@@ -2251,7 +2260,18 @@ extern "C" int et_tile_plan_create(et_tile_plan **plan, int in_feat, int out_fea
     }
 
     et_tile_plan *p = new et_tile_plan();
-    memset(p, 0, sizeof(*p));
+    {
+        static unsigned long long next_uid = 0;
+        p->uid = ++next_uid;
+    }
+    // column-sorted host copy (the layer-tail program is built from it)
+    p->h_row_ptr.assign(row_ptr, row_ptr + nbr + 1);
+    p->h_col.resize(ntile);
+    p->h_data.resize((size_t)ntile * 256);
+    for (int i = 0; i < ntile; i++) {
+        p->h_col[i] = row_offset[order[i]];
+        memcpy(&p->h_data[(size_t)i * 256], src + (size_t)order[i] * 256, 512);
+    }
     p->in_feat = in_feat;
     p->out_feat = out_feat;
     p->ntile = ntile;
@@ -2284,6 +2304,7 @@ extern "C" void et_tile_plan_destroy(et_tile_plan *p) {
     et_free(p->d_cptr);
     et_free(p->d_row_offset);
     et_free(p->d_bias);
+    et::tail_program_destroy(p->tail);
     delete p;
 }
 
@@ -2537,3 +2558,52 @@ extern "C" int et_tile_plan_run(const et_tile_plan *plan, void *Y, const void *X
                        plan->nchunk, gelu != 0, TL_PLAN, static_cast<hipStream_t>(stream));
 }
 
+// ---------------------------------------------------------------------------
+// layer tail with caller-provided scratch: pairs of workgroups over 64-row
+// panels (tile_tail.hip) where that applies and pays
+// ---------------------------------------------------------------------------
+extern "C" size_t et_tile_plan_tail_ws_bytes(const et_tile_plan *pO, const et_tile_plan *p1,
+                                             const et_tile_plan *p2, int M) {
+    return et::tail_pair_ws_bytes(pO, p1, p2, M);
+}
+
+extern "C" size_t et_tail_ws_bytes_for(int d_model, int rows) { return et::tail_ws_bytes_for(d_model, rows); }
+
+extern "C" int et_tile_plan_tail_prepare(const et_tile_plan *pO, const et_tile_plan *p1,
+                                         const et_tile_plan *p2) {
+    using namespace et;
+    ET_REQUIRE(pO && p1 && p2, ET_ERR_INVALID_ARG, "et_tile_plan_tail_prepare: null plan");
+    (void)wait_status_device(); // (allocated here rather than inside a run)
+    if (!tail_pair_applies(pO, p1, p2))
+        return ET_OK; // nothing to prepare: et_tile_plan_run_tail_ws will run the other kernels
+    return tail_pair_prepare(pO, p1, const_cast<et_tile_plan *>(p2));
+}
+
+extern "C" int et_tile_plan_run_tail_ws(const et_tile_plan *pO, const et_tile_plan *p1,
+                                        const et_tile_plan *p2, void *Y, const void *attn, const void *input,
+                                        void *mid, void *hidden, const void *gamma1, const void *beta1,
+                                        const void *gamma2, const void *beta2, int M, void *ws, size_t ws_bytes,
+                                        void *stream) {
+    using namespace et;
+    ET_REQUIRE(pO && p1 && p2 && Y && attn && input && gamma1 && beta1 && gamma2 && beta2,
+               ET_ERR_INVALID_ARG, "et_tile_plan_run_tail_ws: null pointer");
+    if (ws && M > 0 && tail_pair_applies(pO, p1, p2)) {
+        const size_t need = tail_pair_ws_bytes(pO, p1, p2, M);
+        const int cus = std::max(et_device_cu_count(), 1);
+        const int wgs = 2 * ((M + 63) / 64);
+        const int min_wgs = g_tail_pair_min_wgs > 0 ? g_tail_pair_min_wgs : (3 * cus) / 4;
+        if (ws_bytes >= need && (wgs >= min_wgs || !mid || tail_pair_forced())) {
+            ET_REQUIRE(aligned16(Y) && aligned16(attn) && aligned16(input) && aligned16(gamma1) &&
+                           aligned16(beta1) && aligned16(gamma2) && aligned16(beta2) && aligned16(ws),
+                       ET_ERR_ALIGNMENT, "et_tile_plan_run_tail_ws: pointers must be 16-byte aligned");
+            const int rc = tail_pair_prepare(pO, p1, const_cast<et_tile_plan *>(p2)); // (returns at once when prepared)
+            if (rc != ET_OK)
+                return rc;
+            return tail_pair_launch(pO, p1, p2, static_cast<f16 *>(Y), static_cast<const f16 *>(attn),
+                                    static_cast<const f16 *>(input), static_cast<const f16 *>(gamma1),
+                                    static_cast<const f16 *>(beta1), static_cast<const f16 *>(gamma2),
+                                    static_cast<const f16 *>(beta2), M, ws, static_cast<hipStream_t>(stream));
+        }
+    }
+    return et_tile_plan_run_tail(pO, p1, p2, Y, attn, input, mid, hidden, gamma1, beta1, gamma2, beta2, M, stream);
+}

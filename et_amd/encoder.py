@@ -107,23 +107,40 @@ class Linear_tile:
 
     @staticmethod
     def run_tail(out_proj, first, second, attn, inp, gamma1, beta1, gamma2, beta2, out=None, mid=None,
-                 hidden=None, rows=None):
+                 hidden=None, rows=None, ws=None):
         """Steps 6-10 of a layer in one launch: out projection + skip + LayerNorm, feed-forward block + skip +
-        LayerNorm.  `mid` / `hidden` are only used where the fused kernel does not apply; mid=None insists on it."""
+        LayerNorm.  `mid` / `hidden` are only used where the fused kernel does not apply; mid=None insists on it.
+        `ws` (a uint8 device tensor of at least tail_ws_bytes(...) bytes that overlaps no operand) lets the launch
+        take the form of pairs of workgroups over 64-row panels."""
         rows = attn.shape[0] if rows is None else rows
         out = out if out is not None else torch.empty((attn.shape[0], second.out_feat), dtype=torch.float16, device=attn.device)
         what = "Linear_tile.run_tail"
         opt = lambda t, cols, name: _dp2(t, rows, cols, what + name) if t is not None else None
-        check(lib().et_linear_tile_run_rows_tail(out_proj._h, first._h, second._h,
-                                                 _dp2(out, rows, second.out_feat, what + " out"),
-                                                 _dp2(attn, rows, out_proj.in_feat, what + " attn"),
-                                                 _dp2(inp, rows, out_proj.out_feat, what + " inp"),
-                                                 opt(mid, out_proj.out_feat, " mid"), opt(hidden, first.out_feat, " hidden"),
-                                                 _dpn(gamma1, out_proj.out_feat, what + " gamma1"),
-                                                 _dpn(beta1, out_proj.out_feat, what + " beta1"),
-                                                 _dpn(gamma2, second.out_feat, what + " gamma2"),
-                                                 _dpn(beta2, second.out_feat, what + " beta2"), rows, _stream()))
+        ws_ptr, ws_bytes = None, 0
+        if ws is not None:
+            if ws.dtype != torch.uint8 or not ws.is_cuda or not ws.is_contiguous():
+                raise ValueError(what + " ws: a contiguous uint8 device tensor is required")
+            ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
+        check(lib().et_linear_tile_run_rows_tail_ws(out_proj._h, first._h, second._h,
+                                                    _dp2(out, rows, second.out_feat, what + " out"),
+                                                    _dp2(attn, rows, out_proj.in_feat, what + " attn"),
+                                                    _dp2(inp, rows, out_proj.out_feat, what + " inp"),
+                                                    opt(mid, out_proj.out_feat, " mid"), opt(hidden, first.out_feat, " hidden"),
+                                                    _dpn(gamma1, out_proj.out_feat, what + " gamma1"),
+                                                    _dpn(beta1, out_proj.out_feat, what + " beta1"),
+                                                    _dpn(gamma2, second.out_feat, what + " gamma2"),
+                                                    _dpn(beta2, second.out_feat, what + " beta2"), rows,
+                                                    ws_ptr, ws_bytes, _stream()))
         return out
+
+    @staticmethod
+    def tail_ws_bytes(out_proj, first, second, rows):
+        """bytes of scratch the paired form of run_tail needs for `rows` rows (0 where it does not apply)"""
+        return int(lib().et_linear_tile_tail_ws_bytes(out_proj._h, first._h, second._h, rows))
+
+    @staticmethod
+    def tail_prepare(out_proj, first, second):
+        check(lib().et_linear_tile_tail_prepare(out_proj._h, first._h, second._h))
 
     @staticmethod
     def tail_fusable(out_proj, first, second):

@@ -72,11 +72,21 @@ class Linear_tile {
     static void run_rows_tail(const Linear_tile &out_proj, const Linear_tile &first, const Linear_tile &second,
                               half *out, half *attn, const half *input, half *mid, half *hidden,
                               const half *gamma1, const half *beta1, const half *gamma2, const half *beta2,
-                              int rows, void *stream) {
+                              int rows, void *stream, void *ws = nullptr, size_t ws_bytes = 0) {
         etRequire(!out_proj.is_gelu && first.is_gelu && !second.is_gelu,
                   "Linear_tile::run_rows_tail: only the first feed-forward linear is the GELU variant");
-        etChk(et_tile_plan_run_tail(out_proj.plan, first.plan, second.plan, out, attn, input, mid, hidden,
-                                    gamma1, beta1, gamma2, beta2, rows, stream));
+        // with scratch (`ws`, tail_ws_bytes()) the launch may take the form of pairs of
+        // workgroups over 64-row panels; see et_tile_plan_run_tail_ws
+        etChk(et_tile_plan_run_tail_ws(out_proj.plan, first.plan, second.plan, out, attn, input, mid, hidden,
+                                       gamma1, beta1, gamma2, beta2, rows, ws, ws_bytes, stream));
+    }
+    // builds what run_rows_tail with scratch needs (device allocations: not inside a run)
+    static void tail_prepare(const Linear_tile &out_proj, const Linear_tile &first, const Linear_tile &second) {
+        etChk(et_tile_plan_tail_prepare(out_proj.plan, first.plan, second.plan));
+    }
+    static size_t tail_ws_bytes(const Linear_tile &out_proj, const Linear_tile &first, const Linear_tile &second,
+                                int rows) {
+        return et_tile_plan_tail_ws_bytes(out_proj.plan, first.plan, second.plan, rows);
     }
     static bool tail_fusable(const Linear_tile &out_proj, const Linear_tile &first, const Linear_tile &second) {
         return et_tile_plan_tail_fusable(out_proj.plan, first.plan, second.plan) != 0;

@@ -36,8 +36,20 @@ class Encoder_base {
     Weight<int> d_cu;    // row offsets of the packed sequences
     Weight<int> d_order; // packed position -> batch index
     int total_rows; // sum of lengths when set, else batch*seq_len
+    // scratch of the layer tail's paired form (et_tile_plan_run_tail_ws), behind the
+    // activation units (and behind the score buffer of Encoder_length)
+    void *tail_ws;
+    size_t tail_ws_bytes;
 
     int rows() const { return batch * seq_len; }
+    static size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+    static size_t units_bytes(int d_model_, int seq_len_, int batch_) {
+        return (size_t)buffer_num * d_model_ * seq_len_ * batch_ * sizeof(half);
+    }
+    void place_tail_ws(size_t byte_offset) {
+        tail_ws = reinterpret_cast<char *>(buffer) + align256(byte_offset);
+        tail_ws_bytes = et_tail_ws_bytes_for(d_model, batch * seq_len);
+    }
 
   public:
     // ln_* and mask_ are HOST pointers (d_model halves; seq_len*seq_len halves).
@@ -48,7 +60,7 @@ class Encoder_base {
           ln_gamma{Weight<half>(ln_gamma_1, d_model_), Weight<half>(ln_gamma_2, d_model_)},
           ln_beta{Weight<half>(ln_beta_1, d_model_), Weight<half>(ln_beta_2, d_model_)},
           has_mask(mask_ != nullptr), mask_summary(nullptr), stream(nullptr), log2_scale(1.0f),
-          total_rows(batch_ * seq_len_) {
+          total_rows(batch_ * seq_len_), tail_ws(nullptr), tail_ws_bytes(0) {
         if (mask_) {
             mask = Weight<half>(mask_, seq_len_ * seq_len_);
             // the mask never changes after construction: let the attention
@@ -60,6 +72,7 @@ class Encoder_base {
         }
         for (int i = 0; i < buffer_num; i++)
             buffers[i] = buffer + (size_t)i * batch * seq_len * d_model;
+        place_tail_ws(units_bytes(d_model, seq_len, batch));
     }
     virtual ~Encoder_base() {
         if (mask_summary) {
@@ -70,8 +83,10 @@ class Encoder_base {
     Encoder_base(const Encoder_base &) = delete;
     Encoder_base &operator=(const Encoder_base &) = delete;
     virtual void run(half *out, half *in) = 0; // device pointers; out may alias in
+    // the reference's five activation units (encoder/encoder.h:51-53) plus the
+    // layer tail's scratch
     static size_t buffer_size(int d_model_, int seq_len_, int /*nheads_*/, int batch_ = 1) {
-        return (size_t)buffer_num * d_model_ * seq_len_ * batch_ * sizeof(half);
+        return align256(units_bytes(d_model_, seq_len_, batch_)) + et_tail_ws_bytes_for(d_model_, batch_ * seq_len_);
     }
 
     void set_stream(void *s) { stream = s; }
@@ -120,7 +135,8 @@ class Encoder_base {
         // and units 1..4 for the hidden activations are only touched where the
         // fused kernel does not apply)
         Linear_tile::run_rows_tail(O, M1, M2, out, attn, in, buffers[0], buffers[1], ln_gamma[0].get(),
-                                   ln_beta[0].get(), ln_gamma[1].get(), ln_beta[1].get(), nrows, stream);
+                                   ln_beta[0].get(), ln_gamma[1].get(), ln_beta[1].get(), nrows, stream, tail_ws,
+                                   tail_ws_bytes);
     }
 };
 
@@ -142,6 +158,7 @@ class Encoder_tile : public Encoder_base {
           MLP1_linear(std::move(MLP1_linear_)), MLP2_linear(std::move(MLP2_linear_)) {
         // the reference asserts this (encoder/encoder.cu:17)
         etRequire(MLP1_linear.is_gelu, "Encoder_tile: MLP1_linear must be the GELU variant");
+        Linear_tile::tail_prepare(O_linear, MLP1_linear, MLP2_linear);
     }
     void run(half *out, half *in) override {
         const Linear_tile *qkv[3] = {&Q_linear, &K_linear, &V_linear};
@@ -173,6 +190,7 @@ class Encoder_prune : public Encoder_base {
           V_linear(std::move(V_linear_)), O_linear(std::move(O_linear_)),
           MLP1_linear(std::move(MLP1_linear_)), MLP2_linear(std::move(MLP2_linear_)) {
         etRequire(MLP1_linear.is_gelu, "Encoder_prune: MLP1_linear must be the GELU variant");
+        Linear_tile::tail_prepare(O_linear, MLP1_linear, MLP2_linear);
     }
     void run(half *out, half *in) override {
         if (V_linear.plan && V_linear.in_feat == Q_linear.in_features() &&
@@ -289,10 +307,16 @@ class Encoder_length : public Encoder_base {
         // d_model*nheads*buffer_num, which lands inside them)
         QK_buf = buffer + (size_t)buffer_num * d_model * seq_len * batch;
         etRequire(MLP1_linear.is_gelu, "Encoder_length: MLP1_linear must be the GELU variant");
+        place_tail_ws(units_and_scores_bytes(d_model, seq_len, nheads, batch));
+        Linear_tile::tail_prepare(O_linear, MLP1_linear, MLP2_linear);
     }
-    static size_t buffer_size(int d_model_, int seq_len_, int nheads_, int batch_ = 1) {
+    static size_t units_and_scores_bytes(int d_model_, int seq_len_, int nheads_, int batch_) {
         return ((size_t)buffer_num * d_model_ * seq_len_ + (size_t)nheads_ * seq_len_ * seq_len_) *
                batch_ * sizeof(half);
+    }
+    static size_t buffer_size(int d_model_, int seq_len_, int nheads_, int batch_ = 1) {
+        return align256(units_and_scores_bytes(d_model_, seq_len_, nheads_, batch_)) +
+               et_tail_ws_bytes_for(d_model_, batch_ * seq_len_);
     }
 
     // One layer on packed rows: in_p/out_p are [valid_rows() x d_model] with
@@ -329,7 +353,7 @@ class Encoder_length : public Encoder_base {
                 // input are no longer needed by then.)
                 Linear_tile::run_rows_tail(O_linear, MLP1_linear, MLP2_linear, buffers[0], buffers[3], in_p,
                                            buffers[0], buffers[1], ln_gamma[0].get(), ln_beta[0].get(),
-                                           ln_gamma[1].get(), ln_beta[1].get(), n, stream);
+                                           ln_gamma[1].get(), ln_beta[1].get(), n, stream, tail_ws, tail_ws_bytes);
                 etChk(et_unpack_rows_ordered(out, buffers[0], d_cu.get(), d_order.get(), batch, seq_len, d_model, stream));
                 return;
             }

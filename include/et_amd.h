@@ -260,6 +260,34 @@ int et_tile_plan_run_tail(const et_tile_plan *out, const et_tile_plan *first,
                           const void *beta2, int M, void *stream);
 int et_tile_plan_tail_fusable(const et_tile_plan *out, const et_tile_plan *first,
                               const et_tile_plan *second);
+/* The same five steps with device scratch from the caller, which opens a second
+ * form of the launch: PAIRS of workgroups over 64-row panels.  Both workgroups
+ * of a pair run the projection and the first LayerNorm on the panel, each takes
+ * one half of the hidden columns of the feed-forward block, and their fp32
+ * partial sums meet in `ws` (whoever arrives second at a row-half's counter
+ * finishes it: no workgroup waits for another).  A CU then streams half the
+ * weights per row.  Taken where it applies (model width 256, 512 or 768, hidden
+ * width a multiple of 16 and at least 384), ws_bytes >=
+ * et_tile_plan_tail_ws_bytes(out, first, second, M) and there are enough row
+ * panels to fill the device; otherwise this is et_tile_plan_run_tail.  ws must
+ * not overlap any operand; its contents are scratch.  The per-plan program is
+ * built by et_tile_plan_tail_prepare (device allocations; called implicitly by
+ * the first run, so call it beforehand where a run must not allocate).  The
+ * `second` plan carries the program and the per-panel counters: runs that
+ * share it must not overlap in time.  Results differ from et_tile_plan_run_tail
+ * in fp32 summation order only. */
+int et_tile_plan_run_tail_ws(const et_tile_plan *out, const et_tile_plan *first,
+                             const et_tile_plan *second, void *Y, const void *attn,
+                             const void *input, void *mid, void *hidden, const void *gamma1,
+                             const void *beta1, const void *gamma2, const void *beta2, int M,
+                             void *ws, size_t ws_bytes, void *stream);
+int et_tile_plan_tail_prepare(const et_tile_plan *out, const et_tile_plan *first,
+                              const et_tile_plan *second);
+/* bytes of scratch the paired form needs for M rows (0 where it does not apply) */
+size_t et_tile_plan_tail_ws_bytes(const et_tile_plan *out, const et_tile_plan *first,
+                                  const et_tile_plan *second, int M);
+/* the same figure from the shapes alone (what an encoder adds to its workspace) */
+size_t et_tail_ws_bytes_for(int d_model, int rows);
 /* n (<= 4) planned linears with the same in_feat applied to the same X in ONE
  * launch (the Q/K/V projections, encoder/encoder.cu:22-26, which the
  * reference spreads over three streams). */
@@ -424,6 +452,15 @@ int et_device_synchronize(void);
  *   "attn_packed"     0: et_OTF_attention_varlen launches one workgroup per
  *                     possible query block; 1 (default): workgroups walk the
  *                     blocks that exist (up to 256 sequences)
+ *   "tile_tail_pair"  0: et_tile_plan_run_tail_ws never takes the paired form;
+ *                     1 (default): where it applies and pays; 2: wherever it applies
+ *   "tile_tail_pair_min_wgs" fewest workgroups (two per 64-row panel) for the
+ *                     paired form (default: three quarters of the CUs)
+ *   "tile_wait_spin"  polls after which a bounded wait inside a workgroup gives
+ *                     up (default 2^22; negative restores it).  A wave that gives
+ *                     up sets a status word, the launch's result is wrong, and
+ *                     the next launch of that kind returns ET_ERR_HIP once.  0
+ *                     makes every wait give up at once (for testing the report)
  *   "tile_tail_min_panels"  row panels below which the layer tail runs step
  *                     by step when the caller gave it buffers (default 72)
  * Not thread-safe; results never depend on these beyond fp32 summation

@@ -52,6 +52,19 @@ int et_linear_tile_run_rows_tail(const et_linear_tile *out_proj, const et_linear
                                  const et_linear_tile *second, void *out, const void *attn, const void *input,
                                  void *mid, void *hidden, const void *gamma1, const void *beta1,
                                  const void *gamma2, const void *beta2, int rows, void *stream);
+/* the same with device scratch `ws` (et_linear_tile_tail_ws_bytes for these rows),
+ * which lets the launch take the form of pairs of workgroups over 64-row panels
+ * (et_tile_plan_run_tail_ws); et_linear_tile_tail_prepare builds what that form
+ * needs ahead of the first run */
+int et_linear_tile_run_rows_tail_ws(const et_linear_tile *out_proj, const et_linear_tile *first,
+                                    const et_linear_tile *second, void *out, const void *attn, const void *input,
+                                    void *mid, void *hidden, const void *gamma1, const void *beta1,
+                                    const void *gamma2, const void *beta2, int rows, void *ws, size_t ws_bytes,
+                                    void *stream);
+int et_linear_tile_tail_prepare(const et_linear_tile *out_proj, const et_linear_tile *first,
+                                const et_linear_tile *second);
+size_t et_linear_tile_tail_ws_bytes(const et_linear_tile *out_proj, const et_linear_tile *first,
+                                    const et_linear_tile *second, int rows);
 int et_linear_tile_tail_fusable(const et_linear_tile *out_proj, const et_linear_tile *first,
                                 const et_linear_tile *second);
 /* n <= 4 linears over one input in one launch (Q/K/V, encoder/encoder.cu:22-26) */

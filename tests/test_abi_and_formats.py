@@ -258,3 +258,25 @@ def test_seq_lens_outside_the_sequence_are_refused():
     for bad in ([64, 65, 1], [3, -1, 2], [1, 2]):
         with pytest.raises(ValueError):
             encoder._Encoder.set_seq_lens(enc, np.array(bad))
+
+
+def vwin_window_model(v_head_ptr, ldv, hd=64, rows=64):
+    """Host restatement of the value-window staging addresses of attention.hip (window start, per-piece column
+    clamp): yields (head, row, first column) of every 16-byte piece a tile fetches."""
+    rowb = (hd + 16) * 2           # LDS bytes per staged window row: 80 columns, all of them data
+    for h in range(len(v_head_ptr) - 1):
+        vc0 = min(int(v_head_ptr[h]) & ~7, ldv - 8)
+        for p in range(0, rows * rowb, 16):
+            row, cb = divmod(p, rowb)
+            yield h, row, vc0 + min(cb >> 1, ldv - 8 - vc0)
+
+
+@pytest.mark.parametrize("keep", [[3, 64, 0, 17, 8, 1, 64, 33, 64, 5, 21, 64], [64, 40, 16, 0, 0, 0, 0, 0, 0, 0, 0, 0],
+                                  [8] + [0] * 11, [0] * 11 + [8]])
+def test_value_window_pieces_stay_inside_their_row(keep):
+    """every staged piece of a value window lies inside its own row of compact V, also for heads that keep no
+    columns and sit at the very end of the row (v_head_ptr[h] == ldv)"""
+    hp = np.concatenate([[0], np.cumsum(keep)])
+    ldv = (int(hp[-1]) + 7) // 8 * 8
+    for h, row, col in vwin_window_model(hp, ldv):
+        assert 0 <= col and col + 8 <= ldv, (h, row, col, ldv)

@@ -293,6 +293,55 @@ def test_tile_layer_tail_fused(K, M, d, F, sp, fused):
         assert np.array_equal(host(ad), got)
 
 
+PAIR_CASES = [
+    (640, 768, 3072, 0.8),     # BERT-base widths, ten 64-row panels
+    (200, 256, 1024, 0.5),     # a ragged last panel (8 rows), two block-rows per wave
+    (130, 512, 2048, 0.7),     # four block-rows per wave
+    (64, 768, 1008, 0.8),      # hidden width that ends inside a 192-column phase
+    (96, 256, 384, 0.0),       # dense, one phase per half
+    (128, 768, 3072, 0.95),    # block-rows without any tile
+]
+
+
+@pytest.mark.parametrize("M,d,F,sp", PAIR_CASES)
+def test_tile_layer_tail_pairs(K, M, d, F, sp):
+    """the layer tail as pairs of workgroups over 64-row panels (scratch given, mid=None insists on it) == the
+    oracle's chain of five steps; a second run on the same plans (the per-panel counters reset themselves) and a
+    run whose output overwrites the attention buffer give the same bits; close to the one-workgroup form"""
+    from et_amd.encoder import Linear_tile
+    r = rng(7100 + M + d + F)
+    lo = make_tile_linear(r, d, d, sp, seed=3 * M + d, std=0.05, bias_std=0.2)
+    l1 = make_tile_linear(r, F, d, sp, seed=5 * M + F, std=0.05, bias_std=0.2)
+    l2 = make_tile_linear(r, d, F, sp, seed=7 * M + d, std=0.05, bias_std=0.2)
+    attn, inp = randn_h(r, (M, d)), randn_h(r, (M, d))
+    g1, b1 = randn_h(r, (d,), 0.3) + np.float16(1), randn_h(r, (d,), 0.3)
+    g2, b2 = randn_h(r, (d,), 0.3) + np.float16(1), randn_h(r, (d,), 0.3)
+    o = orc.tile_linear(attn, lo["row_ptr"], lo["row_offset"], lo["data"], lo["bias"], d)
+    mid = orc.skip_layernorm(o, inp, g1, b1)
+    h = orc.tile_linear(mid, l1["row_ptr"], l1["row_offset"], l1["data"], l1["bias"], F, gelu=True)
+    y = orc.tile_linear(h, l2["row_ptr"], l2["row_offset"], l2["data"], l2["bias"], d)
+    want = orc.skip_layernorm(y, mid, g2, b2)
+    mk = lambda l, K_, N_, gelu: Linear_tile(K_, N_, M, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], gelu)
+    to, t1, t2 = mk(lo, d, d, False), mk(l1, d, F, True), mk(l2, F, d, False)
+    need = Linear_tile.tail_ws_bytes(to, t1, t2, M)
+    assert need == ((M + 63) // 64) * 64 * (-(-d // 128) * 128) * 4 * 2
+    Linear_tile.tail_prepare(to, t1, t2)
+    ws = torch.full((need,), 0xFF, dtype=torch.uint8, device="cuda")   # NaN patterns: nothing may be read before written
+    ln = [dev(t) for t in (g1, b1, g2, b2)]
+    print(f"pair tail: M={M} d={d} F={F} sp={sp}", flush=True)
+    got = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln, ws=ws))
+    check_close(got, want, max_abs=3e-2, mean_rel=2e-3, what="paired layer tail vs oracle chain")
+    again = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln, ws=ws))
+    assert np.array_equal(got, again)
+    ad = dev(attn)
+    Linear_tile.run_tail(to, t1, t2, ad, dev(inp), *ln, out=ad, ws=ws)
+    assert np.array_equal(host(ad), got)
+    if Linear_tile.tail_fusable(to, t1, t2):
+        one = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln))
+        assert np.abs(got.astype(np.float32) - one.astype(np.float32)).max() <= 3e-2
+        assert (got != one).mean() < 0.05
+
+
 def test_tile_layer_tail_splits_off_a_small_last_round(K):
     """one workgroup per CU and 32-row panel: a last round of few panels runs step by step behind the fused launch"""
     from et_amd import lib
@@ -793,6 +842,24 @@ def test_prune_attention_value_windows(K, S, B, with_mask, with_lens):
     valid = np.ones(B * S, bool) if lens is None else np.concatenate([np.arange(S) < n for n in lens])
     check_close(got[valid], want[valid], max_abs=5e-3, mean_rel=1e-3, what="pruned attention, value windows")
     assert (got[~valid] == 0).all()
+    assert (got[:, np.setdiff1d(np.arange(d), v_id)] == 0).all()
+
+
+def test_prune_attention_value_windows_trailing_empty_heads(K):
+    """the last heads keep no value columns and the row pitch equals the kept total (a multiple of 8): their
+    windows start at the end of the row and must be pulled back inside it"""
+    r = rng(4242)
+    H, d, S, B = 12, 768, 128, 2
+    hd = d // H
+    Q, Kk, V = (randn_h(r, (B * S, d)) for _ in range(3))
+    keep = [64, 40, 16, 0, 0, 0, 0, 0, 0, 0, 0, 0]           # 120 kept columns, nothing behind head 2
+    v_id = np.concatenate([h * hd + np.sort(r.choice(hd, k, replace=False)) for h, k in enumerate(keep)]).astype(np.int32)
+    v_hp = orc.head_ptr(v_id, H, hd)
+    assert v_id.size % 8 == 0 and v_hp[-1] == v_hp[3] == v_id.size
+    Vc = np.ascontiguousarray(V[:, v_id])
+    want = orc.prune_attention(Q, Kk, Vc, None, v_id, v_hp, None, S, d, H, B, None, f64=True)
+    got = host(K.Prune_attention(dev(Q), dev(Kk), dev(Vc), None, dev(v_id), dev(v_hp), None, S, d, H, B, None))
+    check_close(got, want, max_abs=5e-3, mean_rel=1e-3, what="pruned attention, trailing empty heads")
     assert (got[:, np.setdiff1d(np.arange(d), v_id)] == 0).all()
 
 
