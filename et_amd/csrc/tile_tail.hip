@@ -34,12 +34,14 @@
 // for it at plan time (its 6 block-rows of the projection; then, per 192-column
 // phase p, one or two hidden block-rows of the first linear and its 6 output block-rows
 // of the second linear over chunk p, the first linear one phase ahead), through
-// a 4-deep register pipeline that never drains.  Where a segment of the stream
-// ends a descriptor says what to do with the finished 64 x 16 sums: GELU and
-// store into a hidden buffer, or add into one of the wave's output
-// accumulators; and which LDS event counter to wait for or to signal (hidden
-// buffer complete / hidden buffer free), exactly as an s_barrier would order
-// them but without stopping a wave that is not a whole phase ahead.  Waits are
+// a register pipeline of TT_DEPTH pairs that never drains.  Where a segment of the stream
+// ends, a control word that travels with the segment's last pair (next to its
+// operand offsets, so it costs no memory request of its own) says what to do
+// with the finished 64 x 16 sums: GELU and store into a hidden buffer, or add
+// into one of the wave's output accumulators; and which LDS event counter to
+// wait for or to signal (hidden buffer complete / hidden buffer free), exactly
+// as an s_barrier would order them but without stopping a wave that is not a
+// whole phase ahead.  Waits are
 // bounded; a wave that gives up sets the process's wait-status word, which the
 // next launch reports.  Both LayerNorms run on the accumulators where they are
 // (a panel row's 768 columns are spread over the 8 waves; row sums meet in
@@ -52,14 +54,25 @@
 
 namespace et {
 
-constexpr int TT_WAVES = 8;               // two per SIMD: 256 registers each (accumulators for 6 block-rows x 64 rows)
+#ifndef TT_NWAVES
+#define TT_NWAVES 12
+#endif
+constexpr int TT_WAVES = TT_NWAVES;       // 12: three per SIMD, 168 registers each (4 block-rows x 64 rows of accumulators); 8: two per SIMD
+static_assert(TT_WAVES == 8 || TT_WAVES == 12, "eight or twelve waves");
 constexpr int TT_BM = 64;                 // panel rows
 constexpr int TT_HB = 12;                 // hidden block-rows per phase
 constexpr int TT_HC = 16 * TT_HB;         // hidden columns per phase
 constexpr int TT_HW = (TT_HC + 16) * 2;   // bytes of one hidden buffer inside an LDS row
 constexpr int TT_MAX_PHASES = 16;         // per half: counters F[16], S[16]
 constexpr int TT_MAX_PANELS = 8192;       // counters per program: 2 per panel
-constexpr int TT_DESC = 8;                // ints per segment descriptor
+// Tile pairs in flight per wave.
+#ifndef TT_DEPTH
+#define TT_DEPTH (TT_NWAVES == 12 ? 4 : 8)
+#endif
+// stages the X fragments are read ahead of their MFMAs
+#ifndef TT_XA
+#define TT_XA 1
+#endif
 
 template <int D> struct TtGeom {
     static constexpr int NB = (D / 16 + TT_WAVES - 1) / TT_WAVES; // output block-rows per wave
@@ -72,24 +85,40 @@ template <int D> struct TtGeom {
     static_assert(RS % 64 == 32, "row stride must be == 32 (mod 64) bytes");
 };
 
-// segment descriptor (TT_DESC ints): [0] end (pair index in the wave's stream, exclusive), [1] kind | j << 8
-// (kind 0: add into accumulator j, 1: GELU into a hidden buffer), [2] hidden byte offset inside an LDS row,
-// [3] LDS byte offset of the 64-byte vector the running sums start from (zeros, or the block-row's bias),
-// [4] counter to wait for before the hidden store (byte offset | target << 16, -1 none), [5] counter to signal
-// afterwards (byte offset, -1 none), [6] counter to wait for before the NEXT segment's first operand is read
+// A pair's record in the stream: 16 bytes, {offset of tile A, control, offset of
+// tile B, control} - lanes 0-31 read the first half, lanes 32-63 the second.  An
+// offset is the LDS byte offset of the tile's X columns inside the lane's row
+// (panel part or a hidden buffer).  The control word is 0 except on the last
+// pair of a segment:
+//   bit 0      set
+//   bit 1      the segment is a hidden block-row of the first linear (GELU, store)
+//   bits 2-4   accumulator the sums are added to (7: none)
+//   bits 5-8   slot of the hidden block-row in its 192-column buffer
+//   bits 9-12  phase p of the segment (buffer p & 1, counters F[p] / S[p])
+//   bit 13     wait for S[p - 2] (all waves) before the hidden store
+//   bit 14     signal F[p] (hidden block-row) or S[p] (second linear) afterwards
+//   bit 15     before the NEXT segment's first operand is read, wait for
+//   bits 16-19   F[p'] to reach
+//   bits 20-23   this count minus one
+//   bits 24-31 what the next segment's sums start from: 255 zeros, else the
+//              bias of hidden block-row (index inside this half)
+constexpr int TT_C_SET = 1, TT_C_HID = 2, TT_C_WAITF = 1 << 13, TT_C_SIG = 1 << 14, TT_C_WAITN = 1 << 15;
+
 struct TtArgs {
     const f16 *pairs;
-    const int *off;
-    const int *desc;
-    const int *wtab; // per (half, wave): projection pair base, stages, descriptor base; feed-forward ditto; initial wait
+    const int *rec;
+    const int *wtab; // per (half, wave): projection pair base, stages; feed-forward pair base, stages; first start vector; initial wait
     const f16 *attn, *input;
     f16 *Y;
     const f16 *biasO, *bias1, *bias2, *g1, *b1, *g2, *b2;
-    float *ws;
+    unsigned long long *ws;
     int *sync;   // per panel: two row-half counters
     int *status; // set when a bounded wait gives up
     int M, npanels, per_xcd, spin;
     int hb0[2], nb1h[2]; // first hidden block-row and count per half
+#ifdef TT_TRACE
+    long long *trace; // per (workgroup, wave): 16 stamps
+#endif
 };
 
 template <int I> using tt_ic = std::integral_constant<int, I>;
@@ -101,20 +130,28 @@ __device__ __forceinline__ void tt_static_for(F &&f) {
     }
 }
 
-// One pair's operands: 16 bytes of W per lane and the lane's X offset.  The
-// pair's address is wave-uniform and the lane's part a 32-bit offset kept
-// opaque in place, so the loads need no vector address arithmetic.
-__device__ __forceinline__ void tt_load_pair(const char *wq, const char *oq, unsigned &lo, unsigned &lw,
-                                             f16x8 &w, int &o) {
+// One pair's operands: 16 bytes of W per lane, the lane's X offset and the
+// control word.  The pair's address is wave-uniform and the lane's part a 32-bit
+// offset kept opaque in place, so the loads need no vector address arithmetic.
+__device__ __forceinline__ void tt_load_pair(const char *wq, const char *rq, unsigned &lo, unsigned &lw,
+                                             f16x8 &w, int &o, int &c) {
+    typedef int i32x2 __attribute__((ext_vector_type(2)));
     asm("" : "+v"(lo), "+v"(lw));
-    o = *reinterpret_cast<const int *>(oq + lo);
+    const i32x2 r = *reinterpret_cast<const i32x2 *>(rq + lo);
+    o = r[0];
+    c = r[1];
     w = *reinterpret_cast<const f16x8 *>(wq + lw);
 }
 
+// A wave's LDS operations are executed in the order it issued them, so an add
+// that follows the wave's stores in program order is seen after them by
+// everyone: no wait for the stores (a release fence would be an s_waitcnt, i.e.
+// an LDS round trip per signal), only a barrier for the compiler.
 __device__ __forceinline__ void tt_signal(unsigned *ctr, int lane) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local"); // this wave's LDS traffic first
+    asm volatile("" ::: "memory");
     if (lane == 0)
         __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    asm volatile("" ::: "memory");
 }
 // Bounded: after `spin` polls the wave sets the status word and goes on (the
 // result of this launch is then wrong, and the next launch reports it).
@@ -158,36 +195,57 @@ __device__ __forceinline__ void tt_read_x(f16x8 (&x)[4], const char *xl, int off
         x[k] = *reinterpret_cast<const f16x8 *>(p + k * 16 * RS);
 }
 
-// The stream: n stages (a multiple of 4), pair q's operands in w[q % 4] / o[q % 4]
-// (the first four requested by the caller), X fragments read one stage ahead,
-// four MFMAs per stage into cur[0..3] (one per 16-row subtile).  at_end(xn, on)
-// runs where a stage finishes the segment that ends at `send`; xn / on are the
-// fragments and the offset of the NEXT pair, for a handler that has to wait
-// before they may be read.
+// The stream: n stages (a multiple of TT_DEPTH), pair q's operands in slot q %
+// TT_DEPTH of w / o / c (the first TT_DEPTH requested by the caller), X fragments
+// read TT_XA stages ahead, four MFMAs per stage into cur[0..3] (one per 16-row
+// subtile).  at_end(ctl, reread) runs where a stage finishes a segment (its
+// pair's control word is not 0); reread() reads the fragments of the pairs that
+// are already on their way once more, for a handler that has to wait before
+// they may be read.
 template <int RS, class AtEnd>
-__device__ __forceinline__ void tt_stream(const char *xl, const char *wq, const char *oq, int n,
-                                          unsigned &lane_lo, unsigned &lane_lw, f16x8 (&w)[4], int (&o)[4],
-                                          f32x4 (&cur)[4], int &send, AtEnd &&at_end) {
-    f16x8 xf[2][4];
-    tt_read_x<RS>(xf[0], xl, o[0]);
-    const char *wp = wq + 4 * 1024, *op = oq + 4 * 8;
-    for (int q = 0; q < n; q += 4) {
-        tt_static_for<0, 4>([&](auto ic) {
-            constexpr int I = decltype(ic)::value, SN = (I + 1) & 3, P = I & 1;
-            tt_read_x<RS>(xf[P ^ 1], xl, o[SN]);
+__device__ __forceinline__ void tt_stream(const char *xl, const char *wq, const char *rq, int n,
+                                          unsigned &lane_lo, unsigned &lane_lw, f16x8 (&w)[TT_DEPTH],
+                                          int (&o)[TT_DEPTH], int (&c)[TT_DEPTH], f32x4 (&cur)[4],
+                                          AtEnd &&at_end) {
+    constexpr int NX = TT_XA + 1;
+    static_assert(TT_DEPTH % NX == 0 && TT_XA < TT_DEPTH, "fragment buffers rotate inside the unrolled group");
+    f16x8 xf[NX][4];
+#pragma unroll
+    for (int i = 0; i < TT_XA; i++)
+        tt_read_x<RS>(xf[i], xl, o[i]);
+    const char *wp = wq + TT_DEPTH * 1024, *rp = rq + TT_DEPTH * 16;
+    for (int q = 0; q < n; q += TT_DEPTH) {
+        tt_static_for<0, TT_DEPTH>([&](auto ic) {
+            constexpr int I = decltype(ic)::value;
+#if !(defined(TT_ABL) && (TT_ABL & 1))
+            tt_read_x<RS>(xf[(I + TT_XA) % NX], xl, o[(I + TT_XA) % TT_DEPTH]);
+#endif
             // keep the reads above the MFMAs (the scheduler otherwise sinks them
             // and every stage waits out the LDS latency)
             __builtin_amdgcn_sched_barrier(0);
+#if !(defined(TT_ABL) && (TT_ABL & 4))
 #pragma unroll
             for (int k = 0; k < 4; k++)
-                cur[k] = mfma16x16x32(w[I], xf[P][k], cur[k]);
-            // pair q + I + 4 (unconditional: the stream is followed by spare pairs)
-            tt_load_pair(wp + I * 1024, op + I * 8, lane_lo, lane_lw, w[I], o[I]);
-            if (q + I + 1 == send)
-                at_end(xf[P ^ 1], o[SN]);
+                cur[k] = mfma16x16x32(w[I], xf[I % NX][k], cur[k]);
+#endif
+#if (defined(TT_EXP) && TT_EXP == 5) || defined(TT_NOH)
+            const int ctl = 0;
+#else
+            const int ctl = __builtin_amdgcn_readfirstlane(c[I]);
+#endif
+            // pair q + I + TT_DEPTH (unconditional: the stream is followed by spare pairs)
+#if !(defined(TT_ABL) && (TT_ABL & 2))
+            tt_load_pair(wp + I * 1024, rp + I * 16, lane_lo, lane_lw, w[I], o[I], c[I]);
+#endif
+            if (ctl != 0)
+                at_end(ctl, [&]() {
+#pragma unroll
+                    for (int i = 1; i <= TT_XA; i++)
+                        tt_read_x<RS>(xf[(I + i) % NX], xl, o[(I + i) % TT_DEPTH]);
+                });
         });
-        wp += 4 * 1024;
-        op += 4 * 8;
+        wp += TT_DEPTH * 1024;
+        rp += TT_DEPTH * 16;
     }
 }
 
@@ -205,6 +263,9 @@ __device__ __forceinline__ void tt_add_tied(f32x4 &a, const f32x4 &c) {
                  : "v"(c[0]), "v"(c[1]), "v"(c[2]), "v"(c[3]), "n"(K));
     a = f32x4{a0, a1, a2, a3};
 }
+// acc[j] += cur for a wave-uniform run-time j (no accumulator for j >= NB).  A
+// sequence of independent ifs with something opaque between them: as an if /
+// else chain it becomes a switch whose lowering copies the accumulators around.
 template <int NB>
 __device__ __forceinline__ void tt_acc_add(f32x4 (&acc)[NB][4], int j, const f32x4 (&cur)[4]) {
     tt_static_for<0, NB>([&](auto kc) {
@@ -221,11 +282,12 @@ __device__ __forceinline__ void tt_acc_add(f32x4 (&acc)[NB][4], int j, const f32
 
 // Skip + LayerNorm on values held in the accumulator layout: lane (c16, g4) of
 // wave w holds, per block-row j and 16-row subtile ms, columns 16*(NB*w + j) +
-// 4*g4 .. +3 of panel row 16*(ms0 + ms) + c16, already as x = half(y) + skip.
-// The math of skip_layernorm.hip (fp32 mean, two-pass biased variance, eps
-// 1e-6; kernels/skip_layernorm.cu:4-43).  A row's partial sums of the eight waves
-// meet in the hidden-buffer part of that row in LDS (free whenever this runs)
-// and are added in wave order.  Two workgroup barriers.
+// 4*g4 .. +3 of panel row 16*(ms0 + ms) + c16, already as x = half(y) + skip
+// (zeros in block-rows beyond the matrix).  The math of skip_layernorm.hip (fp32
+// mean, two-pass biased variance, eps 1e-6; kernels/skip_layernorm.cu:4-43).  A
+// row's partial sums of the eight waves meet in the hidden-buffer part of that
+// row in LDS (free whenever this runs) and are added in wave order.  Two
+// workgroup barriers.
 template <int D, int NMS>
 __device__ __forceinline__ void tt_ln(f16x4 (&x)[TtGeom<D>::NB][NMS], int ms0,
                                       const f16x4 (&gam)[TtGeom<D>::NB], const f16x4 (&bet)[TtGeom<D>::NB],
@@ -236,15 +298,19 @@ __device__ __forceinline__ void tt_ln(f16x4 (&x)[TtGeom<D>::NB][NMS], int ms0,
     float mean[NMS], rstd[NMS];
     auto total = [&](int ms, int at) {
         const f32x4 *p = reinterpret_cast<const f32x4 *>(smem + (16 * (ms0 + ms) + c16) * RS + XW + at);
-        static_assert(TT_WAVES == 8, "eight partial sums per row");
         const f32x4 a0 = p[0], a1 = p[1];
-        return ((a0[0] + a0[1]) + (a0[2] + a0[3])) + ((a1[0] + a1[1]) + (a1[2] + a1[3]));
+        float t = ((a0[0] + a0[1]) + (a0[2] + a0[3])) + ((a1[0] + a1[1]) + (a1[2] + a1[3]));
+        if constexpr (TT_WAVES == 12) {
+            const f32x4 a2 = p[2];
+            t += (a2[0] + a2[1]) + (a2[2] + a2[3]);
+        }
+        return t;
     };
 #pragma unroll
     for (int ms = 0; ms < NMS; ms++) {
         float s = 0.f;
 #pragma unroll
-        for (int j = 0; j < NB; j++) { // (block-rows beyond the matrix hold zeros)
+        for (int j = 0; j < NB; j++) {
             s = __builtin_amdgcn_fdot2(h2{x[j][ms][0], x[j][ms][1]}, h2{(f16)1, (f16)1}, s, false);
             s = __builtin_amdgcn_fdot2(h2{x[j][ms][2], x[j][ms][3]}, h2{(f16)1, (f16)1}, s, false);
         }
@@ -260,14 +326,15 @@ __device__ __forceinline__ void tt_ln(f16x4 (&x)[TtGeom<D>::NB][NMS], int ms0,
     for (int ms = 0; ms < NMS; ms++) {
         float v = 0.f;
 #pragma unroll
-        for (int j = 0; j < NB; j++)
-            if (j < nvalid) {
+        for (int j = 0; j < NB; j++) {
+            float vj = 0.f;
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const float d = (float)x[j][ms][r] - mean[ms];
-                    v += d * d;
-                }
+            for (int r = 0; r < 4; r++) {
+                const float d = (float)x[j][ms][r] - mean[ms];
+                vj += d * d;
             }
+            v += j < nvalid ? vj : 0.f; // (a block-row beyond the matrix is not part of the row)
+        }
         v = tt_xor_sum_16_32(v);
         if (g4 == 0)
             *reinterpret_cast<float *>(smem + (16 * (ms0 + ms) + c16) * RS + XW + 64 + wave * 4) = v;
@@ -289,7 +356,7 @@ __device__ __forceinline__ void tt_ln(f16x4 (&x)[TtGeom<D>::NB][NMS], int ms0,
 template <int D>
 __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtArgs a) {
     using G = TtGeom<D>;
-    constexpr int NB = G::NB, RS = G::RS, nbrD = D / 16;
+    constexpr int NB = G::NB, RS = G::RS, XW = G::XW, nbrD = D / 16;
     extern __shared__ __attribute__((aligned(16))) unsigned char tt_smem[];
     char *const smem = reinterpret_cast<char *>(tt_smem);
     // the two workgroups of a panel get neighbouring slots of ONE XCD (hardware
@@ -306,8 +373,18 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
     unsigned *const ctr = reinterpret_cast<unsigned *>(smem + G::CT);
     int *const misc = reinterpret_cast<int *>(smem + G::MISC);
     const int nvalid = min(max(nbrD - NB * wave, 0), NB); // this wave's block-rows inside the matrix
+#ifdef TT_TRACE
+    long long tr_wait = 0, tr_hand = 0;
+    int tr_nh = 0;
+#define TT_STAMP(i_) if (lane == 0) a.trace[((size_t)vid * TT_WAVES + wave) * 16 + (i_)] = wall_clock64();
+#define TT_STAMPV(i_, v_) if (lane == 0) a.trace[((size_t)vid * TT_WAVES + wave) * 16 + (i_)] = (v_);
+#else
+#define TT_STAMP(i_)
+#define TT_STAMPV(i_, v_)
+#endif
+    TT_STAMP(0)
 
-    // the panel (attention output): DMA, wave w takes rows w, w + 12, ...
+    // the panel (attention output): DMA, wave w takes rows w, w + 8, ...
     {
         constexpr int PCPR = D / 8; // 16-byte pieces per row, <= 124
         for (int r = wave; r < TT_BM; r += TT_WAVES)
@@ -332,24 +409,20 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
     }
     typedef const __attribute__((address_space(4))) int *ScalarInts;
     const ScalarInts wt = (ScalarInts)a.wtab + (half * TT_WAVES + wave) * 8;
-    const int o_base = __builtin_amdgcn_readfirstlane(wt[0]), o_n = __builtin_amdgcn_readfirstlane(wt[1]),
-              o_desc = __builtin_amdgcn_readfirstlane(wt[2]), f_base = __builtin_amdgcn_readfirstlane(wt[3]),
-              f_n = __builtin_amdgcn_readfirstlane(wt[4]), f_desc = __builtin_amdgcn_readfirstlane(wt[5]),
-              f_wait0 = __builtin_amdgcn_readfirstlane(wt[6]);
-    const ScalarInts dsc = (ScalarInts)a.desc;
-    // (descriptor words are wave-uniform; saying so keeps every branch on them scalar)
-#define TT_U(x_) __builtin_amdgcn_readfirstlane(x_)
-    unsigned lane_lo = hi * 4u, lane_lw = (hi * 256 + c16 * 16 + khalf8) * 2u;
+    const int o_base = wt[0], o_n = wt[1], f_base = wt[2], f_n = wt[3], f_init = wt[4], f_wait0 = wt[5];
+    unsigned lane_lo = hi * 8u, lane_lw = (hi * 256 + c16 * 16 + khalf8) * 2u;
     const char *const pairs = reinterpret_cast<const char *>(a.pairs);
-    const char *const offs = reinterpret_cast<const char *>(a.off);
-    f16x8 w[4];
-    int o[4];
+    const char *const recs = reinterpret_cast<const char *>(a.rec);
+    f16x8 w[TT_DEPTH];
+    int o[TT_DEPTH], c[TT_DEPTH];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
-        tt_load_pair(pairs + (size_t)(o_base + i) * 1024, offs + (size_t)(o_base + i) * 8, lane_lo, lane_lw, w[i],
-                     o[i]);
+    for (int i = 0; i < TT_DEPTH; i++)
+        tt_load_pair(pairs + (size_t)(o_base + i) * 1024, recs + (size_t)(o_base + i) * 16, lane_lo, lane_lw, w[i],
+                     o[i], c[i]);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's part of the panel has landed
+    TT_STAMP(1)
     __syncthreads();
+    TT_STAMP(2)
 
     f32x4 acc[NB][4], cur[4];
 #pragma unroll
@@ -363,56 +436,59 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
     const char *const xl = smem + c16 * RS + khalf8 * 2;
 
     // ---- the projection: this wave's NB block-rows over the whole panel ----
-    {
-        int seg = 0;
-        int d_kind = TT_U(dsc[(size_t)o_desc * TT_DESC + 1]);
-        int send = TT_U(dsc[(size_t)o_desc * TT_DESC]);
-        int n_end = TT_U(dsc[(size_t)(o_desc + 1) * TT_DESC]), n_kind = TT_U(dsc[(size_t)(o_desc + 1) * TT_DESC + 1]);
-        tt_stream<RS>(xl, pairs + (size_t)o_base * 1024, offs + (size_t)o_base * 8, o_n, lane_lo, lane_lw, w, o, cur,
-                      send, [&](f16x8(&)[4], int) {
-                          tt_acc_add<NB>(acc, d_kind >> 8, cur);
+    tt_stream<RS>(xl, pairs + (size_t)o_base * 1024, recs + (size_t)o_base * 16, o_n, lane_lo, lane_lw, w, o, c, cur,
+                  [&](int ctl, auto &&) {
+                      tt_acc_add<NB>(acc, (ctl >> 2) & 7, cur);
 #pragma unroll
-                          for (int ms = 0; ms < 4; ms++)
-                              cur[ms] = f32x4{0.f, 0.f, 0.f, 0.f};
-                          d_kind = n_kind;
-                          send = n_end;
-                          seg++;
-                          n_end = TT_U(dsc[(size_t)(o_desc + seg + 1) * TT_DESC]);
-                          n_kind = TT_U(dsc[(size_t)(o_desc + seg + 1) * TT_DESC + 1]);
-                      });
+                      for (int ms = 0; ms < 4; ms++)
+                          cur[ms] = f32x4{0.f, 0.f, 0.f, 0.f};
+                  });
+    TT_STAMP(3)
+#if defined(TT_EXP) && (TT_EXP == 5 || TT_EXP == 6)
+    if (a.M > 0) {
+        a.Y[(size_t)m0 * D + tid] = (f16)(cur[0][0] + acc[0][0][0]);
+        return;
     }
-    // the first pairs of the feed-forward stream travel under the LayerNorm
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-        tt_load_pair(pairs + (size_t)(f_base + i) * 1024, offs + (size_t)(f_base + i) * 8, lane_lo, lane_lw, w[i],
-                     o[i]);
+#endif
 
     // ---- bias + skip (the layer input) + LayerNorm 1, written over the panel ----
     {
-        f16x4 x[NB][4], gam[NB], bet[NB];
+        // every operand is requested before any is used, from addresses that are
+        // legal for all lanes (block-rows beyond the matrix read column 0 and are
+        // zeroed afterwards): one memory latency for the whole step
+        f16x4 x[NB][4], gam[NB], bet[NB], bo[NB];
 #pragma unroll
         for (int j = 0; j < NB; j++) {
-            const int col = (NB * wave + j) * 16 + g4 * 4;
-            f16x4 bo = f16x4{0, 0, 0, 0};
-            gam[j] = bet[j] = bo;
-            if (j < nvalid) {
-                bo = *reinterpret_cast<const f16x4 *>(a.biasO + col);
-                gam[j] = *reinterpret_cast<const f16x4 *>(a.g1 + col);
-                bet[j] = *reinterpret_cast<const f16x4 *>(a.b1 + col);
-            }
-            const f32x4 bf = __builtin_convertvector(bo, f32x4);
+            const int col = j < nvalid ? (NB * wave + j) * 16 + g4 * 4 : 0;
+            bo[j] = *reinterpret_cast<const f16x4 *>(a.biasO + col);
+            gam[j] = *reinterpret_cast<const f16x4 *>(a.g1 + col);
+            bet[j] = *reinterpret_cast<const f16x4 *>(a.b1 + col);
+#pragma unroll
+            for (int ms = 0; ms < 4; ms++)
+                x[j][ms] = *reinterpret_cast<const f16x4 *>(
+                    a.input + (size_t)min(m0 + 16 * ms + c16, a.M - 1) * D + col);
+        }
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            const f32x4 bf = __builtin_convertvector(bo[j], f32x4);
+            const f16x4 zero = f16x4{0, 0, 0, 0};
 #pragma unroll
             for (int ms = 0; ms < 4; ms++) {
-                f16x4 sk = f16x4{0, 0, 0, 0};
-                if (j < nvalid)
-                    sk = *reinterpret_cast<const f16x4 *>(
-                        a.input + (size_t)min(m0 + 16 * ms + c16, a.M - 1) * D + col);
                 // half(acc + bias) is the linear's output as the reference stores it; the
                 // skip connection is added in half (kernels/skip_layernorm.cu:20)
-                x[j][ms] = __builtin_convertvector(acc[j][ms] + bf, f16x4) + sk;
+                const f16x4 v = __builtin_convertvector(acc[j][ms] + bf, f16x4) + x[j][ms];
+                x[j][ms] = j < nvalid ? v : zero;
             }
         }
+        TT_STAMP(13)
+        // the first pairs of the feed-forward stream travel under the LayerNorm
+#pragma unroll
+        for (int i = 0; i < TT_DEPTH; i++)
+            tt_load_pair(pairs + (size_t)(f_base + i) * 1024, recs + (size_t)(f_base + i) * 16, lane_lo, lane_lw,
+                         w[i], o[i], c[i]);
+        TT_STAMP(14)
         tt_ln<D, 4>(x, 0, gam, bet, smem, wave, c16, g4, nvalid);
+        TT_STAMP(15)
         // (every wave has passed a barrier since its last read of the attention panel)
 #pragma unroll
         for (int j = 0; j < NB; j++)
@@ -427,36 +503,47 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
 #pragma unroll
         for (int ms = 0; ms < 4; ms++)
             acc[j][ms] = f32x4{0.f, 0.f, 0.f, 0.f};
+    TT_STAMP(4)
     __syncthreads(); // the feed-forward input panel is complete
+    TT_STAMP(5)
+#if defined(TT_EXP) && TT_EXP == 1
+    return;
+#endif
 
     // ---- the feed-forward block over this half of the hidden columns ----
     {
-        int seg = 0;
-        int send, d_kind, d_hoff, d_wf, d_sig, d_wn;
-        int n_end, n_kind, n_hoff, n_init, n_wf, n_sig, n_wn;
-        {
-            const ScalarInts p = dsc + (size_t)f_desc * TT_DESC;
-            send = TT_U(p[0]), d_kind = TT_U(p[1]), d_hoff = TT_U(p[2]), d_wf = TT_U(p[4]), d_sig = TT_U(p[5]),
-            d_wn = TT_U(p[6]);
-            const f32x4 init = *reinterpret_cast<const f32x4 *>(smem + p[3] + g4 * 16);
+        auto start_vector = [&](int idx) { // what a segment's sums start from: zeros or a hidden block-row's bias
+            f32x4 init = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (idx != 255) // (most segments start from zeros: no LDS round trip for those)
+                init = *reinterpret_cast<const f32x4 *>(smem + G::BI + idx * 64 + g4 * 16);
 #pragma unroll
             for (int ms = 0; ms < 4; ms++)
                 cur[ms] = init;
-            const ScalarInts pn = p + TT_DESC;
-            n_end = TT_U(pn[0]), n_kind = TT_U(pn[1]), n_hoff = TT_U(pn[2]), n_init = TT_U(pn[3]), n_wf = TT_U(pn[4]),
-            n_sig = TT_U(pn[5]), n_wn = TT_U(pn[6]);
-        }
+        };
+        start_vector(f_init);
         if (f_wait0 >= 0)
-            tt_wait(ctr + ((f_wait0 & 0xffff) >> 2), (unsigned)f_wait0 >> 16, a.spin, a.status, lane);
+            tt_wait(ctr + (f_wait0 & 15), (unsigned)(f_wait0 >> 8), a.spin, a.status, lane);
         tt_stream<RS>(
-            xl, pairs + (size_t)f_base * 1024, offs + (size_t)f_base * 8, f_n, lane_lo, lane_lw, w, o, cur, send,
-            [&](f16x8(&xn)[4], int on) {
-                if ((d_kind & 0xff) == 1) {
+            xl, pairs + (size_t)f_base * 1024, recs + (size_t)f_base * 16, f_n, lane_lo, lane_lw, w, o, c, cur,
+            [&](int ctl, auto &&reread) {
+#ifdef TT_TRACE
+                const long long th0 = wall_clock64();
+                tr_nh++;
+#endif
+                const int p = (ctl >> 9) & 15;
+                if (ctl & TT_C_HID) {
                     // a finished hidden block-row (its bias was the starting value): GELU,
                     // rounded to half as the reference stores it, into the hidden buffer
-                    if (d_wf >= 0) // ... once everyone has finished reading what it held before
-                        tt_wait(ctr + ((d_wf & 0xffff) >> 2), (unsigned)d_wf >> 16, a.spin, a.status, lane);
-                    char *hp = smem + c16 * RS + d_hoff + g4 * 8;
+                    if (ctl & TT_C_WAITF) { // ... once everyone has finished reading what it held before
+#ifdef TT_TRACE
+                        const long long tw0 = wall_clock64();
+#endif
+                        tt_wait(ctr + TT_MAX_PHASES + p - 2, TT_WAVES, a.spin, a.status, lane);
+#ifdef TT_TRACE
+                        tr_wait += wall_clock64() - tw0;
+#endif
+                    }
+                    char *hp = smem + c16 * RS + (XW + (p & 1) * TT_HW + ((ctl >> 5) & 15) * 32) + g4 * 8;
 #pragma unroll
                     for (int ms = 0; ms < 4; ms++) {
                         *reinterpret_cast<f16x4 *>(hp + ms * 16 * RS) =
@@ -466,111 +553,150 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
                 }
                 // (not in an else branch: as a part of that if / else the accumulators were
                 // given a second set of registers behind the handler; a hidden block-row's
-                // descriptor carries j = 255, which matches no accumulator)
-                tt_acc_add<NB>(acc, d_kind >> 8, cur);
-                if (d_sig >= 0)
-                    tt_signal(ctr + (d_sig >> 2), lane);
-                if (d_wn >= 0) {
+                // control word names accumulator 7, which does not exist)
+                tt_acc_add<NB>(acc, (ctl >> 2) & 7, cur);
+                if (ctl & TT_C_SIG)
+                    tt_signal(ctr + ((ctl & TT_C_HID) ? p : TT_MAX_PHASES + p), lane);
+                if (ctl & TT_C_WAITN) {
                     // the next segment multiplies a hidden buffer: wait until it is complete
                     // and read the next pair's fragments again
-                    tt_wait(ctr + ((d_wn & 0xffff) >> 2), (unsigned)d_wn >> 16, a.spin, a.status, lane);
-                    tt_read_x<RS>(xn, xl, on);
+#ifdef TT_TRACE
+                    const long long tw0 = wall_clock64();
+#endif
+                    tt_wait(ctr + ((ctl >> 16) & 15), (unsigned)((ctl >> 20) & 15) + 1u, a.spin, a.status, lane);
+#ifdef TT_TRACE
+                    tr_wait += wall_clock64() - tw0;
+#endif
+                    reread();
                 }
-                const f32x4 init = *reinterpret_cast<const f32x4 *>(smem + n_init + g4 * 16);
-#pragma unroll
-                for (int ms = 0; ms < 4; ms++)
-                    cur[ms] = init;
-                send = n_end, d_kind = n_kind, d_hoff = n_hoff, d_wf = n_wf, d_sig = n_sig, d_wn = n_wn;
-                seg++;
-                const ScalarInts pn = dsc + (size_t)(f_desc + seg + 1) * TT_DESC;
-                n_end = TT_U(pn[0]), n_kind = TT_U(pn[1]), n_hoff = TT_U(pn[2]), n_init = TT_U(pn[3]), n_wf = TT_U(pn[4]),
-                n_sig = TT_U(pn[5]), n_wn = TT_U(pn[6]);
+                start_vector((int)((unsigned)ctl >> 24));
+#ifdef TT_TRACE
+                tr_hand += wall_clock64() - th0;
+#endif
             });
-#undef TT_U
     }
+    TT_STAMP(6)
+    TT_STAMPV(10, tr_wait)
+    TT_STAMPV(11, tr_hand)
+    TT_STAMPV(12, tr_nh)
+#if defined(TT_EXP) && TT_EXP == 2
+    return;
+#endif
 
     // ---- the two halves' partial sums meet; bias + skip + LayerNorm 2; store ----
     f16x4 b2[NB], gam[NB], bet[NB];
 #pragma unroll
     for (int j = 0; j < NB; j++) {
-        const int col = (NB * wave + j) * 16 + g4 * 4;
-        b2[j] = gam[j] = bet[j] = f16x4{0, 0, 0, 0};
-        if (j < nvalid) {
-            b2[j] = *reinterpret_cast<const f16x4 *>(a.bias2 + col);
-            gam[j] = *reinterpret_cast<const f16x4 *>(a.g2 + col);
-            bet[j] = *reinterpret_cast<const f16x4 *>(a.b2 + col);
-        }
+        const int col = j < nvalid ? (NB * wave + j) * 16 + g4 * 4 : 0;
+        b2[j] = *reinterpret_cast<const f16x4 *>(a.bias2 + col);
+        gam[j] = *reinterpret_cast<const f16x4 *>(a.g2 + col);
+        bet[j] = *reinterpret_cast<const f16x4 *>(a.b2 + col);
     }
-    __syncthreads(); // every wave has left the hidden buffers
-    // scratch of (panel, half, row-half): [wave][j][subtile][lane] float4, coalesced both ways
-    constexpr size_t PART = (size_t)TT_WAVES * NB * 2 * 64 * 4; // floats per (panel, half, row-half)
-    for (int visit = 0; visit < 2; visit++) {
-        const int h = visit == 0 ? 1 - half : half; // the other workgroup's row-half first
-        int *const cnt = a.sync + 2 * panel + h;
-        if (tid == 0)
-            misc[0] = __hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        int arrived = misc[0]; // 1: the partner's partial of this row-half is in scratch
-        if (arrived == 0) {
-            f32x4 *dst = reinterpret_cast<f32x4 *>(a.ws + ((size_t)(panel * 2 + half) * 2 + h) * PART) +
-                         (size_t)wave * NB * 2 * 64 + lane;
+    // Scratch of (panel, half, row-half): [wave][j][subtile][piece][lane] 8-byte
+    // words, coalesced both ways.  Every access to it is an agent-scope atomic
+    // (relaxed): such a store is complete at the device's coherence point when the
+    // wave's memory counter says so, and such a load does not take a stale line
+    // from another XCD's L2 - the data of one row-half costs what it is, not a
+    // write-back and invalidation of the whole L2 as a device-scope fence would.
+    // Order: all waves wait for their stores, barrier, THEN thread 0 touches the
+    // counter; a reader loads only after the barrier behind thread 0's counter read.
+    constexpr size_t PART = (size_t)TT_WAVES * NB * 2 * 2 * 64; // words per (panel, half, row-half)
+    auto publish = [&](int h) {
+        unsigned long long *dst = a.ws + ((size_t)(panel * 2 + half) * 2 + h) * PART + (size_t)wave * NB * 4 * 64 + lane;
 #pragma unroll
-            for (int j = 0; j < NB; j++)
+        for (int j = 0; j < NB; j++)
+#pragma unroll
+            for (int m2 = 0; m2 < 2; m2++) {
+                const f32x4 v = h ? acc[j][2 + m2] : acc[j][m2]; // (selected, not indexed: acc stays in registers)
+                typedef float f32x2 __attribute__((ext_vector_type(2)));
+                __hip_atomic_store(dst + ((j * 2 + m2) * 2 + 0) * 64,
+                                   __builtin_bit_cast(unsigned long long, f32x2{v[0], v[1]}), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(dst + ((j * 2 + m2) * 2 + 1) * 64,
+                                   __builtin_bit_cast(unsigned long long, f32x2{v[2], v[3]}), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            }
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's stores are complete
+    };
+    auto finish = [&](int h) {
+        const unsigned long long *src =
+            a.ws + ((size_t)(panel * 2 + (1 - half)) * 2 + h) * PART + (size_t)wave * NB * 4 * 64 + lane;
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        f32x4 other[NB][2];
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+#pragma unroll
+            for (int m2 = 0; m2 < 2; m2++) {
+                const f32x2 lo = __builtin_bit_cast(
+                    f32x2, __hip_atomic_load(src + ((j * 2 + m2) * 2 + 0) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                const f32x2 hi2 = __builtin_bit_cast(
+                    f32x2, __hip_atomic_load(src + ((j * 2 + m2) * 2 + 1) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                other[j][m2] = f32x4{lo[0], lo[1], hi2[0], hi2[1]};
+            }
+        f16x4 x[NB][2];
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            const f32x4 bf = __builtin_convertvector(b2[j], f32x4);
+            const f16x4 zero = f16x4{0, 0, 0, 0};
+#pragma unroll
+            for (int m2 = 0; m2 < 2; m2++) {
+                const int col = j < nvalid ? (NB * wave + j) * 16 + g4 * 4 : 0;
+                const f16x4 sk = *reinterpret_cast<const f16x4 *>(smem + (16 * (2 * h + m2) + c16) * RS + col * 2);
+                const f32x4 mine = h ? acc[j][2 + m2] : acc[j][m2];
+                const f16x4 v = __builtin_convertvector((mine + other[j][m2]) + bf, f16x4) + sk;
+                x[j][m2] = j < nvalid ? v : zero;
+            }
+        }
+        tt_ln<D, 2>(x, 2 * h, gam, bet, smem, wave, c16, g4, nvalid);
+        // in place over the skip operand (each lane overwrites what it read), then
+        // whole rows leave with 16-byte stores
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+            if (j < nvalid)
 #pragma unroll
                 for (int m2 = 0; m2 < 2; m2++)
-                    dst[(j * 2 + m2) * 64] = h ? acc[j][2 + m2] : acc[j][m2]; // (selected, not indexed: acc stays in registers)
-            __threadfence(); // the partial is visible to the device before the counter says so
-            __syncthreads();
-            if (tid == 0)
-                misc[1] = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-            __syncthreads();
-            arrived = misc[1];
+                    *reinterpret_cast<f16x4 *>(smem + (16 * (2 * h + m2) + c16) * RS +
+                                               ((NB * wave + j) * 16 + g4 * 4) * 2) = x[j][m2];
+        __syncthreads();
+        constexpr int PR = D / 8;
+        for (int i = tid; i < 32 * PR; i += TT_WAVES * 64) {
+            const int r = 32 * h + i / PR, cc = i % PR;
+            if (m0 + r < a.M)
+                *reinterpret_cast<u32x4 *>(a.Y + (size_t)(m0 + r) * D + cc * 8) =
+                    *reinterpret_cast<const u32x4 *>(smem + r * RS + cc * 16);
         }
-        if (arrived != 0) { // (workgroup-uniform)
-            __threadfence();
-            const f32x4 *src =
-                reinterpret_cast<const f32x4 *>(a.ws + ((size_t)(panel * 2 + (1 - half)) * 2 + h) * PART) +
-                (size_t)wave * NB * 2 * 64 + lane;
-            f16x4 x[NB][2];
-#pragma unroll
-            for (int j = 0; j < NB; j++) {
-                const f32x4 bf = __builtin_convertvector(b2[j], f32x4);
-#pragma unroll
-                for (int m2 = 0; m2 < 2; m2++) {
-                    f32x4 other = f32x4{0.f, 0.f, 0.f, 0.f};
-                    f16x4 sk = f16x4{0, 0, 0, 0};
-                    if (j < nvalid) {
-                        other = src[(j * 2 + m2) * 64];
-                        sk = *reinterpret_cast<const f16x4 *>(smem + (16 * (2 * h + m2) + c16) * RS +
-                                                              ((NB * wave + j) * 16 + g4 * 4) * 2);
-                    }
-                    const f32x4 mine = h ? acc[j][2 + m2] : acc[j][m2];
-                    x[j][m2] = __builtin_convertvector((mine + other) + bf, f16x4) + sk;
-                }
-            }
-            tt_ln<D, 2>(x, 2 * h, gam, bet, smem, wave, c16, g4, nvalid);
-            // in place over the skip operand (each lane overwrites what it read), then
-            // whole rows leave with 16-byte stores
-#pragma unroll
-            for (int j = 0; j < NB; j++)
-                if (j < nvalid)
-#pragma unroll
-                    for (int m2 = 0; m2 < 2; m2++)
-                        *reinterpret_cast<f16x4 *>(smem + (16 * (2 * h + m2) + c16) * RS +
-                                                   ((NB * wave + j) * 16 + g4 * 4) * 2) = x[j][m2];
-            __syncthreads();
-            constexpr int PR = D / 8;
-            for (int i = tid; i < 32 * PR; i += TT_WAVES * 64) {
-                const int r = 32 * h + i / PR, c = i % PR;
-                if (m0 + r < a.M)
-                    *reinterpret_cast<u32x4 *>(a.Y + (size_t)(m0 + r) * D + c * 8) =
-                        *reinterpret_cast<const u32x4 *>(smem + r * RS + c * 16);
-            }
-            if (tid == 0) // ready for the next launch
-                __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        __syncthreads(); // misc[] is free again
+        if (tid == 0) // ready for the next launch
+            __hip_atomic_store(a.sync + 2 * panel + h, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+    const int other_h = 1 - half;
+    publish(other_h); // the partner finishes that row-half unless it has long gone
+    __syncthreads();  // (also: every wave has left the hidden buffers)
+    TT_STAMP(7)
+    if (tid == 0) {
+        // one round trip: arrive at the other row-half's counter, look at the own one
+        misc[0] = __hip_atomic_fetch_add(a.sync + 2 * panel + other_h, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        misc[1] = __hip_atomic_load(a.sync + 2 * panel + half, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    __syncthreads();
+    const int arrived_other = misc[0]; // 1: the partner's partial of that row-half was there first: finish it here
+    int arrived_own = misc[1];         // 1: the partner's partial of the own row-half is in scratch
+    if (arrived_own == 0) {
+        // not yet: leave the own partial as well; whoever adds second finishes
+        publish(half);
+        __syncthreads();
+        if (tid == 0)
+            misc[2] = __hip_atomic_fetch_add(a.sync + 2 * panel + half, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        arrived_own = misc[2];
+    }
+    TT_STAMP(8)
+    if (arrived_own != 0)
+        finish(half);
+    if (arrived_other != 0) {
+        __syncthreads(); // (the statistics area and the broadcast words are free again)
+        finish(other_h);
+    }
+    TT_STAMP(9)
 }
 
 // ---------------------------------------------------------------------------
@@ -580,7 +706,7 @@ struct TailProgram {
     int D = 0, Hd = 0;
     int nphase[2] = {0, 0}, hb0[2] = {0, 0}, nb1h[2] = {0, 0};
     f16 *d_pairs = nullptr;
-    int *d_off = nullptr, *d_desc = nullptr, *d_wtab = nullptr, *d_sync = nullptr;
+    int *d_rec = nullptr, *d_wtab = nullptr, *d_sync = nullptr;
     size_t lds_bytes = 0;
     size_t npairs = 0; // including padding (for reports)
 };
@@ -589,14 +715,18 @@ void tail_program_destroy(TailProgram *p) {
     if (!p)
         return;
     et_free(p->d_pairs);
-    et_free(p->d_off);
-    et_free(p->d_desc);
+    et_free(p->d_rec);
     et_free(p->d_wtab);
     et_free(p->d_sync);
     delete p;
 }
 
-static int g_tail_pair = 1;          // et_tuning_set("tile_tail_pair"): 0 never, 1 where it pays, 2 wherever it applies
+#ifdef TT_TRACE
+long long *g_tt_trace = nullptr;
+#endif
+// et_tuning_set("tile_tail_pair"): 0 never (default: at BERT-base / 80 % / 8192 rows the paired form takes 69 us
+// against 55 us of the one-workgroup form), 1 where there are enough panels, 2 wherever it applies
+static int g_tail_pair = 0;
 static int g_tail_spin = 1 << 22;    // et_tuning_set("tile_wait_spin"): polls before a bounded LDS wait gives up
 void set_tail_pair(int v) { g_tail_pair = v; }
 bool tail_pair_forced() { return g_tail_pair >= 2; }
@@ -622,22 +752,13 @@ bool tail_pair_applies(const et_tile_plan *pO, const et_tile_plan *p1, const et_
         Hd % 16)
         return false;
     const int nchunk = (Hd + TT_HC - 1) / TT_HC, per_half = (nchunk + 1) / 2;
-    if (nchunk < 2 || per_half > TT_MAX_PHASES)
+    if (nchunk < 2 || per_half > TT_MAX_PHASES || per_half * TT_HB > 255)
         return false;
     int nb, xw;
     if (!tail_geom(D, &nb, &xw))
         return false;
     const size_t lds = (size_t)TT_BM * (xw + 2 * TT_HW) + 2 * TT_MAX_PHASES * 4 + 128 + (size_t)per_half * TT_HB * 64;
     return lds <= 160 * 1024;
-}
-
-size_t tail_pair_ws_bytes(const et_tile_plan *pO, const et_tile_plan *p1, const et_tile_plan *p2, int M) {
-    if (!tail_pair_applies(pO, p1, p2) || M <= 0)
-        return 0;
-    int nb, xw;
-    tail_geom(pO->out_feat, &nb, &xw);
-    const size_t npanels = ((size_t)M + TT_BM - 1) / TT_BM;
-    return npanels * 4 * ((size_t)TT_WAVES * nb * 2 * 64 * 4) * sizeof(float);
 }
 
 size_t tail_ws_bytes_for(int D, int rows) {
@@ -648,45 +769,75 @@ size_t tail_ws_bytes_for(int D, int rows) {
     return npanels * 4 * ((size_t)TT_WAVES * nb * 2 * 64 * 4) * sizeof(float);
 }
 
+size_t tail_pair_ws_bytes(const et_tile_plan *pO, const et_tile_plan *p1, const et_tile_plan *p2, int M) {
+    if (!tail_pair_applies(pO, p1, p2) || M <= 0)
+        return 0;
+    return tail_ws_bytes_for(pO->out_feat, M);
+}
+
 namespace {
+// one wave's stream while it is being laid out
+struct Segment {
+    int end;                 // pair index inside the stream, exclusive
+    bool hidden;             // a hidden block-row of the first linear
+    int j, slot, p;          // accumulator; slot in the hidden buffer; phase
+    bool wait_store, signal; // wait for S[p - 2] before the hidden store; signal F[p] / S[p] afterwards
+    int init;                // what its sums start from (255: zeros)
+    int wait_p, wait_n;      // before its first operand is read: F[wait_p] has to reach wait_n (wait_p < 0: nothing)
+};
 struct ProgBuilder {
     std::vector<uint16_t> pairs; // 512 halves per pair
-    std::vector<int> off;        // 2 ints per pair
-    std::vector<int> desc;       // TT_DESC ints per segment
-    size_t npairs() const { return off.size() / 2; }
-    int nseg() const { return (int)(desc.size() / TT_DESC); }
+    std::vector<int> rec;        // 4 ints per pair: offset A, control, offset B, control
+    size_t npairs() const { return rec.size() / 4; }
 
     // tiles of block-row bn of plan pl with column in [lo, hi), two per pair
     // (an odd last one gets an all-zero partner at its own offset); returns pairs added
     template <class OffsetOf>
     int add_tiles(const et_tile_plan *pl, int bn, int lo, int hi, OffsetOf &&offset_of) {
         int cnt = 0, last = 0;
+        auto put = [&](int off, const uint16_t *tile) {
+            rec.push_back(off);
+            rec.push_back(0);
+            if (tile)
+                pairs.insert(pairs.end(), tile, tile + 256);
+            else
+                pairs.insert(pairs.end(), 256, (uint16_t)0);
+            cnt++;
+        };
         for (int i = pl->h_row_ptr[bn]; i < pl->h_row_ptr[bn + 1]; i++) {
             const int col = pl->h_col[i];
             if (col < lo || col >= hi)
                 continue;
             last = offset_of(col);
-            off.push_back(last);
-            pairs.insert(pairs.end(), pl->h_data.begin() + (size_t)i * 256, pl->h_data.begin() + (size_t)i * 256 + 256);
-            cnt++;
+            put(last, &pl->h_data[(size_t)i * 256]);
         }
-        if (cnt & 1) {
-            off.push_back(last);
-            pairs.insert(pairs.end(), 256, (uint16_t)0);
-            cnt++;
-        }
+        if (cnt & 1)
+            put(last, nullptr);
         return cnt / 2;
     }
     void add_zero_pair(int offset) {
-        off.push_back(offset);
-        off.push_back(offset);
+        const int r[4] = {offset, 0, offset, 0};
+        rec.insert(rec.end(), r, r + 4);
         pairs.insert(pairs.end(), 512, (uint16_t)0);
     }
-    void add_desc(int end, int kind, int j, int hoff, int init, int wf, int sig) {
-        const int d[TT_DESC] = {end, kind | (j << 8), hoff, init, wf, sig, -1, 0};
-        desc.insert(desc.end(), d, d + TT_DESC);
+    // control words of a finished stream that starts at pair `base`
+    void seal(size_t base, const std::vector<Segment> &segs) {
+        for (size_t i = 0; i < segs.size(); i++) {
+            const Segment &g = segs[i];
+            int ctl = TT_C_SET | (g.hidden ? TT_C_HID : 0) | ((g.hidden ? 7 : g.j) << 2) | (g.slot << 5) | (g.p << 9) |
+                      (g.wait_store ? TT_C_WAITF : 0) | (g.signal ? TT_C_SIG : 0);
+            int next_init = 255;
+            if (i + 1 < segs.size()) {
+                const Segment &nx = segs[i + 1];
+                next_init = nx.init;
+                if (nx.wait_p >= 0)
+                    ctl |= TT_C_WAITN | (nx.wait_p << 16) | ((nx.wait_n - 1) << 20);
+            }
+            ctl |= (int)((unsigned)next_init << 24);
+            const size_t q = base + g.end - 1;
+            rec[q * 4 + 1] = rec[q * 4 + 3] = ctl;
+        }
     }
-    void sentinel(int init) { add_desc(0x7fffffff, 0, 0, 0, init, -1, -1); }
 };
 } // namespace
 
@@ -718,83 +869,62 @@ int tail_pair_prepare(const et_tile_plan *pO, const et_tile_plan *p1, et_tile_pl
     for (int h = 0; h < 2; h++)
         for (int w = 0; w < TT_WAVES; w++) {
             int *wt = &wtab[(h * TT_WAVES + w) * 8];
+            std::vector<Segment> segs;
             // ---- projection: block-rows NB*w .. NB*w + NB - 1 ----
             size_t base = B.npairs();
             wt[0] = (int)base;
-            wt[2] = B.nseg();
-            int segs = 0;
             for (int j = 0; j < NB; j++) {
                 const int bn = NB * w + j;
                 if (bn >= nbrD)
                     continue;
-                if (B.add_tiles(pO, bn, 0, D, [](int col) { return col * 2; }) > 0) {
-                    B.add_desc((int)(B.npairs() - base), 0, j, 0, ZV, -1, -1);
-                    segs++;
-                }
+                if (B.add_tiles(pO, bn, 0, D, [](int col) { return col * 2; }) > 0)
+                    segs.push_back(Segment{(int)(B.npairs() - base), false, j, 0, 0, false, false, 255, -1, 0});
             }
-            if (segs) {
-                while ((B.npairs() - base) % 4)
+            if (!segs.empty()) {
+                while ((B.npairs() - base) % TT_DEPTH)
                     B.add_zero_pair(0);
-                B.desc[B.desc.size() - TT_DESC] = (int)(B.npairs() - base); // the padding belongs to the last segment
+                segs.back().end = (int)(B.npairs() - base); // the padding belongs to the last segment
             }
             wt[1] = (int)(B.npairs() - base);
-            B.sentinel(ZV);
+            B.seal(base, segs);
             // ---- feed-forward: F(0) F(1) S(0) F(2) S(1) ... F(n-1) S(n-2) S(n-1) ----
+            segs.clear();
             base = B.npairs();
-            wt[3] = (int)base;
-            wt[5] = B.nseg();
-            wt[6] = -1;
+            wt[2] = (int)base;
             const int np = P->nphase[h];
-            int last_desc = -1; // index of the stream's latest descriptor
-            auto ctrF = [](int p) { return 4 * p; };
-            auto ctrS = [](int p) { return 4 * (TT_MAX_PHASES + p); };
             auto first = [&](int p) { // F(p): this wave's one or two hidden block-rows of chunk c0 + p
-                // slot s of the chunk's 12 goes to wave (s + 4p) mod 8: four waves have two
-                // block-rows in a phase, and they are the other four in the next one
+                // twelve waves: slot s of the chunk's 12 goes to wave s.  Eight waves: to wave
+                // (s + 4p) mod 8 - four waves have two block-rows in a phase, and they are the
+                // other four in the next one
                 for (int s = 0; s < TT_HB; s++) {
                     const int hb = (c0[h] + p) * TT_HB + s;
-                    if ((s + 4 * p) % TT_WAVES != w || hb >= nbr1)
+                    if ((TT_WAVES == 12 ? s : (s + 4 * p) % TT_WAVES) != w || hb >= nbr1)
                         continue;
                     if (B.add_tiles(p1, hb, 0, D, [](int col) { return col * 2; }) == 0)
                         B.add_zero_pair(0); // bias only: one pair of zeros so that the segment exists
-                    const int wf = p >= 2 ? (ctrS(p - 2) | (TT_WAVES << 16)) : -1;
-                    last_desc = B.nseg();
-                    B.add_desc((int)(B.npairs() - base), 1, 255, XW + (p & 1) * TT_HW + s * 32,
-                               BI + (hb - P->hb0[h]) * 64, wf, ctrF(p));
+                    segs.push_back(Segment{(int)(B.npairs() - base), true, 7, s, p, p >= 2, true, hb - P->hb0[h], -1, 0});
                 }
             };
             auto second = [&](int p) { // S(p): this wave's output block-rows over hidden chunk c0 + p
                 const int c = c0[h] + p, lo = c * TT_HC, hi = std::min(lo + TT_HC, Hd);
                 const int nF = std::min(TT_HB, nbr1 - c * TT_HB); // hidden block-rows of the chunk, each signalled once
-                const int wait = ctrF(p) | (nF << 16);
                 const int hbase = XW + (p & 1) * TT_HW;
-                bool any = false;
-                auto begin_phase = [&]() {
-                    if (any)
-                        return;
-                    any = true;
-                    if (last_desc >= 0)
-                        B.desc[(size_t)last_desc * TT_DESC + 6] = wait;
-                    else
-                        wt[6] = wait;
-                };
+                const size_t nseg0 = segs.size();
                 for (int j = 0; j < NB; j++) {
                     const int bn = NB * w + j;
                     if (bn >= nbrD)
                         continue;
                     if (B.add_tiles(p2, bn, lo, hi, [&](int col) { return hbase + (col - lo) * 2; }) == 0)
                         continue;
-                    begin_phase();
-                    last_desc = B.nseg();
-                    B.add_desc((int)(B.npairs() - base), 0, j, 0, ZV, -1, -1);
+                    segs.push_back(Segment{(int)(B.npairs() - base), false, j, 0, p, false, false, 255, -1, 0});
                 }
-                if (!any) { // nothing of this chunk in the wave's block-rows: the phase still has to be signalled
+                if (segs.size() == nseg0) { // nothing of this chunk in the wave's block-rows: the phase is still signalled
                     B.add_zero_pair(hbase);
-                    begin_phase();
-                    last_desc = B.nseg();
-                    B.add_desc((int)(B.npairs() - base), 0, 0, 0, ZV, -1, -1);
+                    segs.push_back(Segment{(int)(B.npairs() - base), false, 0, 0, p, false, false, 255, -1, 0});
                 }
-                B.desc[(size_t)last_desc * TT_DESC + 5] = ctrS(p); // the phase's last segment signals S[p]
+                segs[nseg0].wait_p = p; // the phase's first segment reads the hidden buffer: F[p] complete
+                segs[nseg0].wait_n = nF;
+                segs.back().signal = true; // its last one signals S[p]
             };
             for (int p = 0; p < np; p++) {
                 if (p == 0)
@@ -803,22 +933,26 @@ int tail_pair_prepare(const et_tile_plan *pO, const et_tile_plan *p1, et_tile_pl
                     first(p + 1);
                 second(p);
             }
-            while ((B.npairs() - base) % 4)
+            while ((B.npairs() - base) % TT_DEPTH)
                 B.add_zero_pair(XW + ((np - 1) & 1) * TT_HW);
-            B.desc[(size_t)last_desc * TT_DESC] = (int)(B.npairs() - base);
-            wt[4] = (int)(B.npairs() - base);
-            B.sentinel(ZV);
+            segs.back().end = (int)(B.npairs() - base);
+            wt[3] = (int)(B.npairs() - base);
+            wt[4] = segs.front().init;
+            wt[5] = segs.front().wait_p >= 0 ? (segs.front().wait_p | (segs.front().wait_n << 8)) : -1;
+            B.seal(base, segs);
         }
-    B.sentinel(ZV); // (a handler reads one descriptor past its stream's sentinel)
     P->npairs = B.npairs();
-    for (int i = 0; i < 8; i++) // the last stages of a stream request up to seven pairs past its end
+    for (int i = 0; i < 2 * TT_DEPTH; i++) // the last stages of a stream request up to TT_DEPTH - 1 pairs past its end
         B.add_zero_pair(0);
     // every offset must address the panel or a hidden buffer of the lane's row
-    for (int v : B.off)
-        if (v < 0 || v + 32 > RS) {
-            tail_program_destroy(P);
-            set_error("layer tail (pairs): internal error, operand offset %d outside the LDS row", v);
-            return ET_ERR_FORMAT;
+    for (size_t q = 0; q < B.npairs(); q++)
+        for (int t = 0; t < 2; t++) {
+            const int v = B.rec[q * 4 + 2 * t];
+            if (v < 0 || v + 32 > RS) {
+                tail_program_destroy(P);
+                set_error("layer tail (pairs): internal error, operand offset %d outside the LDS row", v);
+                return ET_ERR_FORMAT;
+            }
         }
 
     int rc = ET_OK;
@@ -830,8 +964,7 @@ int tail_pair_prepare(const et_tile_plan *pO, const et_tile_plan *p1, et_tile_pl
             rc = et_memcpy_h2d(*dst, hsrc, bytes);
     };
     up((void **)&P->d_pairs, B.pairs.data(), B.pairs.size() * 2);
-    up((void **)&P->d_off, B.off.data(), B.off.size() * 4);
-    up((void **)&P->d_desc, B.desc.data(), B.desc.size() * 4);
+    up((void **)&P->d_rec, B.rec.data(), B.rec.size() * 4);
     up((void **)&P->d_wtab, wtab.data(), wtab.size() * 4);
     const std::vector<int> zeros(2 * TT_MAX_PANELS, 0);
     up((void **)&P->d_sync, zeros.data(), zeros.size() * 4);
@@ -887,8 +1020,7 @@ int tail_pair_launch(const et_tile_plan *pO, const et_tile_plan *p1, const et_ti
     TtArgs a;
     memset(&a, 0, sizeof(a));
     a.pairs = P->d_pairs;
-    a.off = P->d_off;
-    a.desc = P->d_desc;
+    a.rec = P->d_rec;
     a.wtab = P->d_wtab;
     a.attn = attn;
     a.input = input;
@@ -900,7 +1032,7 @@ int tail_pair_launch(const et_tile_plan *pO, const et_tile_plan *p1, const et_ti
     a.b1 = beta1;
     a.g2 = gamma2;
     a.b2 = beta2;
-    a.ws = static_cast<float *>(ws);
+    a.ws = static_cast<unsigned long long *>(ws);
     a.sync = P->d_sync;
     a.status = status;
     a.M = M;
@@ -911,6 +1043,15 @@ int tail_pair_launch(const et_tile_plan *pO, const et_tile_plan *p1, const et_ti
         a.hb0[h] = P->hb0[h];
         a.nb1h[h] = P->nb1h[h];
     }
+#ifdef TT_TRACE
+    {
+        static long long *trace = nullptr;
+        if (!trace)
+            (void)hipMalloc(&trace, (size_t)4096 * TT_WAVES * 16 * 8);
+        a.trace = trace;
+        g_tt_trace = trace;
+    }
+#endif
     switch (P->D) {
     case 768: return tt_launch<768>(a, P->lds_bytes, st);
     case 512: return tt_launch<512>(a, P->lds_bytes, st);
@@ -922,3 +1063,8 @@ int tail_pair_launch(const et_tile_plan *pO, const et_tile_plan *p1, const et_ti
 }
 
 } // namespace et
+#ifdef TT_TRACE
+extern "C" int et_tt_trace_read(long long *host, int nwg) {
+    return hipMemcpy(host, et::g_tt_trace, (size_t)nwg * et::TT_WAVES * 16 * 8, hipMemcpyDeviceToHost) == hipSuccess ? 0 : -1;
+}
+#endif

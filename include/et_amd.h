@@ -266,7 +266,8 @@ int et_tile_plan_tail_fusable(const et_tile_plan *out, const et_tile_plan *first
  * one half of the hidden columns of the feed-forward block, and their fp32
  * partial sums meet in `ws` (whoever arrives second at a row-half's counter
  * finishes it: no workgroup waits for another).  A CU then streams half the
- * weights per row.  Taken where it applies (model width 256, 512 or 768, hidden
+ * weights per row.  Taken only when switched on (et_tuning_set
+ * "tile_tail_pair"), where it applies (model width 256, 512 or 768, hidden
  * width a multiple of 16 and at least 384), ws_bytes >=
  * et_tile_plan_tail_ws_bytes(out, first, second, M) and there are enough row
  * panels to fill the device; otherwise this is et_tile_plan_run_tail.  ws must
@@ -452,8 +453,10 @@ int et_device_synchronize(void);
  *   "attn_packed"     0: et_OTF_attention_varlen launches one workgroup per
  *                     possible query block; 1 (default): workgroups walk the
  *                     blocks that exist (up to 256 sequences)
- *   "tile_tail_pair"  0: et_tile_plan_run_tail_ws never takes the paired form;
- *                     1 (default): where it applies and pays; 2: wherever it applies
+ *   "tile_tail_pair"  0 (default): et_tile_plan_run_tail_ws never takes the paired
+ *                     form (measured slower than the one-workgroup form on the
+ *                     BERT-base shapes); 1: where it applies and there are
+ *                     enough row panels; 2: wherever it applies
  *   "tile_tail_pair_min_wgs" fewest workgroups (two per 64-row panel) for the
  *                     paired form (default: three quarters of the CUs)
  *   "tile_wait_spin"  polls after which a bounded wait inside a workgroup gives

@@ -323,19 +323,25 @@ def test_tile_layer_tail_pairs(K, M, d, F, sp):
     want = orc.skip_layernorm(y, mid, g2, b2)
     mk = lambda l, K_, N_, gelu: Linear_tile(K_, N_, M, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], gelu)
     to, t1, t2 = mk(lo, d, d, False), mk(l1, d, F, True), mk(l2, F, d, False)
-    need = Linear_tile.tail_ws_bytes(to, t1, t2, M)
-    assert need == ((M + 63) // 64) * 64 * (-(-d // 128) * 128) * 4 * 2
-    Linear_tile.tail_prepare(to, t1, t2)
-    ws = torch.full((need,), 0xFF, dtype=torch.uint8, device="cuda")   # NaN patterns: nothing may be read before written
+    from et_amd import lib
     ln = [dev(t) for t in (g1, b1, g2, b2)]
-    print(f"pair tail: M={M} d={d} F={F} sp={sp}", flush=True)
-    got = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln, ws=ws))
-    check_close(got, want, max_abs=3e-2, mean_rel=2e-3, what="paired layer tail vs oracle chain")
-    again = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln, ws=ws))
-    assert np.array_equal(got, again)
-    ad = dev(attn)
-    Linear_tile.run_tail(to, t1, t2, ad, dev(inp), *ln, out=ad, ws=ws)
-    assert np.array_equal(host(ad), got)
+    assert Linear_tile.tail_ws_bytes(to, t1, t2, M) == 0          # the paired form is off by default
+    lib().et_tuning_set(b"tile_tail_pair", 2)
+    try:
+        need = Linear_tile.tail_ws_bytes(to, t1, t2, M)
+        assert need == ((M + 63) // 64) * 64 * (-(-d // 192) * 192) * 4 * 2   # twelve waves x block-rows per wave x 16 columns
+        Linear_tile.tail_prepare(to, t1, t2)
+        ws = torch.full((need,), 0xFF, dtype=torch.uint8, device="cuda")   # NaN patterns: nothing may be read before written
+        print(f"pair tail: M={M} d={d} F={F} sp={sp}", flush=True)
+        got = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln, ws=ws))
+        check_close(got, want, max_abs=3e-2, mean_rel=2e-3, what="paired layer tail vs oracle chain")
+        again = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln, ws=ws))
+        assert np.array_equal(got, again)
+        ad = dev(attn)
+        Linear_tile.run_tail(to, t1, t2, ad, dev(inp), *ln, out=ad, ws=ws)
+        assert np.array_equal(host(ad), got)
+    finally:
+        lib().et_tuning_set(b"tile_tail_pair", 0)
     if Linear_tile.tail_fusable(to, t1, t2):
         one = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln))
         assert np.abs(got.astype(np.float32) - one.astype(np.float32)).max() <= 3e-2
