@@ -48,6 +48,8 @@ PROTOTYPES = {
     "et_tile_plan_tail_prepare": (_i, [_vp, _vp, _vp]),
     "et_tile_plan_tail_ws_bytes": (_sz, [_vp, _vp, _vp, _i]),
     "et_tail_ws_bytes_for": (_sz, [_i, _i]),
+    "et_wait_status_take": (_i, []),
+    "et_wait_status_raise_for_test": (None, []),
     "et_tile_plan_run_multi": (_i, [C.POINTER(_vp), C.POINTER(_vp), _i, _vp, _i, _vp]),
     "et_tile_plan_query": (_i, [_vp, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
     "et_prune_tile_mat": (_i, [_vp, _i, _i, _f, _ip, _ip]),

@@ -46,6 +46,12 @@ struct AttnArgs {
     const unsigned *msum;
     int msum_words;
     int ldq, ldv, ldo, seq_len, nhead, batch, nqb, total, per_xcd;
+    // columns per head in Q, K, V and the output where that is not the kernel's
+    // HD (any multiple of 16 below it; the register-staged kernel only): 0 = HD
+    int head_width;
+    // columns per head in Q and K where they are narrower than the head (compact Q / K with the same number of
+    // kept columns in every head; register-staged kernel): 0 = the head's width
+    int qk_width;
     float log2_scale, scale;
 };
 
@@ -190,6 +196,17 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
         return;
 
     int qc0 = h * HDK, nqk = HD, vc0 = h * HD, nv = HD;
+    // head width of the data (HD unless the launcher says otherwise: heads of 48,
+    // 80, 96 ... columns run as ragged heads of the next built width)
+    const int hw = (PRUNED && !VWIN && a.head_width) ? a.head_width : HD;
+    if (PRUNED && !VWIN && a.head_width) {
+        qc0 = vc0 = h * hw;
+        nqk = nv = hw;
+    }
+    if (PRUNED && !VWIN && a.qk_width) {
+        qc0 = h * a.qk_width;
+        nqk = a.qk_width;
+    }
     if (PRUNED) {
         if (a.qk_head_ptr) {
             qc0 = a.qk_head_ptr[h];
@@ -219,7 +236,7 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
     const int lane = tid & 63;
     const int c16 = lane & 15;
     const int g4 = lane >> 4;
-    f16 *obase = a.out + (size_t)row0 * a.ldo + h * HD;
+    f16 *obase = a.out + (size_t)row0 * a.ldo + h * hw;
     const f16x8 zero8 = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
 
     if (q0 < len) {
@@ -833,8 +850,8 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
                     for (int r = 0; r < 4; r++) {
                         const int j = d * 16 + g4 * 4 + r;
                         if (j < nv) {
-                            const int col = (a.v_col_id ? a.v_col_id[vc0 + j] : vc0 + j) - h * HD;
-                            if (col >= 0 && col < HD)
+                            const int col = (a.v_col_id ? a.v_col_id[vc0 + j] : vc0 + j) - h * hw;
+                            if (col >= 0 && col < hw)
                                 os[ql * LDO + col] = o[r];
                         }
                     }
@@ -847,7 +864,7 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
         for (int idx = tid; idx < QB * CPR; idx += AT_THREADS) {
             const int ql = idx / CPR, dc = idx % CPR;
             const int q = q0 + ql;
-            if (q < rows_alloc) {
+            if (q < rows_alloc && dc * 8 < hw) {
                 f16x8 v = zero8;
                 if (q < len)
                     v = *reinterpret_cast<const f16x8 *>(os + ql * LDO + dc * 8);
@@ -860,7 +877,7 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
         for (int idx = tid; idx < QB * CPR; idx += AT_THREADS) {
             const int ql = idx / CPR, dc = idx % CPR;
             const int q = q0 + ql;
-            if (q < rows_alloc)
+            if (q < rows_alloc && dc * 8 < hw)
                 *reinterpret_cast<f16x8 *>(obase + (size_t)q * a.ldo + dc * 8) = zero8;
         }
     }
@@ -1167,9 +1184,22 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
     ET_REQUIRE(a.seq_len > 0 && d_model > 0 && a.nhead > 0 && a.batch > 0, ET_ERR_INVALID_ARG,
                "%s: seq_len=%d d_model=%d nhead=%d batch=%d", who, a.seq_len, d_model, a.nhead, a.batch);
     ET_REQUIRE(d_model % a.nhead == 0, ET_ERR_INVALID_ARG, "%s: d_model %% nhead != 0", who);
-    const int hd = d_model / a.nhead;
-    ET_REQUIRE(hd == 32 || hd == 64 || hd == 128, ET_ERR_UNSUPPORTED,
-               "%s: head_dim %d not in {32,64,128}", who, hd);
+    const int hd_data = d_model / a.nhead;
+    // Kernels are built for heads of 32, 64 and 128 columns.  Any other multiple
+    // of 16 up to 128 (the reference loops over head_dim in steps of 16,
+    // kernels/attention.cu:86-90) runs on the register-staged kernel of the next
+    // built width as ragged heads: it reads the columns beyond a head's end as
+    // zeros and writes none of them.
+    const bool odd_width = !(hd_data == 32 || hd_data == 64 || hd_data == 128);
+    ET_REQUIRE(!odd_width || (hd_data % 16 == 0 && hd_data > 0 && hd_data < 128 && !sharedqk && !a.qk_head_ptr &&
+                              !a.v_head_ptr && !a.cu_seqlens),
+               ET_ERR_UNSUPPORTED,
+               "%s: head_dim %d: multiples of 16 up to 128 (dense heads, padded batches) or 32 / 64 / 128", who, hd_data);
+    const int hd = !odd_width ? hd_data : hd_data < 32 ? 32 : hd_data < 64 ? 64 : 128;
+    if (odd_width) {
+        pruned = true;
+        a.head_width = hd_data;
+    }
     ET_REQUIRE(aligned16(a.out) && aligned16(a.Q) && aligned16(a.K) && aligned16(a.V),
                ET_ERR_ALIGNMENT, "%s: out/Q/K/V must be 16-byte aligned", who);
     if (!pruned) {
@@ -1177,7 +1207,7 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
                    "%s: d_model must be a multiple of 8", who);
     }
     a.ldo = d_model;
-    a.scale = head_scale(hd);
+    a.scale = head_scale(hd_data);
     bool no_mask;
     if (given_summary && a.mask) {
         a.msum = given_summary;
@@ -1211,11 +1241,18 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
         else if (pruned) attn_launch_variant<HDV, true, false>(variant, false, a, st);                  \
         else attn_launch_variant<HDV, false, false>(variant, plain, a, st);                             \
     }
-    if (qk_width && qk_width != hd) {
-        ET_REQUIRE(hd == 64 && qk_width == 32 && !pruned && !sharedqk, ET_ERR_UNSUPPORTED,
-                   "%s: %d of %d columns per head in Q and K is not built (32 of 64 is)", who, qk_width, hd);
-        attn_launch_variant<64, false, false, 32>(variant, plain, a, st);
-        return launch_status(who);
+    if (qk_width && qk_width != hd_data) {
+        ET_REQUIRE(qk_width > 0 && qk_width < hd_data && qk_width % 16 == 0 && !sharedqk && !a.qk_head_ptr &&
+                       !a.v_head_ptr && !a.cu_seqlens,
+                   ET_ERR_UNSUPPORTED, "%s: %d of %d columns per head in Q and K: a multiple of 16 below the head width",
+                   who, qk_width, hd_data);
+        if (hd == 64 && qk_width == 32 && !pruned) { // the DMA-staged kernel with a 32-wide K tile
+            attn_launch_variant<64, false, false, 32>(variant, plain, a, st);
+            return launch_status(who);
+        }
+        // any other width: ragged heads on the register-staged kernel
+        pruned = true;
+        a.qk_width = qk_width;
     }
     // packed sequences: the grid the chip holds, every workgroup walks its share of the query blocks that exist
     if (a.cu_seqlens && !pruned && !sharedqk && variant == 2 && a.batch <= 64 * AT_PX && g_attn_packed) {

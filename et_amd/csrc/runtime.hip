@@ -26,6 +26,7 @@ int hip_fail(hipError_t e, const char *what) {
 // once per process (by the first plan that is created, never inside a run).
 static int *g_status_host = nullptr, *g_status_dev = nullptr;
 static bool g_status_tried = false;
+static int g_status_local = 0; // stands in where there is no device (the host-side plumbing can still be exercised)
 static void status_init() {
     if (g_status_tried)
         return;
@@ -33,12 +34,14 @@ static void status_init() {
     void *h = nullptr, *d = nullptr;
     if (hipHostMalloc(&h, 64, hipHostMallocMapped) != hipSuccess) {
         (void)hipGetLastError();
+        g_status_host = &g_status_local;
         return;
     }
     memset(h, 0, 64);
     if (hipHostGetDevicePointer(&d, h, 0) != hipSuccess) {
         (void)hipGetLastError();
         (void)hipHostFree(h);
+        g_status_host = &g_status_local;
         return;
     }
     g_status_host = static_cast<int *>(h);
@@ -143,6 +146,12 @@ const char *et_strerror(int code) {
 }
 
 const char *et_last_error(void) { return et::g_err; }
+int et_wait_status_take(void) { return et::check_wait_status("et_wait_status_take"); }
+void et_wait_status_raise_for_test(void) {
+    volatile int *h = et::wait_status_host();
+    if (h)
+        *h = 1;
+}
 int et_abi_version(void) { return 2; } // 2: the container loaders take the expected sizes
 
 int et_malloc(void **ptr, size_t bytes) {

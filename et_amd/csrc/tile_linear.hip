@@ -93,6 +93,8 @@ struct TlArgs {
     // fused skip + LayerNorm epilogue (plan kernels with LN = true)
     const f16 *skip, *gamma, *beta;
     const f16 *gamma2, *beta2; // second LayerNorm of the fused layer tail
+    int *status;               // fused feed-forward kernels: set when a bounded LDS wait gives up
+    int spin;                  // ... after this many polls
 };
 #define TL_SEL(f) (lin == 0 ? a.f[0] : lin == 1 ? a.f[1] : lin == 2 ? a.f[2] : a.f[3])
 
@@ -1122,15 +1124,22 @@ __device__ __forceinline__ void tl_signal(unsigned *ctr, int lane) {
     if (lane == 0)
         __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
-// The wait is bounded (about 4 million polls, tens of milliseconds): should a
-// wave ever fail to signal, the kernel ends with a wrong result instead of
-// hanging the GPU.  Every launch site checks on the host that the phase count
-// fits the counters (tile_launch_ffn).
-__device__ __forceinline__ void tl_wait_count(unsigned *ctr, unsigned target) {
-    for (int spin = 0; spin < (1 << 22); spin++) {
+// The wait is bounded (about 4 million polls by default, tens of milliseconds):
+// should a wave ever fail to signal, the waiting wave sets the process's
+// wait-status word and goes on - the kernel ends with a wrong result instead of
+// hanging the GPU, and the next launch of a fused kernel reports ET_ERR_HIP.
+// Every launch site checks on the host that the phase count fits the counters
+// (tile_launch_ffn).
+__device__ __forceinline__ void tl_wait_count(unsigned *ctr, unsigned target, int spin, int *status, int lane) {
+    for (int s = 0;; s++) {
         if ((unsigned)__builtin_amdgcn_readfirstlane(
                 (int)__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) >= target)
             break;
+        if (s >= spin) {
+            if (lane == 0)
+                __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            break;
+        }
         __builtin_amdgcn_s_sleep(1);
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -1319,7 +1328,7 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
         if (fq >= 1 && fq < a.nchunk) {
             const int bvecF2 = TL_FFN_BVEC1(min(fq + 1, a.nchunk - 1)); // (scalar loads, used after the stream)
             if (fq >= 2) // F(fq) overwrites the buffer that S(fq-2) read
-                tl_wait_count(ctr + TL_FFN_MAX_PHASES + fq - 2, NW);
+                tl_wait_count(ctr + TL_FFN_MAX_PHASES + fq - 2, NW, a.spin, a.status, lane);
             TL_FFN_FIRST(fq, bvecFn, b1n, wB, oB)
             bvecFn = bvecF2;
             if (fq + 1 < a.nchunk) { // F(fq+1), a stream (or two) ahead
@@ -1327,7 +1336,7 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
                 TL_FFN_BIAS1(b1n, fq + 1)
             }
         }
-        tl_wait_count(ctr + p, NW); // hidden buffer p & 1 is complete
+        tl_wait_count(ctr + p, NW, a.spin, a.status, lane); // hidden buffer p & 1 is complete
         {
             const char *const xlane2 =
                 reinterpret_cast<const char *>(hs + (p & 1) * hbuf + c16 * ldh + x.khalf8);
@@ -1692,8 +1701,18 @@ static int tile_launch_ffn(const TlProblem *pO, const TlProblem &p1, const TlPro
     // the kernel's LDS event counters cover TL_FFN_MAX_PHASES phases: every launch passes through here
     ET_REQUIRE(nchunk2 >= 1 && nchunk2 <= TL_FFN_MAX_PHASES, ET_ERR_UNSUPPORTED,
                "fused feed-forward: %d phases, the kernel covers %d", nchunk2, TL_FFN_MAX_PHASES);
+    // a wave of an earlier launch that gave up an LDS wait left a wrong result behind: say so once
+    int *const status = wait_status_device();
+    ET_REQUIRE(status, ET_ERR_HIP, "fused feed-forward: no wait-status word");
+    {
+        const int rc = check_wait_status("fused feed-forward");
+        if (rc != ET_OK)
+            return rc;
+    }
     TlArgs a;
     memset(&a, 0, sizeof(a));
+    a.status = status;
+    a.spin = tail_spin();
     const TlProblem *ps[3] = {pO ? pO : &p1, pO ? &p1 : &p2, &p2};
     for (int i = 0; i < TL_MAX_LIN; i++) {
         const TlProblem &p = *ps[std::min(i, 2)];

@@ -90,7 +90,11 @@ int et_row_spmm_prefers_gemm(int M, int N, int K);
 
 /* Replaces OTF_attention_kernelLauncher (kernels/kernels.h:22-24,
  * kernels/attention.cu:122-134).  out, Q, K, V are [batch*seq_len x d_model];
- * head h owns columns h*hd..(h+1)*hd-1, hd = d_model/nhead in {32,64,128}.
+ * head h owns columns h*hd..(h+1)*hd-1, hd = d_model/nhead a multiple of 16
+ * up to 128 (the reference walks the head in steps of 16,
+ * kernels/attention.cu:86-90); 32, 64 and 128 have kernels of their own, the
+ * other widths run as ragged heads on the register-staged kernel of the next
+ * of these (padded batches only: not through et_OTF_attention_varlen).
  * Z = softmax((Q*scale) K^T + mask) V per head without writing the score
  * matrix to memory; scale = half(sqrt(1/hd)) applied to Q in half; mask is
  * one additive [seq_len x seq_len] half matrix shared by heads and batch, or
@@ -144,8 +148,9 @@ int et_OTF_attention_noalloc(void *out, const void *Q, const void *K,
  * h*qk_width, the scores contract over qk_width and are scaled by
  * half(1/sqrt(head_dim)) as before; V and out keep d_model columns.  Same
  * result as et_Prune_attention with qk_head_ptr[h] = h*qk_width, through the
- * faster on-the-fly kernel.  Built for qk_width 32 with head_dim 64
- * (ET_ERR_UNSUPPORTED otherwise).  No counterpart in the reference, whose
+ * on-the-fly kernel: the DMA-staged one for qk_width 32 with head_dim 64, the
+ * register-staged one for any other multiple of 16 below head_dim.  No
+ * counterpart in the reference, whose
  * Prune_attention (kernels/kernels.h:26-30) prunes V only. */
 int et_OTF_attention_qk_width(void *out, const void *Q, const void *K,
                               const void *V, const void *mask, int qk_width,
@@ -484,6 +489,16 @@ int et_tuning_set(const char *key, int value);
  *           units = v_mfma_f32_16x16x32_f16 per MFMA-issuing wave.
  * seconds = duration of one launch on every CU of the device. */
 int et_microbench(int what, int p0, int p1, double *seconds, double *units_per_cu);
+/* The fused layer-tail kernels order their waves with bounded waits on LDS
+ * counters.  A wave that gives up (it never should) sets one status word per
+ * process and goes on, so the kernel ends - with a wrong result - instead of
+ * hanging the GPU; the next launch of such a kernel returns ET_ERR_HIP once and
+ * clears the word.  et_wait_status_take does the same check on demand (ET_OK or
+ * ET_ERR_HIP); et_wait_status_raise_for_test sets the word from the host, which
+ * is how the report is tested without a wave ever missing a signal.  No
+ * counterpart in the reference, which has no kernel that waits. */
+int et_wait_status_take(void);
+void et_wait_status_raise_for_test(void);
 /* number of compute units of the current device (0 if none) */
 int et_device_cu_count(void);
 

@@ -280,3 +280,16 @@ def test_value_window_pieces_stay_inside_their_row(keep):
     ldv = (int(hp[-1]) + 7) // 8 * 8
     for h, row, col in vwin_window_model(hp, ldv):
         assert 0 <= col and col + 8 <= ldv, (h, row, col, ldv)
+
+
+def test_wait_status_word_is_reported_once_and_cleared():
+    """the status word that a fused kernel's bounded wait sets: raised from the host here (no device needed),
+    the next check returns ET_ERR_HIP with a message, the one after that is clean again"""
+    l = _lib.lib()
+    assert l.et_wait_status_take() == 0
+    l.et_wait_status_raise_for_test()
+    rc = l.et_wait_status_take()
+    assert rc < 0 and l.et_strerror(rc) == b"HIP runtime error"
+    assert b"gave up a bounded wait" in l.et_last_error()
+    assert l.et_wait_status_take() == 0
+

@@ -348,6 +348,46 @@ def test_tile_layer_tail_pairs(K, M, d, F, sp):
         assert (got != one).mean() < 0.05
 
 
+@pytest.mark.parametrize("paired", [False, True])
+def test_fused_tail_reports_a_wait_that_gave_up(K, paired):
+    """with a poll limit of zero every bounded LDS wait of the fused layer-tail kernels gives up at once (no wave
+    ever misses a signal: the kernels run to their normal end, only without waiting), the status word is set, and
+    the NEXT launch of such a kernel returns ET_ERR_HIP once; afterwards the kernels work as before"""
+    from et_amd import lib
+    from et_amd._lib import EtError
+    from et_amd.encoder import Linear_tile
+    M, d, F, sp = 256, 768, 3072, 0.8
+    r = rng(8800 + paired)
+    lo = make_tile_linear(r, d, d, sp, seed=31, std=0.05, bias_std=0.2)
+    l1 = make_tile_linear(r, F, d, sp, seed=32, std=0.05, bias_std=0.2)
+    l2 = make_tile_linear(r, d, F, sp, seed=33, std=0.05, bias_std=0.2)
+    attn, inp = randn_h(r, (M, d)), randn_h(r, (M, d))
+    ln = [dev(np.ones(d, np.float16)), dev(np.zeros(d, np.float16))] * 2
+    mk = lambda l, K_, N_, gelu: Linear_tile(K_, N_, M, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], gelu)
+    to, t1, t2 = mk(lo, d, d, False), mk(l1, d, F, True), mk(l2, F, d, False)
+    lib().et_tuning_set(b"tile_tail_pair", 2 if paired else 0)
+    ws = None
+    try:
+        if paired:
+            Linear_tile.tail_prepare(to, t1, t2)
+            ws = torch.zeros(Linear_tile.tail_ws_bytes(to, t1, t2, M), dtype=torch.uint8, device="cuda")
+        run = lambda: host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln, ws=ws))
+        good = run()
+        assert lib().et_wait_status_take() == 0
+        lib().et_tuning_set(b"tile_wait_spin", 0)
+        print(f"zero-poll launch, paired={paired}", flush=True)
+        run()                                   # ends normally; its waves did not wait for each other
+        lib().et_tuning_set(b"tile_wait_spin", -1)
+        with pytest.raises(EtError) as e:
+            run()
+        assert "gave up a bounded wait" in str(e.value)
+        assert np.array_equal(run(), good)      # reported once; the kernels are fine
+    finally:
+        lib().et_tuning_set(b"tile_wait_spin", -1)
+        lib().et_tuning_set(b"tile_tail_pair", 0)
+        lib().et_wait_status_take()
+
+
 def test_tile_layer_tail_splits_off_a_small_last_round(K):
     """one workgroup per CU and 32-row panel: a last round of few panels runs step by step behind the fused launch"""
     from et_amd import lib
@@ -595,6 +635,31 @@ def test_otf_attention(K, S, H, d, B, lens, use_mask, ls):
     got = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), None if mask is None else dev(mask), S, H, B,
                                None if lens is None else dev(lens_np), ls))
     check_close(got, want, max_abs=5e-3, mean_rel=1e-3, what="OTF attention")
+    if lens is not None:
+        for b, L in enumerate(lens):
+            assert (got[b * S + L:(b + 1) * S] == 0).all()
+
+
+@pytest.mark.parametrize("S,H,d,B,lens,use_mask,ls", [
+    (256, 8, 768, 2, None, False, 1.0),          # head_dim 96, the reference's `tile_test 8 768` shape
+    (200, 8, 768, 2, [200, 77], True, LOG2E),
+    (128, 8, 384, 1, None, True, 1.0),           # head_dim 48
+    (96, 3, 240, 3, [96, 1, 50], True, 1.0),     # head_dim 80
+    (64, 2, 224, 1, None, False, 1.0),           # head_dim 112
+    (80, 4, 64, 2, [80, 33], True, 1.0),         # head_dim 16
+])
+def test_otf_attention_other_head_widths(K, S, H, d, B, lens, use_mask, ls):
+    """head widths that are multiples of 16 but none of 32 / 64 / 128 (the reference loops over head_dim in steps
+    of 16, kernels/attention.cu:86-90) == the oracle; the neighbouring heads' output columns are not touched"""
+    r = rng(4400 + S + H + d)
+    Q, Kk, V = (randn_h(r, (B * S, d)) for _ in range(3))
+    mask = randn_h(r, (S, S)) if use_mask else None
+    lens_np = None if lens is None else np.array(lens, np.int32)
+    want = orc.otf_attention(Q, Kk, V, mask, S, H, B, lens_np, ls, f64=True)
+    print(f"attention head_dim {d // H}: S={S} H={H} B={B}", flush=True)
+    got = host(K.OTF_attention(dev(Q), dev(Kk), dev(V), None if mask is None else dev(mask), S, H, B,
+                               None if lens is None else dev(lens_np), ls))
+    check_close(got, want, max_abs=5e-3, mean_rel=1e-3, what="OTF attention, other head widths")
     if lens is not None:
         for b, L in enumerate(lens):
             assert (got[b * S + L:(b + 1) * S] == 0).all()
@@ -892,8 +957,14 @@ def test_otf_attention_narrow_qk_heads(K, S, B, with_mask, with_lens):
     check_close(got[valid], want[valid], max_abs=5e-3, mean_rel=1e-3, what="narrow Q/K heads")
     check_close(got[valid], other[valid], max_abs=2e-3, mean_rel=1e-3, what="narrow Q/K heads vs pruned kernel")
     assert (got[~valid] == 0).all()
-    with pytest.raises(Exception):   # only 32 of 64 is built
-        K.OTF_attention_qk_width(dev(Qc[:, :192]), dev(Kc[:, :192]), dev(V), md, 16, S, H, B, ld)
+    # another width (16 of 64) runs on the register-staged kernel: == the oracle on the narrower column set
+    qk16 = orc.gen_head_balanced_rows(H, hd, 16, seed=3)
+    Q16, K16 = np.ascontiguousarray(Q[:, qk16]), np.ascontiguousarray(Kk[:, qk16])
+    want16 = orc.prune_attention(Q16, K16, V, orc.head_ptr(qk16, H, hd), None, None, mask, S, d, H, B, lens, f64=True)
+    got16 = host(K.OTF_attention_qk_width(dev(Q16), dev(K16), dev(V), md, 16, S, H, B, ld))
+    check_close(got16[valid], want16[valid], max_abs=5e-3, mean_rel=1e-3, what="narrow Q/K heads, 16 of 64")
+    with pytest.raises(Exception):   # not a multiple of 16
+        K.OTF_attention_qk_width(dev(Qc[:, :96]), dev(Kc[:, :96]), dev(V), md, 8, S, H, B, ld)
 
 
 def test_sharedqk_attention_and_scores(K):
