@@ -26,7 +26,6 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 MFMA_F16_PEAK_TF = 2500.0   # MI355X dense fp16 MFMA, published
@@ -84,7 +83,7 @@ def product_tile_linear(r, N, K, sparsity, seed, std=0.02):
     """dense W ~ N(0, std) -> seeded tile_mat through the library's own generator and packer
     (et_gen_sparse_tile_mat / et_tile_pack); same dictionary as tests/helpers.make_tile_linear"""
     from et_amd import formats
-    from helpers import randn_h
+    from et_amd.synthetic import randn_h
     W = randn_h(r, (N, K), std)
     row_ptr, row_offset = formats.gen_sparse_tile_mat(N, K, sparsity, seed)
     return dict(W=W, row_ptr=row_ptr, row_offset=row_offset, data=formats.tile_pack(W, row_ptr, row_offset),
@@ -125,7 +124,7 @@ def main():
     import oracle.et_oracle as orc          # checker / CPU baseline only
     from et_amd import kernels as K
     from et_amd.encoder import Encoder_tile, Linear_tile, run_multi
-    from helpers import randn_h, rng
+    from et_amd.synthetic import randn_h, rng
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
@@ -328,10 +327,18 @@ def run_micro():
     MFMA-only loop implies (a v_mfma_f32_16x16x32_f16 occupies its SIMD's matrix unit for 16 cycles)."""
     import ctypes as C
     from et_amd._lib import check, lib
+    from et_amd.build import MICROBENCH_LIB
+
+    lib()                                        # (the microbenchmark library links against the main one)
+    if not os.path.exists(MICROBENCH_LIB):
+        raise ImportError(f"{MICROBENCH_LIB} is missing: build it with `python -m et_amd.build`")
+    mbl = C.CDLL(MICROBENCH_LIB)
+    mbl.et_microbench.restype = C.c_int
+    mbl.et_microbench.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
 
     def mb(what, p0, p1):
         sec, units = C.c_double(), C.c_double()
-        check(lib().et_microbench(what, p0, p1, C.byref(sec), C.byref(units)))
+        check(mbl.et_microbench(what, p0, p1, C.byref(sec), C.byref(units)))
         return sec.value, units.value
 
     res = {}
@@ -381,7 +388,7 @@ def second_targets(torch, K, dev, enc, out, x, B, S, mask_h, lins, ln):
     operands beyond the 256 MB last-level cache (an HBM figure, not a cache figure), BASELINE config 1
     (dense layer, batch 1 x seq 128) and the headline layer with a padding mask instead of the all-zero one."""
     from et_amd.encoder import Encoder_tile, Linear_tile
-    from helpers import randn_h, rng
+    from et_amd.synthetic import randn_h, rng
     res = {}
     rows = 131072
     gam = torch.ones(D, dtype=torch.float16, device=dev)
@@ -434,7 +441,7 @@ def second_targets(torch, K, dev, enc, out, x, B, S, mask_h, lins, ln):
 def run_extras(torch, orc, K, dev):
     """Other BASELINE configurations, timed with HIP events (reported, not the headline)."""
     from et_amd.encoder import Encoder_tile, Linear_tile
-    from helpers import randn_h, rng
+    from et_amd.synthetic import randn_h, rng
     out = {}
 
     def timeit(fn, reps=100, warm=10):

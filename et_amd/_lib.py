@@ -26,6 +26,7 @@ PROTOTYPES = {
     "et_row_spmm_add_bias_multi": (_i, [C.POINTER(_vp), _vp, C.POINTER(_vp), C.POINTER(_vp), _ip, _i, _i, _i, _vp]),
     "et_row_spmm_prefers_gemm": (_i, [_i, _i, _i]),
     "et_OTF_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _ip, _f, _vp]),
+    "et_OTF_attention_summary": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _ip, _f, _vp]),
     "et_OTF_attention_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _ip, _f, _vp]),
     "et_attention_mask_summary_bytes": (C.c_size_t, [_i]),
     "et_attention_mask_summary": (_i, [_vp, _i, _vp, _vp]),
@@ -117,7 +118,6 @@ PROTOTYPES = {
     "et_stream_synchronize": (_i, [_vp]),
     "et_device_synchronize": (_i, []),
     "et_device_cu_count": (_i, []),
-    "et_microbench": (_i, [_i, _i, _i, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "et_tuning_set": (_i, [C.c_char_p, _i]),
 }
 

@@ -1,5 +1,6 @@
 // Microbenchmarks of the three delivery paths that bound the tile kernels and
-// the attention kernel on gfx950, callable through the C ABI (bench.py --micro):
+// the attention kernel on gfx950.  A library of its own (libet_microbench.so, next to
+// this file; it is not part of the encoder's C ABI), loaded by bench.py --micro:
 //   * LDS fragment reads (ds_read_b128 in the X-panel / K-tile access pattern),
 //   * the weight stream (global_load_dwordx4, one kilobyte per wave request,
 //     from a buffer that stays in L2),
@@ -9,7 +10,7 @@
 // into bytes / instructions per nanosecond and CU by the caller.  The matrix
 // unit's own loop (16 cycles per v_mfma_f32_16x16x32_f16 and SIMD) gives the
 // clock that the other figures are quoted against.
-#include "common.h"
+#include "../csrc/common.h"
 
 namespace et {
 
@@ -129,65 +130,93 @@ __global__ void __launch_bounds__(1024) mb_coexec_kernel(float *out, int iters) 
 
 template <class Launch>
 static int mb_time(Launch launch, double *seconds) {
-    hipEvent_t e0, e1;
-    ET_HIP(hipEventCreate(&e0));
-    ET_HIP(hipEventCreate(&e1));
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t err = hipEventCreate(&e0);
+    if (err == hipSuccess)
+        err = hipEventCreate(&e1);
     float ms = 0.f;
-    for (int rep = 0; rep < 3; rep++) { // the last of three launches counts
-        ET_HIP(hipEventRecord(e0, nullptr));
+    for (int rep = 0; rep < 3 && err == hipSuccess; rep++) { // the last of three launches counts
+        err = hipEventRecord(e0, nullptr);
+        if (err != hipSuccess)
+            break;
         launch();
-        ET_HIP(hipEventRecord(e1, nullptr));
-        ET_HIP(hipEventSynchronize(e1));
-        ET_HIP(hipEventElapsedTime(&ms, e0, e1));
+        err = hipEventRecord(e1, nullptr);
+        if (err == hipSuccess)
+            err = hipEventSynchronize(e1);
+        if (err == hipSuccess)
+            err = hipEventElapsedTime(&ms, e0, e1);
     }
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
+    if (e0)
+        (void)hipEventDestroy(e0);
+    if (e1)
+        (void)hipEventDestroy(e1);
+    if (err != hipSuccess)
+        return hip_fail(err, "microbenchmark timing");
     *seconds = ms * 1e-3;
     return launch_status("microbenchmark launch");
 }
 
+// device memory that is released on every way out
+struct MbBuffer {
+    void *p = nullptr;
+    ~MbBuffer() {
+        if (p)
+            (void)hipFree(p);
+    }
+    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes); }
+};
+
 } // namespace et
 
+// what 0: LDS fragment reads (ds_read_b128); p0 = row stride in bytes of the 16-row x 64-byte fragment pattern, a
+//         multiple of 16 (0: 64 x 16 consecutive bytes), p1 = waves per CU.  units = bytes read per CU.
+// what 1: the weight stream: one-kilobyte global_load_dwordx4 requests, four in flight per wave, from 2 MiB that
+//         stay in L2; p1 = waves per CU.  units = bytes requested per CU.
+// what 2: matrix unit and vector ALU: p0 = 0 every wave issues MFMAs only, 1 v_fma_f32 only (four per MFMA of mode
+//         0), 2 both, strictly alternating in every wave, 3 four waves MFMAs and four waves (on the same SIMDs) the
+//         FMAs; p1 = waves per CU (modes 0-2).  units = v_mfma_f32_16x16x32_f16 per MFMA-issuing wave.
+// seconds = duration of one launch on every CU of the device.  Allocates and synchronises.
 extern "C" int et_microbench(int what, int p0, int p1, double *seconds, double *units_per_cu) {
     using namespace et;
     ET_REQUIRE(seconds && units_per_cu, ET_ERR_INVALID_ARG, "et_microbench: null pointer");
+    // everything that can be refused is refused before anything is allocated
+    ET_REQUIRE(what >= 0 && what <= 2, ET_ERR_INVALID_ARG, "et_microbench: what=%d", what);
+    if (what == 0)
+        ET_REQUIRE(p0 >= 0 && p0 % 16 == 0 && 15 * p0 + 64 + 112 <= 60000, ET_ERR_INVALID_ARG,
+                   "et_microbench: stride %d (a multiple of 16 up to 3984)", p0);
+    if (what == 2)
+        ET_REQUIRE(p0 >= 0 && p0 <= 3, ET_ERR_INVALID_ARG, "et_microbench: mode %d", p0);
     const int cus = et_device_cu_count();
     ET_REQUIRE(cus > 0, ET_ERR_HIP, "et_microbench: no device");
-    float *out = nullptr;
-    ET_HIP(hipMalloc(&out, (size_t)cus * 1024 * sizeof(float)));
+    MbBuffer outb, wb;
+    ET_HIP(outb.alloc((size_t)cus * 1024 * sizeof(float)));
+    float *out = static_cast<float *>(outb.p);
     int rc = ET_OK;
     const int iters = 2000;
-    if (what == 0) { // LDS fragment reads: p0 = row stride in bytes (0: linear pattern), p1 = waves per CU
+    if (what == 0) {
         const int waves = p1 > 0 && p1 <= 16 ? p1 : 16;
-        ET_REQUIRE(p0 >= 0 && 15 * p0 + 64 + 112 <= 60000, ET_ERR_INVALID_ARG, "et_microbench: stride %d", p0);
         if (p0 == 0)
             rc = mb_time([&] { hipLaunchKernelGGL(mb_lds_kernel<1>, dim3(cus), dim3(waves * 64), 60000, 0, out, 0, iters); }, seconds);
         else
             rc = mb_time([&] { hipLaunchKernelGGL(mb_lds_kernel<0>, dim3(cus), dim3(waves * 64), 60000, 0, out, p0, iters); }, seconds);
         *units_per_cu = (double)waves * iters * 4 * 1024; // bytes read per CU
-    } else if (what == 1) { // weight stream from L2: p1 = waves per CU; every CU walks the same 2 MiB
+    } else if (what == 1) { // every CU walks the same 2 MiB
         const int waves = p1 > 0 && p1 <= 16 ? p1 : 16;
         const int per_wave = (2 << 20) / 16, rounds = 8;
-        f16 *w = nullptr;
-        ET_HIP(hipMalloc(&w, (size_t)16 * per_wave));
-        ET_HIP(hipMemset(w, 0, (size_t)16 * per_wave));
+        ET_HIP(wb.alloc((size_t)16 * per_wave));
+        ET_HIP(hipMemset(wb.p, 0, (size_t)16 * per_wave));
+        const f16 *w = static_cast<const f16 *>(wb.p);
         rc = mb_time([&] { hipLaunchKernelGGL(mb_wstream_kernel, dim3(cus), dim3(waves * 64), 0, 0, out, w, per_wave, rounds); }, seconds);
-        (void)hipFree(w);
         *units_per_cu = (double)waves * per_wave * rounds; // bytes requested per CU
-    } else if (what == 2) { // co-execution: p0 = mode (0 MFMA, 1 FMA, 2 mixed in one wave, 3 specialised waves), p1 = waves per CU
+    } else {
         const int waves = p0 == 3 ? 8 : (p1 > 0 && p1 <= 16 ? p1 : 4);
         switch (p0) {
         case 0: rc = mb_time([&] { hipLaunchKernelGGL(mb_coexec_kernel<0>, dim3(cus), dim3(waves * 64), 0, 0, out, iters); }, seconds); break;
         case 1: rc = mb_time([&] { hipLaunchKernelGGL(mb_coexec_kernel<1>, dim3(cus), dim3(waves * 64), 0, 0, out, iters); }, seconds); break;
         case 2: rc = mb_time([&] { hipLaunchKernelGGL(mb_coexec_kernel<2>, dim3(cus), dim3(waves * 64), 0, 0, out, iters); }, seconds); break;
-        case 3: rc = mb_time([&] { hipLaunchKernelGGL(mb_coexec_kernel<3>, dim3(cus), dim3(waves * 64), 0, 0, out, iters); }, seconds); break;
-        default: set_error("et_microbench: mode %d", p0); rc = ET_ERR_INVALID_ARG;
+        default: rc = mb_time([&] { hipLaunchKernelGGL(mb_coexec_kernel<3>, dim3(cus), dim3(waves * 64), 0, 0, out, iters); }, seconds); break;
         }
         *units_per_cu = (double)iters * 16; // MFMAs per MFMA wave (and 4x as many FMAs per FMA wave)
-    } else {
-        set_error("et_microbench: what=%d", what);
-        rc = ET_ERR_INVALID_ARG;
     }
-    (void)hipFree(out);
     return rc;
 }

@@ -9,7 +9,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libet_amd.so")
 
-SOURCES = ["runtime.hip", "formats.cpp", "skip_layernorm.hip", "tile_linear.hip", "tile_tail.hip", "dense_gemm.hip", "attention.hip", "microbench.hip",
+SOURCES = ["runtime.hip", "formats.cpp", "skip_layernorm.hip", "tile_linear.hip", "tile_tail.hip", "dense_gemm.hip", "attention.hip",
            "encoder_capi.cpp"]
 
 # packed fp32 ops stay off: some of their forms have produced wrong results on
@@ -55,7 +55,28 @@ def build(verbose: bool = False) -> str:
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     subprocess.check_call(cmd)
     build_examples(verbose)
+    build_microbench(verbose)
     return LIB
+
+
+MICROBENCH_LIB = os.path.join(HERE, "bench", "libet_microbench.so")
+
+
+def build_microbench(verbose: bool = False) -> str:
+    """The delivery-path microbenchmarks of bench.py --micro: a library of their own (they are a measuring tool,
+    not part of the encoder's C ABI), linked against libet_amd.so for its error plumbing."""
+    src = os.path.join(HERE, "bench", "microbench.hip")
+    cmd = [hipcc(), "-x", "hip", src, "-shared", "-o", MICROBENCH_LIB, "-I", os.path.join(HERE, "..", "include"),
+           "-I", HERE] + HIP_FLAGS + ["-L", HERE, "-let_amd", "-Wl,-rpath,$ORIGIN/.."]
+    if verbose:
+        print(" ".join(cmd))
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in p.stdout.splitlines() if "is not a recognized feature" not in l)
+    if p.returncode != 0:
+        raise RuntimeError(out)
+    if verbose and out.strip():
+        print(out)
+    return MICROBENCH_LIB
 
 
 def build_examples(verbose: bool = False) -> str:

@@ -1176,14 +1176,28 @@ static bool attach_mask_summary(AttnArgs &a) {
 // qk_width: columns per head in Q and K (0 = head_dim)
 // given_summary: a summary of a.mask supplied by the caller of this function
 // (it then replaces the lookup among the attached ones)
-static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedqk,
-                              hipStream_t st, const char *who, int qk_width = 0,
-                              const unsigned *given_summary = nullptr) {
+static int attention_check(const AttnArgs &a, int d_model, bool sharedqk, const char *who) {
     ET_REQUIRE(a.out && a.V, ET_ERR_INVALID_ARG, "%s: null pointer", who);
     ET_REQUIRE(sharedqk ? a.QK != nullptr : (a.Q && a.K), ET_ERR_INVALID_ARG, "%s: null pointer", who);
     ET_REQUIRE(a.seq_len > 0 && d_model > 0 && a.nhead > 0 && a.batch > 0, ET_ERR_INVALID_ARG,
                "%s: seq_len=%d d_model=%d nhead=%d batch=%d", who, a.seq_len, d_model, a.nhead, a.batch);
     ET_REQUIRE(d_model % a.nhead == 0, ET_ERR_INVALID_ARG, "%s: d_model %% nhead != 0", who);
+    const int hd = d_model / a.nhead;
+    ET_REQUIRE(hd % 16 == 0 && hd <= 128, ET_ERR_UNSUPPORTED,
+               "%s: head_dim %d: multiples of 16 up to 128", who, hd);
+    ET_REQUIRE(aligned16(a.out) && aligned16(a.Q) && aligned16(a.K) && aligned16(a.V),
+               ET_ERR_ALIGNMENT, "%s: out/Q/K/V must be 16-byte aligned", who);
+    return ET_OK;
+}
+
+static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedqk,
+                              hipStream_t st, const char *who, int qk_width = 0,
+                              const unsigned *given_summary = nullptr) {
+    {
+        const int rc = attention_check(a, d_model, sharedqk, who);
+        if (rc != ET_OK)
+            return rc;
+    }
     const int hd_data = d_model / a.nhead;
     // Kernels are built for heads of 32, 64 and 128 columns.  Any other multiple
     // of 16 up to 128 (the reference loops over head_dim in steps of 16,
@@ -1200,8 +1214,6 @@ static int attention_dispatch(AttnArgs a, int d_model, bool pruned, bool sharedq
         pruned = true;
         a.head_width = hd_data;
     }
-    ET_REQUIRE(aligned16(a.out) && aligned16(a.Q) && aligned16(a.K) && aligned16(a.V),
-               ET_ERR_ALIGNMENT, "%s: out/Q/K/V must be 16-byte aligned", who);
     if (!pruned) {
         ET_REQUIRE(a.ldq % 8 == 0 && a.ldv % 8 == 0, ET_ERR_ALIGNMENT,
                    "%s: d_model must be a multiple of 8", who);
@@ -1363,7 +1375,12 @@ extern "C" int et_OTF_attention_noalloc(void *out, const void *Q, const void *K,
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (!mask) // nothing to summarise: no scratch memory is touched
         return attention_dispatch(a, d_model, false, false, st, "et_OTF_attention_noalloc");
-    ET_REQUIRE(seq_len > 0, ET_ERR_INVALID_ARG, "et_OTF_attention_noalloc: seq_len=%d", seq_len);
+    {
+        // everything the attention launch would refuse is refused before the scratch array is written
+        const int rc = attention_check(a, d_model, false, "et_OTF_attention_noalloc");
+        if (rc != ET_OK)
+            return rc;
+    }
     ET_REQUIRE(seq_len <= NOALLOC_MAX_SEQ, ET_ERR_UNSUPPORTED,
                "et_OTF_attention_noalloc: seq_len %d beyond the %d that the static scratch array covers",
                seq_len, NOALLOC_MAX_SEQ);
@@ -1379,6 +1396,28 @@ extern "C" int et_OTF_attention_noalloc(void *out, const void *Q, const void *K,
     if (rs != ET_OK)
         return rs;
     return attention_dispatch(a, d_model, false, false, st, "et_OTF_attention_noalloc", 0, summary);
+}
+
+extern "C" int et_OTF_attention_summary(void *out, const void *Q, const void *K, const void *V,
+                                        const void *mask, const void *mask_summary, int seq_len, int d_model,
+                                        int nhead, int batch, const int *seq_lens, float log2_scale,
+                                        void *stream) {
+    using namespace et;
+    AttnArgs a = {};
+    a.out = static_cast<f16 *>(out);
+    a.Q = static_cast<const f16 *>(Q);
+    a.K = static_cast<const f16 *>(K);
+    a.V = static_cast<const f16 *>(V);
+    a.mask = static_cast<const f16 *>(mask);
+    a.seq_lens = seq_lens;
+    a.ldq = a.ldv = d_model;
+    a.seq_len = seq_len;
+    a.nhead = nhead;
+    a.batch = batch;
+    a.log2_scale = log2_scale;
+    ET_REQUIRE(!mask_summary || mask, ET_ERR_INVALID_ARG, "et_OTF_attention_summary: a summary without a mask");
+    return attention_dispatch(a, d_model, false, false, static_cast<hipStream_t>(stream), "et_OTF_attention_summary",
+                              0, static_cast<const unsigned *>(mask_summary));
 }
 
 extern "C" int et_OTF_attention_qk_width(void *out, const void *Q, const void *K, const void *V,

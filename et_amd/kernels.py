@@ -113,6 +113,22 @@ def OTF_attention(Q, K, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2_sc
     return Z
 
 
+def OTF_attention_summary(Q, K, V, mask, summary, seq_len, nhead, batch=1, seq_lens=None, log2_scale=1.0, out=None):
+    """OTF_attention with the mask's summary (attention_mask_summary(mask, seq_len), or None) passed along
+    instead of looked up by the mask's address"""
+    d_model = Q.shape[1]
+    Z = out if out is not None else torch.empty_like(Q)
+    for t, name in ((Q, "Q"), (K, "K"), (V, "V"), (Z, "out")):
+        _want(t, "OTF_attention_summary " + name, batch * seq_len, d_model)
+    _want(mask, "OTF_attention_summary mask", seq_len * seq_len)
+    _want(seq_lens, "OTF_attention_summary seq_lens", batch)
+    if summary is not None and summary.numel() * summary.element_size() < lib().et_attention_mask_summary_bytes(seq_len):
+        raise ValueError("OTF_attention_summary: the summary is smaller than et_attention_mask_summary_bytes(seq_len)")
+    check(lib().et_OTF_attention_summary(_h(Z), _h(Q), _h(K), _h(V), _h(mask), None if summary is None else summary.data_ptr(),
+                                         seq_len, d_model, nhead, batch, _i32(seq_lens), log2_scale, _stream()))
+    return Z
+
+
 def OTF_attention_noalloc(Q, K, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2_scale=1.0, out=None):
     """OTF_attention through the entry point that allocates nothing: the mask summary is computed into a
     static device array of the library (seq_len <= 4096 with a mask).  `out` is required: this wrapper
@@ -199,9 +215,17 @@ def sharedQK_attention(QK, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2
     return Z
 
 
+_checked_cu = {}   # (address, elements, seq_len, rows) -> tensor version that passed
+
+
 def _check_cu(cu_seqlens, seq_len, total_rows, what):
     """the packed row offsets must start at 0, rise by at most seq_len per sequence and end at the packed
-    tensor's row count: the kernels trust them for every address (one small device-to-host copy)"""
+    tensor's row count: the kernels trust them for every address.  Checking costs one small device-to-host copy,
+    which waits for the stream; a tensor that passed is remembered by address and version counter, so only its
+    first use (and the first one after it was written to in place) synchronises."""
+    key = (cu_seqlens.data_ptr(), cu_seqlens.numel(), seq_len, total_rows)
+    if _checked_cu.get(key) == cu_seqlens._version:
+        return
     cu = cu_seqlens.detach().cpu().numpy().astype("int64")
     if cu.size < 1 or cu[0] != 0 or cu[-1] != total_rows:
         raise ValueError(f"{what}: cu_seqlens must run from 0 to the {total_rows} packed rows, got "
@@ -209,6 +233,9 @@ def _check_cu(cu_seqlens, seq_len, total_rows, what):
     step = cu[1:] - cu[:-1]
     if step.size and (step.min() < 0 or step.max() > seq_len):
         raise ValueError(f"{what}: every sequence must hold 0..{seq_len} rows")
+    if len(_checked_cu) > 64:
+        _checked_cu.clear()
+    _checked_cu[key] = cu_seqlens._version
 
 
 def pack_rows(padded, cu_seqlens, seq_len, total_rows, order=None):

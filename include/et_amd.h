@@ -120,6 +120,15 @@ int et_OTF_attention(void *out, const void *Q, const void *K, const void *V,
 size_t et_attention_mask_summary_bytes(int seq_len);
 int et_attention_mask_summary(const void *mask, int seq_len, void *summary, void *stream);
 int et_attention_mask_summary_attach(const void *mask, int seq_len, const void *summary);
+/* et_OTF_attention with the mask's summary passed along (a device buffer filled
+ * by et_attention_mask_summary for this mask and seq_len; NULL: the mask is
+ * added everywhere): nothing is attached to, or looked up by, the mask's
+ * address, so the summary's lifetime is the caller's own business and a freed
+ * mask leaves nothing behind.  Same bits as the other forms. */
+int et_OTF_attention_summary(void *out, const void *Q, const void *K, const void *V,
+                             const void *mask, const void *mask_summary, int seq_len,
+                             int d_model, int nhead, int batch, const int *seq_lens,
+                             float log2_scale, void *stream);
 
 /* et_OTF_attention for callers that cannot allocate device memory (code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
@@ -474,21 +483,6 @@ int et_device_synchronize(void);
  * Not thread-safe; results never depend on these beyond fp32 summation
  * order. */
 int et_tuning_set(const char *key, int value);
-/* Microbenchmarks of the delivery paths that bound the kernels (no counterpart
- * in the reference; they allocate and synchronise, so not for hot paths).
- *   what 0: LDS fragment reads (ds_read_b128); p0 = row stride in bytes of the
- *           16-row x 64-byte fragment pattern (0: 64 x 16 consecutive bytes),
- *           p1 = waves per CU.  units = bytes read per CU.
- *   what 1: the weight stream: one-kilobyte global_load_dwordx4 requests, four
- *           in flight per wave, from 2 MiB that stay in L2; p1 = waves per CU.
- *           units = bytes requested per CU.
- *   what 2: matrix unit and vector ALU: p0 = 0 every wave issues MFMAs only,
- *           1 v_fma_f32 only (four per MFMA of mode 0), 2 both, strictly
- *           alternating in every wave, 3 four waves MFMAs and four waves (on
- *           the same SIMDs) the FMAs; p1 = waves per CU (modes 0-2).
- *           units = v_mfma_f32_16x16x32_f16 per MFMA-issuing wave.
- * seconds = duration of one launch on every CU of the device. */
-int et_microbench(int what, int p0, int p1, double *seconds, double *units_per_cu);
 /* The fused layer-tail kernels order their waves with bounded waits on LDS
  * counters.  A wave that gives up (it never should) sets one status word per
  * process and goes on, so the kernel ends - with a wrong result - instead of

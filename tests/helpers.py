@@ -6,12 +6,7 @@ MAX_ABS = 2e-2
 MEAN_REL = 1e-3
 
 
-def rng(seed):
-    return np.random.default_rng(seed)
-
-
-def randn_h(r, shape, std=1.0):
-    return (r.standard_normal(shape) * std).astype(np.float16)
+from et_amd.synthetic import randn_h, rng  # noqa: F401  (the product's generator: tests and bench see the same bits)
 
 
 def check_close(got, want, max_abs=MAX_ABS, mean_rel=MEAN_REL, what=""):

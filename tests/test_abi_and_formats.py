@@ -84,10 +84,9 @@ def test_argument_errors_return_codes_without_a_device():
     p = C.addressof(buf)
     assert l.et_tile_spmm_add_bias(p, p, p, p, p, 16, 24, 16, p, None) == -3          # N not a multiple of 16
     assert l.et_OTF_attention(p, p, p, p, None, 128, 768, 7, 1, None, 1.0, None) == -1  # d_model % nhead
-    assert l.et_OTF_attention(p, p, p, p, None, 128, 96, 2, 1, None, 1.0, None) == -3   # head_dim 48 unsupported
+    assert l.et_OTF_attention(p, p, p, p, None, 128, 80, 2, 1, None, 1.0, None) == -3   # head_dim 40: not a multiple of 16
     assert b"head_dim" in l.et_last_error()
     assert l.et_strerror(-3) == b"unsupported shape"
-    assert l.et_microbench(0, 1568, 16, None, None) == -1                               # no result pointers
     with pytest.raises(_lib.EtError):
         formats.gen_sparse_tile_mat(100, 64, 0.5, 1)     # nrow not a multiple of 16
     with pytest.raises(_lib.EtError):
