@@ -454,6 +454,35 @@ __device__ __forceinline__ void tl_flush_acc(f32x4 (&acc)[NB][2], int j, f32x4 c
     }
 }
 
+// The same with a branch per accumulator instead of NB masked multiply-adds
+// (eight adds per flush instead of 8 NB fused multiply-adds and NB selects).
+// Two things keep the compiler from undoing it: the adds are inline assembly
+// with tied operands (the sum replaces the accumulator in its own registers;
+// otherwise every accumulator gets a second set of registers behind the
+// branches), and the cases are independent ifs with something opaque between
+// them (as an if / else chain they become a switch, whose lowering copies the
+// accumulators around or addresses them through scratch memory).
+template <int K>
+__device__ __forceinline__ void tl_add_tied(f32x4 &a, const f32x4 &c) {
+    float a0 = a[0], a1 = a[1], a2 = a[2], a3 = a[3];
+    asm volatile("v_add_f32 %0, %0, %4 ; accumulator %8\n\tv_add_f32 %1, %1, %5\n\t"
+                 "v_add_f32 %2, %2, %6\n\tv_add_f32 %3, %3, %7"
+                 : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3)
+                 : "v"(c[0]), "v"(c[1]), "v"(c[2]), "v"(c[3]), "n"(K));
+    a = f32x4{a0, a1, a2, a3};
+}
+template <int NB>
+__device__ __forceinline__ void tl_flush_acc_branch(f32x4 (&acc)[NB][2], int j, const f32x4 &cur0, const f32x4 &cur1) {
+    tl_static_for<0, NB>([&](auto kc) {
+        constexpr int k = decltype(kc)::value;
+        if (j == k) {
+            tl_add_tied<k>(acc[k][0], cur0);
+            tl_add_tied<k>(acc[k][1], cur1);
+        }
+        asm volatile("; after case %0" ::"n"(k));
+    });
+}
+
 // Fused skip connection + LayerNorm over a workgroup's 32 finished rows (the
 // math of skip_layernorm.hip: x = half(y + skip), fp32 mean and biased
 // two-pass variance, eps 1e-6).  The workgroup covers the whole row: wave k's
@@ -1112,6 +1141,11 @@ __global__ void __launch_bounds__(TL_CTHREADS) tile_linear_chunked_ln_kernel(con
 // K = input width, KC / nchunk = the second plan's chunking; skip / gamma /
 // beta belong to the first LayerNorm that runs, gamma2 / beta2 to the second.
 // ---------------------------------------------------------------------------
+#ifdef TL_FFN_MASKED_FLUSH
+#define TL_FFN_FLUSH(acc_, j_, c0_, c1_) tl_flush_acc<NB>(acc_, j_, c0_, c1_)
+#else
+#define TL_FFN_FLUSH(acc_, j_, c0_, c1_) tl_flush_acc_branch<NB>(acc_, j_, c0_, c1_)
+#endif
 constexpr int TL_FFN_WAVES = 16;
 constexpr int TL_FFN_MAX_PHASES = 16;
 
@@ -1297,7 +1331,7 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
             const int q0_ = __builtin_amdgcn_readfirstlane(bvecO), qe_ = __builtin_amdgcn_readlane(bvecO, NB);
             tl_stream<NB>(xlane1, xrow1, a.data[0], a.row_offset[0], lane_w, hi, q0_, qe_, max(qe_ - 1, q0_),
                           bvecO, wB, oB,
-                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); });
+                          [&](int j, f32x4 c0, f32x4 c1) { TL_FFN_FLUSH(acc, j, c0, c1); });
         }
         TL_FFN_PRELOAD(data1, poff1, bvecF, wA, oA)
         TlLnOperands<NB, NW, NW> lnop1; // (requested here: their latency runs under the wait for the other waves)
@@ -1342,7 +1376,7 @@ __global__ void __launch_bounds__(TL_FFN_WAVES * 64) tile_ffn_fused_kernel(const
                 reinterpret_cast<const char *>(hs + (p & 1) * hbuf + c16 * ldh + x.khalf8);
             const int q0_ = __builtin_amdgcn_readfirstlane(bvecS), qe_ = __builtin_amdgcn_readlane(bvecS, NB);
             tl_stream<NB>(xlane2, xrow2, data2, poff2, lane_w, hi, q0_, qe_, max(qe_ - 1, q0_), bvecS, wA, oA,
-                          [&](int j, f32x4 c0, f32x4 c1) { tl_flush_acc<NB>(acc, j, c0, c1); });
+                          [&](int j, f32x4 c0, f32x4 c1) { TL_FFN_FLUSH(acc, j, c0, c1); });
             tl_signal(ctr + TL_FFN_MAX_PHASES + p, lane);
         }
         bvecS = bvecSn;
