@@ -1,51 +1,60 @@
 // Layer tail (encoder/encoder.cu:33-44: O_linear, skip + LayerNorm, MLP1 with
-// GELU, MLP2, skip + LayerNorm) as PAIRS of workgroups over 64-row panels.
+// GELU, MLP2, skip + LayerNorm) as PAIRS of workgroups over one row panel.
 //
 // Why.  With one workgroup per 32-row panel every CU streams the whole of the
 // three weight matrices (2.1 MB at BERT-base / 80 %) through the L2 -> CU path
-// for 32 rows of work, two MFMAs per kilobyte, and all CUs together saturate
-// the L2s.  Here a panel has 64 rows (four MFMAs per kilobyte of W) and the
-// hidden dimension of the feed-forward block is split over the two workgroups
-// of a pair: workgroup `half` of panel P runs the projection and the first
-// LayerNorm on the panel (both do: 11 % duplicated work), then the first
-// feed-forward linear for ITS half of the hidden columns and the second linear
-// over those columns only.  A CU streams 1.2 MB of W instead of 2.1.
+// for 32 rows of work, two MFMAs per kilobyte, and a workgroup is one chain of
+// dependent phases with nothing beside it on its CU.  Here the hidden dimension
+// of the feed-forward block is split over the two workgroups of a pair:
+// workgroup `half` of panel P runs the projection and the first LayerNorm on
+// the panel (both do: 11 % duplicated work), then the first feed-forward linear
+// for ITS half of the hidden columns and the second linear over those columns
+// only.  Two panel heights are built (template parameter MS, 16-row subtiles
+// per panel): 64 rows - four MFMAs per kilobyte of W, a CU streams 1.2 MB
+// instead of 2.1, one workgroup per CU - and 32 rows - 77 KB of LDS, so that two
+// workgroups share a CU and one's waits are the other's issue slots.  Neither
+// beats the one-workgroup form of tile_linear.hip at BERT-base sizes (8192
+// rows, 80 % pruned: 74 and 89 us against 53): with hidden buffers of 192
+// columns, which is what fits, a segment of the second linear is one or two
+// tile pairs long and the per-segment work (flush, hand-over, start vector)
+// outweighs what the split saves.  Both stay available as an option
+// (et_tuning_set "tile_tail_pair") and are tested like the default.
 //
 // The two partial sums of a panel meet without any workgroup waiting for the
-// other one.  Rows 0-31 of the panel are finished by whoever arrives second at
-// that row-half's counter, rows 32-63 likewise; a workgroup visits the other
-// row-half first.  At a row-half it looks at the counter: zero means the
-// partner has not published yet, so it writes its own fp32 partial (scratch),
-// fences, and adds one to the counter - if the add returns one the partner
+// other one.  The first half of the panel's rows is finished by whoever arrives
+// second at that row-half's counter, the second half likewise; a workgroup
+// visits the other row-half first.  At a row-half it looks at the counter: zero
+// means the partner has not published yet, so it writes its own fp32 partial
+// (scratch) and adds one to the counter - if the add returns one the partner
 // arrived in between.  Whoever finds (or gets) one reads the partner's partial,
-// adds the two, runs bias + skip + LayerNorm 2 on those 32 rows, stores them
-// and resets the counter.  When the pair runs in step each workgroup writes one
+// adds the two, runs bias + skip + LayerNorm 2 on those rows, stores them and
+// resets the counter.  When the pair runs in step each workgroup writes one
 // row-half, reads one and normalises one; when one is late the other leaves
 // both of its partials and exits, and the late one finishes both.  No spin, no
 // assumption that the partner is resident.  a + b == b + a in fp32, so the
 // bits do not depend on who finishes.
 //
-// Inside a workgroup (8 waves, two per SIMD, 256 registers each).  LDS holds the panel and two 192-column hidden
+// Inside a workgroup (8 waves).  LDS holds the panel and two 192-column hidden
 // buffers INTERLEAVED per row (row stride = panel width + 2 x 208 halves, which
 // keeps ds_read_b128 conflict-free), so a tile's X operand is "lane's row base
 // + one byte offset" whether it multiplies the panel (projection, first
 // linear) or a hidden buffer (second linear): one stage body serves all three.
 // Every wave walks ONE continuous stream of tile pairs that the host lays out
-// for it at plan time (its 6 block-rows of the projection; then, per 192-column
-// phase p, one or two hidden block-rows of the first linear and its 6 output block-rows
-// of the second linear over chunk p, the first linear one phase ahead), through
-// a register pipeline of TT_DEPTH pairs that never drains.  Where a segment of the stream
-// ends, a control word that travels with the segment's last pair (next to its
-// operand offsets, so it costs no memory request of its own) says what to do
-// with the finished 64 x 16 sums: GELU and store into a hidden buffer, or add
-// into one of the wave's output accumulators; and which LDS event counter to
-// wait for or to signal (hidden buffer complete / hidden buffer free), exactly
-// as an s_barrier would order them but without stopping a wave that is not a
-// whole phase ahead.  Waits are
-// bounded; a wave that gives up sets the process's wait-status word, which the
-// next launch reports.  Both LayerNorms run on the accumulators where they are
-// (a panel row's 768 columns are spread over the 8 waves; row sums meet in
-// LDS), so no staging tile is needed for them.
+// for it at plan time (its block-rows of the projection; then, per 192-column
+// phase p, one or two hidden block-rows of the first linear and its output
+// block-rows of the second linear over chunk p, the first linear one phase
+// ahead), through a register pipeline of 4 or 8 pairs that never drains.  Where
+// a segment of the stream ends, a control word that travels with the segment's
+// last pair (next to its operand offsets, so it costs no memory request of its
+// own) says what to do with the finished sums: GELU and store into a hidden
+// buffer, or add into one of the wave's output accumulators; and which LDS
+// event counter to wait for or to signal (hidden buffer complete / hidden
+// buffer free), exactly as an s_barrier would order them but without stopping
+// a wave that is not a whole phase ahead.  Waits are bounded; a wave that gives
+// up sets the process's wait-status word, which the next launch reports.  Both
+// LayerNorms run on the accumulators where they are (a panel row's columns are
+// spread over the 8 waves; row sums meet in LDS), so no staging tile is needed
+// for them.
 #include "tile_plan.h"
 
 #include <algorithm>
@@ -55,35 +64,38 @@
 namespace et {
 
 #ifndef TT_NWAVES
-#define TT_NWAVES 12
+#define TT_NWAVES 8
 #endif
-constexpr int TT_WAVES = TT_NWAVES;       // 12: three per SIMD, 168 registers each (4 block-rows x 64 rows of accumulators); 8: two per SIMD
+constexpr int TT_WAVES = TT_NWAVES;       // 8: two per SIMD and workgroup; 12: three (64-row panels: 168 registers each)
 static_assert(TT_WAVES == 8 || TT_WAVES == 12, "eight or twelve waves");
-constexpr int TT_BM = 64;                 // panel rows
+// A panel has 16 * MS rows, MS = 4 or 2 (template parameter of the kernel): 64 rows, one workgroup per CU,
+// or 32 rows, two workgroups per CU (either the two of a panel or of two different ones), whose chains of
+// dependent phases overlap.
 constexpr int TT_HB = 12;                 // hidden block-rows per phase
 constexpr int TT_HC = 16 * TT_HB;         // hidden columns per phase
 constexpr int TT_HW = (TT_HC + 16) * 2;   // bytes of one hidden buffer inside an LDS row
 constexpr int TT_MAX_PHASES = 16;         // per half: counters F[16], S[16]
 constexpr int TT_MAX_PANELS = 8192;       // counters per program: 2 per panel
-// Tile pairs in flight per wave.
-#ifndef TT_DEPTH
-#define TT_DEPTH (TT_NWAVES == 12 ? 4 : 8)
-#endif
+// Tile pairs in flight per wave: 8 where a wave has 256 registers (eight waves, 64-row panels), else 4.  The
+// host lays every stream out as a multiple of TT_PAD pairs, which suits both.
+constexpr int TT_PAD = 8;
+constexpr int tt_depth(int ms) { return (TT_WAVES == 8 && ms == 4) ? 8 : 4; }
 // stages the X fragments are read ahead of their MFMAs
 #ifndef TT_XA
 #define TT_XA 1
 #endif
 
-template <int D> struct TtGeom {
+template <int D, int MS = 4> struct TtGeom {
     static constexpr int NB = (D / 16 + TT_WAVES - 1) / TT_WAVES; // output block-rows per wave
     static constexpr int XW = (D + ((D & 31) ? 0 : 16)) * 2;      // bytes of the panel part of an LDS row
     static constexpr int RS = XW + 2 * TT_HW;                     // LDS row stride, == 32 (mod 64)
-    static constexpr int CT = TT_BM * RS;                         // event counters: F[16], S[16]
+    static constexpr int CT = 16 * MS * RS;                       // event counters: F[16], S[16]
     static constexpr int ZV = CT + 2 * TT_MAX_PHASES * 4;         // 16 zero floats
     static constexpr int MISC = ZV + 64;                          // workgroup broadcasts
-    static constexpr int BI = MISC + 64;                          // first linear's bias as fp32, 64 B per block-row
+    static constexpr int BI = MISC + 64;                          // first linear's bias (halves), 32 B per block-row
     static_assert(RS % 64 == 32, "row stride must be == 32 (mod 64) bytes");
 };
+constexpr int TT_BI_BYTES = 32; // per hidden block-row
 
 // A pair's record in the stream: 16 bytes, {offset of tile A, control, offset of
 // tile B, control} - lanes 0-31 read the first half, lanes 32-63 the second.  An
@@ -116,9 +128,6 @@ struct TtArgs {
     int *status; // set when a bounded wait gives up
     int M, npanels, per_xcd, spin;
     int hb0[2], nb1h[2]; // first hidden block-row and count per half
-#ifdef TT_TRACE
-    long long *trace; // per (workgroup, wave): 16 stamps
-#endif
 };
 
 template <int I> using tt_ic = std::integral_constant<int, I>;
@@ -187,65 +196,55 @@ __device__ __forceinline__ float tt_xor_sum_16_32(float v) {
     return __builtin_bit_cast(float, z0);
 }
 
-template <int RS>
-__device__ __forceinline__ void tt_read_x(f16x8 (&x)[4], const char *xl, int off) {
+template <int RS, int MS>
+__device__ __forceinline__ void tt_read_x(f16x8 (&x)[MS], const char *xl, int off) {
     const char *p = xl + off;
 #pragma unroll
-    for (int k = 0; k < 4; k++)
+    for (int k = 0; k < MS; k++)
         x[k] = *reinterpret_cast<const f16x8 *>(p + k * 16 * RS);
 }
 
-// The stream: n stages (a multiple of TT_DEPTH), pair q's operands in slot q %
-// TT_DEPTH of w / o / c (the first TT_DEPTH requested by the caller), X fragments
-// read TT_XA stages ahead, four MFMAs per stage into cur[0..3] (one per 16-row
+// The stream: n stages (a multiple of DEPTH), pair q's operands in slot q %
+// DEPTH of w / o / c (the first DEPTH requested by the caller), X fragments
+// read TT_XA stages ahead, MS MFMAs per stage into cur[] (one per 16-row
 // subtile).  at_end(ctl, reread) runs where a stage finishes a segment (its
 // pair's control word is not 0); reread() reads the fragments of the pairs that
 // are already on their way once more, for a handler that has to wait before
 // they may be read.
-template <int RS, class AtEnd>
+template <int RS, int MS, int DEPTH, class AtEnd>
 __device__ __forceinline__ void tt_stream(const char *xl, const char *wq, const char *rq, int n,
-                                          unsigned &lane_lo, unsigned &lane_lw, f16x8 (&w)[TT_DEPTH],
-                                          int (&o)[TT_DEPTH], int (&c)[TT_DEPTH], f32x4 (&cur)[4],
+                                          unsigned &lane_lo, unsigned &lane_lw, f16x8 (&w)[DEPTH],
+                                          int (&o)[DEPTH], int (&c)[DEPTH], f32x4 (&cur)[MS],
                                           AtEnd &&at_end) {
     constexpr int NX = TT_XA + 1;
-    static_assert(TT_DEPTH % NX == 0 && TT_XA < TT_DEPTH, "fragment buffers rotate inside the unrolled group");
-    f16x8 xf[NX][4];
+    static_assert(DEPTH % NX == 0 && TT_XA < DEPTH, "fragment buffers rotate inside the unrolled group");
+    f16x8 xf[NX][MS];
 #pragma unroll
     for (int i = 0; i < TT_XA; i++)
-        tt_read_x<RS>(xf[i], xl, o[i]);
-    const char *wp = wq + TT_DEPTH * 1024, *rp = rq + TT_DEPTH * 16;
-    for (int q = 0; q < n; q += TT_DEPTH) {
-        tt_static_for<0, TT_DEPTH>([&](auto ic) {
+        tt_read_x<RS, MS>(xf[i], xl, o[i]);
+    const char *wp = wq + DEPTH * 1024, *rp = rq + DEPTH * 16;
+    for (int q = 0; q < n; q += DEPTH) {
+        tt_static_for<0, DEPTH>([&](auto ic) {
             constexpr int I = decltype(ic)::value;
-#if !(defined(TT_ABL) && (TT_ABL & 1))
-            tt_read_x<RS>(xf[(I + TT_XA) % NX], xl, o[(I + TT_XA) % TT_DEPTH]);
-#endif
+            tt_read_x<RS, MS>(xf[(I + TT_XA) % NX], xl, o[(I + TT_XA) % DEPTH]);
             // keep the reads above the MFMAs (the scheduler otherwise sinks them
             // and every stage waits out the LDS latency)
             __builtin_amdgcn_sched_barrier(0);
-#if !(defined(TT_ABL) && (TT_ABL & 4))
 #pragma unroll
-            for (int k = 0; k < 4; k++)
+            for (int k = 0; k < MS; k++)
                 cur[k] = mfma16x16x32(w[I], xf[I % NX][k], cur[k]);
-#endif
-#if (defined(TT_EXP) && TT_EXP == 5) || defined(TT_NOH)
-            const int ctl = 0;
-#else
             const int ctl = __builtin_amdgcn_readfirstlane(c[I]);
-#endif
-            // pair q + I + TT_DEPTH (unconditional: the stream is followed by spare pairs)
-#if !(defined(TT_ABL) && (TT_ABL & 2))
+            // pair q + I + DEPTH (unconditional: the stream is followed by spare pairs)
             tt_load_pair(wp + I * 1024, rp + I * 16, lane_lo, lane_lw, w[I], o[I], c[I]);
-#endif
             if (ctl != 0)
                 at_end(ctl, [&]() {
 #pragma unroll
                     for (int i = 1; i <= TT_XA; i++)
-                        tt_read_x<RS>(xf[(I + i) % NX], xl, o[(I + i) % TT_DEPTH]);
+                        tt_read_x<RS, MS>(xf[(I + i) % NX], xl, o[(I + i) % DEPTH]);
                 });
         });
-        wp += TT_DEPTH * 1024;
-        rp += TT_DEPTH * 16;
+        wp += DEPTH * 1024;
+        rp += DEPTH * 16;
     }
 }
 
@@ -266,15 +265,14 @@ __device__ __forceinline__ void tt_add_tied(f32x4 &a, const f32x4 &c) {
 // acc[j] += cur for a wave-uniform run-time j (no accumulator for j >= NB).  A
 // sequence of independent ifs with something opaque between them: as an if /
 // else chain it becomes a switch whose lowering copies the accumulators around.
-template <int NB>
-__device__ __forceinline__ void tt_acc_add(f32x4 (&acc)[NB][4], int j, const f32x4 (&cur)[4]) {
+template <int NB, int MS>
+__device__ __forceinline__ void tt_acc_add(f32x4 (&acc)[NB][MS], int j, const f32x4 (&cur)[MS]) {
     tt_static_for<0, NB>([&](auto kc) {
         constexpr int k = decltype(kc)::value;
         if (j == k) {
-            tt_add_tied<k>(acc[k][0], cur[0]);
-            tt_add_tied<k>(acc[k][1], cur[1]);
-            tt_add_tied<k>(acc[k][2], cur[2]);
-            tt_add_tied<k>(acc[k][3], cur[3]);
+#pragma unroll
+            for (int ms = 0; ms < MS; ms++)
+                tt_add_tied<k>(acc[k][ms], cur[ms]);
         }
         asm volatile("; after case %0" ::"n"(k));
     });
@@ -353,10 +351,11 @@ __device__ __forceinline__ void tt_ln(f16x4 (&x)[TtGeom<D>::NB][NMS], int ms0,
     }
 }
 
-template <int D>
-__global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtArgs a) {
-    using G = TtGeom<D>;
+template <int D, int MS>
+__global__ void __launch_bounds__(TT_WAVES * 64, MS == 2 ? 4 : 1) tile_tail_pair_kernel(const TtArgs a) {
+    using G = TtGeom<D, MS>;
     constexpr int NB = G::NB, RS = G::RS, XW = G::XW, nbrD = D / 16;
+    constexpr int TT_BM = 16 * MS, TT_DEPTH = tt_depth(MS), HS = MS / 2; // rows; pairs in flight; subtiles per row-half
     extern __shared__ __attribute__((aligned(16))) unsigned char tt_smem[];
     char *const smem = reinterpret_cast<char *>(tt_smem);
     // the two workgroups of a panel get neighbouring slots of ONE XCD (hardware
@@ -373,16 +372,6 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
     unsigned *const ctr = reinterpret_cast<unsigned *>(smem + G::CT);
     int *const misc = reinterpret_cast<int *>(smem + G::MISC);
     const int nvalid = min(max(nbrD - NB * wave, 0), NB); // this wave's block-rows inside the matrix
-#ifdef TT_TRACE
-    long long tr_wait = 0, tr_hand = 0;
-    int tr_nh = 0;
-#define TT_STAMP(i_) if (lane == 0) a.trace[((size_t)vid * TT_WAVES + wave) * 16 + (i_)] = wall_clock64();
-#define TT_STAMPV(i_, v_) if (lane == 0) a.trace[((size_t)vid * TT_WAVES + wave) * 16 + (i_)] = (v_);
-#else
-#define TT_STAMP(i_)
-#define TT_STAMPV(i_, v_)
-#endif
-    TT_STAMP(0)
 
     // the panel (attention output): DMA, wave w takes rows w, w + 8, ...
     {
@@ -403,9 +392,9 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
         reinterpret_cast<float *>(smem + G::ZV)[tid - 64] = 0.f;
     {
         const int hb0 = half ? a.hb0[1] : a.hb0[0], nb1h = half ? a.nb1h[1] : a.nb1h[0];
-        float *bi = reinterpret_cast<float *>(smem + G::BI);
+        f16 *bi = reinterpret_cast<f16 *>(smem + G::BI);
         for (int i = tid; i < nb1h * 16; i += TT_WAVES * 64)
-            bi[i] = (float)a.bias1[hb0 * 16 + i];
+            bi[i] = a.bias1[hb0 * 16 + i];
     }
     typedef const __attribute__((address_space(4))) int *ScalarInts;
     const ScalarInts wt = (ScalarInts)a.wtab + (half * TT_WAVES + wave) * 8;
@@ -420,43 +409,34 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
         tt_load_pair(pairs + (size_t)(o_base + i) * 1024, recs + (size_t)(o_base + i) * 16, lane_lo, lane_lw, w[i],
                      o[i], c[i]);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's part of the panel has landed
-    TT_STAMP(1)
     __syncthreads();
-    TT_STAMP(2)
 
-    f32x4 acc[NB][4], cur[4];
+    f32x4 acc[NB][MS], cur[MS];
 #pragma unroll
     for (int j = 0; j < NB; j++)
 #pragma unroll
-        for (int ms = 0; ms < 4; ms++)
+        for (int ms = 0; ms < MS; ms++)
             acc[j][ms] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ms = 0; ms < 4; ms++)
+    for (int ms = 0; ms < MS; ms++)
         cur[ms] = f32x4{0.f, 0.f, 0.f, 0.f};
     const char *const xl = smem + c16 * RS + khalf8 * 2;
 
     // ---- the projection: this wave's NB block-rows over the whole panel ----
-    tt_stream<RS>(xl, pairs + (size_t)o_base * 1024, recs + (size_t)o_base * 16, o_n, lane_lo, lane_lw, w, o, c, cur,
-                  [&](int ctl, auto &&) {
-                      tt_acc_add<NB>(acc, (ctl >> 2) & 7, cur);
+    tt_stream<RS, MS, TT_DEPTH>(xl, pairs + (size_t)o_base * 1024, recs + (size_t)o_base * 16, o_n, lane_lo, lane_lw,
+                                w, o, c, cur, [&](int ctl, auto &&) {
+                                    tt_acc_add<NB, MS>(acc, (ctl >> 2) & 7, cur);
 #pragma unroll
-                      for (int ms = 0; ms < 4; ms++)
-                          cur[ms] = f32x4{0.f, 0.f, 0.f, 0.f};
-                  });
-    TT_STAMP(3)
-#if defined(TT_EXP) && (TT_EXP == 5 || TT_EXP == 6)
-    if (a.M > 0) {
-        a.Y[(size_t)m0 * D + tid] = (f16)(cur[0][0] + acc[0][0][0]);
-        return;
-    }
-#endif
+                                    for (int ms = 0; ms < MS; ms++)
+                                        cur[ms] = f32x4{0.f, 0.f, 0.f, 0.f};
+                                });
 
     // ---- bias + skip (the layer input) + LayerNorm 1, written over the panel ----
     {
         // every operand is requested before any is used, from addresses that are
         // legal for all lanes (block-rows beyond the matrix read column 0 and are
         // zeroed afterwards): one memory latency for the whole step
-        f16x4 x[NB][4], gam[NB], bet[NB], bo[NB];
+        f16x4 x[NB][MS], gam[NB], bet[NB], bo[NB];
 #pragma unroll
         for (int j = 0; j < NB; j++) {
             const int col = j < nvalid ? (NB * wave + j) * 16 + g4 * 4 : 0;
@@ -464,7 +444,7 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
             gam[j] = *reinterpret_cast<const f16x4 *>(a.g1 + col);
             bet[j] = *reinterpret_cast<const f16x4 *>(a.b1 + col);
 #pragma unroll
-            for (int ms = 0; ms < 4; ms++)
+            for (int ms = 0; ms < MS; ms++)
                 x[j][ms] = *reinterpret_cast<const f16x4 *>(
                     a.input + (size_t)min(m0 + 16 * ms + c16, a.M - 1) * D + col);
         }
@@ -473,79 +453,62 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
             const f32x4 bf = __builtin_convertvector(bo[j], f32x4);
             const f16x4 zero = f16x4{0, 0, 0, 0};
 #pragma unroll
-            for (int ms = 0; ms < 4; ms++) {
+            for (int ms = 0; ms < MS; ms++) {
                 // half(acc + bias) is the linear's output as the reference stores it; the
                 // skip connection is added in half (kernels/skip_layernorm.cu:20)
                 const f16x4 v = __builtin_convertvector(acc[j][ms] + bf, f16x4) + x[j][ms];
                 x[j][ms] = j < nvalid ? v : zero;
             }
         }
-        TT_STAMP(13)
         // the first pairs of the feed-forward stream travel under the LayerNorm
 #pragma unroll
         for (int i = 0; i < TT_DEPTH; i++)
             tt_load_pair(pairs + (size_t)(f_base + i) * 1024, recs + (size_t)(f_base + i) * 16, lane_lo, lane_lw,
                          w[i], o[i], c[i]);
-        TT_STAMP(14)
-        tt_ln<D, 4>(x, 0, gam, bet, smem, wave, c16, g4, nvalid);
-        TT_STAMP(15)
+        tt_ln<D, MS>(x, 0, gam, bet, smem, wave, c16, g4, nvalid);
         // (every wave has passed a barrier since its last read of the attention panel)
 #pragma unroll
         for (int j = 0; j < NB; j++)
             if (j < nvalid)
 #pragma unroll
-                for (int ms = 0; ms < 4; ms++)
+                for (int ms = 0; ms < MS; ms++)
                     *reinterpret_cast<f16x4 *>(smem + (16 * ms + c16) * RS + ((NB * wave + j) * 16 + g4 * 4) * 2) =
                         x[j][ms];
     }
 #pragma unroll
     for (int j = 0; j < NB; j++)
 #pragma unroll
-        for (int ms = 0; ms < 4; ms++)
+        for (int ms = 0; ms < MS; ms++)
             acc[j][ms] = f32x4{0.f, 0.f, 0.f, 0.f};
-    TT_STAMP(4)
     __syncthreads(); // the feed-forward input panel is complete
-    TT_STAMP(5)
-#if defined(TT_EXP) && TT_EXP == 1
-    return;
-#endif
 
     // ---- the feed-forward block over this half of the hidden columns ----
     {
         auto start_vector = [&](int idx) { // what a segment's sums start from: zeros or a hidden block-row's bias
             f32x4 init = f32x4{0.f, 0.f, 0.f, 0.f};
             if (idx != 255) // (most segments start from zeros: no LDS round trip for those)
-                init = *reinterpret_cast<const f32x4 *>(smem + G::BI + idx * 64 + g4 * 16);
+                init = __builtin_convertvector(
+                    *reinterpret_cast<const f16x4 *>(smem + G::BI + idx * TT_BI_BYTES + g4 * 8), f32x4);
 #pragma unroll
-            for (int ms = 0; ms < 4; ms++)
+            for (int ms = 0; ms < MS; ms++)
                 cur[ms] = init;
         };
         start_vector(f_init);
         if (f_wait0 >= 0)
             tt_wait(ctr + (f_wait0 & 15), (unsigned)(f_wait0 >> 8), a.spin, a.status, lane);
-        tt_stream<RS>(
+        tt_stream<RS, MS, TT_DEPTH>(
             xl, pairs + (size_t)f_base * 1024, recs + (size_t)f_base * 16, f_n, lane_lo, lane_lw, w, o, c, cur,
             [&](int ctl, auto &&reread) {
-#ifdef TT_TRACE
-                const long long th0 = wall_clock64();
-                tr_nh++;
-#endif
                 const int p = (ctl >> 9) & 15;
                 if (ctl & TT_C_HID) {
                     // a finished hidden block-row (its bias was the starting value): GELU,
                     // rounded to half as the reference stores it, into the hidden buffer
                     if (ctl & TT_C_WAITF) { // ... once everyone has finished reading what it held before
-#ifdef TT_TRACE
-                        const long long tw0 = wall_clock64();
-#endif
                         tt_wait(ctr + TT_MAX_PHASES + p - 2, TT_WAVES, a.spin, a.status, lane);
-#ifdef TT_TRACE
-                        tr_wait += wall_clock64() - tw0;
-#endif
                     }
                     char *hp = smem + c16 * RS + (XW + (p & 1) * TT_HW + ((ctl >> 5) & 15) * 32) + g4 * 8;
 #pragma unroll
-                    for (int ms = 0; ms < 4; ms++) {
+                    for (int ms = 0; ms < MS; ms++) {
                         *reinterpret_cast<f16x4 *>(hp + ms * 16 * RS) =
                             gelu4(__builtin_convertvector(cur[ms], f16x4));
                         __builtin_amdgcn_sched_barrier(0); // one subtile at a time: few temporaries
@@ -554,34 +517,18 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
                 // (not in an else branch: as a part of that if / else the accumulators were
                 // given a second set of registers behind the handler; a hidden block-row's
                 // control word names accumulator 7, which does not exist)
-                tt_acc_add<NB>(acc, (ctl >> 2) & 7, cur);
+                tt_acc_add<NB, MS>(acc, (ctl >> 2) & 7, cur);
                 if (ctl & TT_C_SIG)
                     tt_signal(ctr + ((ctl & TT_C_HID) ? p : TT_MAX_PHASES + p), lane);
                 if (ctl & TT_C_WAITN) {
                     // the next segment multiplies a hidden buffer: wait until it is complete
                     // and read the next pair's fragments again
-#ifdef TT_TRACE
-                    const long long tw0 = wall_clock64();
-#endif
                     tt_wait(ctr + ((ctl >> 16) & 15), (unsigned)((ctl >> 20) & 15) + 1u, a.spin, a.status, lane);
-#ifdef TT_TRACE
-                    tr_wait += wall_clock64() - tw0;
-#endif
                     reread();
                 }
                 start_vector((int)((unsigned)ctl >> 24));
-#ifdef TT_TRACE
-                tr_hand += wall_clock64() - th0;
-#endif
             });
     }
-    TT_STAMP(6)
-    TT_STAMPV(10, tr_wait)
-    TT_STAMPV(11, tr_hand)
-    TT_STAMPV(12, tr_nh)
-#if defined(TT_EXP) && TT_EXP == 2
-    return;
-#endif
 
     // ---- the two halves' partial sums meet; bias + skip + LayerNorm 2; store ----
     f16x4 b2[NB], gam[NB], bet[NB];
@@ -600,19 +547,20 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
     // write-back and invalidation of the whole L2 as a device-scope fence would.
     // Order: all waves wait for their stores, barrier, THEN thread 0 touches the
     // counter; a reader loads only after the barrier behind thread 0's counter read.
-    constexpr size_t PART = (size_t)TT_WAVES * NB * 2 * 2 * 64; // words per (panel, half, row-half)
+    constexpr size_t PART = (size_t)TT_WAVES * NB * HS * 2 * 64; // words per (panel, half, row-half)
     auto publish = [&](int h) {
-        unsigned long long *dst = a.ws + ((size_t)(panel * 2 + half) * 2 + h) * PART + (size_t)wave * NB * 4 * 64 + lane;
+        unsigned long long *dst =
+            a.ws + ((size_t)(panel * 2 + half) * 2 + h) * PART + (size_t)wave * NB * HS * 2 * 64 + lane;
 #pragma unroll
         for (int j = 0; j < NB; j++)
 #pragma unroll
-            for (int m2 = 0; m2 < 2; m2++) {
-                const f32x4 v = h ? acc[j][2 + m2] : acc[j][m2]; // (selected, not indexed: acc stays in registers)
+            for (int m2 = 0; m2 < HS; m2++) {
+                const f32x4 v = h ? acc[j][HS + m2] : acc[j][m2]; // (selected, not indexed: acc stays in registers)
                 typedef float f32x2 __attribute__((ext_vector_type(2)));
-                __hip_atomic_store(dst + ((j * 2 + m2) * 2 + 0) * 64,
+                __hip_atomic_store(dst + ((j * HS + m2) * 2 + 0) * 64,
                                    __builtin_bit_cast(unsigned long long, f32x2{v[0], v[1]}), __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(dst + ((j * 2 + m2) * 2 + 1) * 64,
+                __hip_atomic_store(dst + ((j * HS + m2) * 2 + 1) * 64,
                                    __builtin_bit_cast(unsigned long long, f32x2{v[2], v[3]}), __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
             }
@@ -620,47 +568,47 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
     };
     auto finish = [&](int h) {
         const unsigned long long *src =
-            a.ws + ((size_t)(panel * 2 + (1 - half)) * 2 + h) * PART + (size_t)wave * NB * 4 * 64 + lane;
+            a.ws + ((size_t)(panel * 2 + (1 - half)) * 2 + h) * PART + (size_t)wave * NB * HS * 2 * 64 + lane;
         typedef float f32x2 __attribute__((ext_vector_type(2)));
-        f32x4 other[NB][2];
+        f32x4 other[NB][HS];
 #pragma unroll
         for (int j = 0; j < NB; j++)
 #pragma unroll
-            for (int m2 = 0; m2 < 2; m2++) {
+            for (int m2 = 0; m2 < HS; m2++) {
                 const f32x2 lo = __builtin_bit_cast(
-                    f32x2, __hip_atomic_load(src + ((j * 2 + m2) * 2 + 0) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                    f32x2, __hip_atomic_load(src + ((j * HS + m2) * 2 + 0) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
                 const f32x2 hi2 = __builtin_bit_cast(
-                    f32x2, __hip_atomic_load(src + ((j * 2 + m2) * 2 + 1) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                    f32x2, __hip_atomic_load(src + ((j * HS + m2) * 2 + 1) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
                 other[j][m2] = f32x4{lo[0], lo[1], hi2[0], hi2[1]};
             }
-        f16x4 x[NB][2];
+        f16x4 x[NB][HS];
 #pragma unroll
         for (int j = 0; j < NB; j++) {
             const f32x4 bf = __builtin_convertvector(b2[j], f32x4);
             const f16x4 zero = f16x4{0, 0, 0, 0};
 #pragma unroll
-            for (int m2 = 0; m2 < 2; m2++) {
+            for (int m2 = 0; m2 < HS; m2++) {
                 const int col = j < nvalid ? (NB * wave + j) * 16 + g4 * 4 : 0;
-                const f16x4 sk = *reinterpret_cast<const f16x4 *>(smem + (16 * (2 * h + m2) + c16) * RS + col * 2);
-                const f32x4 mine = h ? acc[j][2 + m2] : acc[j][m2];
+                const f16x4 sk = *reinterpret_cast<const f16x4 *>(smem + (16 * (HS * h + m2) + c16) * RS + col * 2);
+                const f32x4 mine = h ? acc[j][HS + m2] : acc[j][m2];
                 const f16x4 v = __builtin_convertvector((mine + other[j][m2]) + bf, f16x4) + sk;
                 x[j][m2] = j < nvalid ? v : zero;
             }
         }
-        tt_ln<D, 2>(x, 2 * h, gam, bet, smem, wave, c16, g4, nvalid);
+        tt_ln<D, HS>(x, HS * h, gam, bet, smem, wave, c16, g4, nvalid);
         // in place over the skip operand (each lane overwrites what it read), then
         // whole rows leave with 16-byte stores
 #pragma unroll
         for (int j = 0; j < NB; j++)
             if (j < nvalid)
 #pragma unroll
-                for (int m2 = 0; m2 < 2; m2++)
-                    *reinterpret_cast<f16x4 *>(smem + (16 * (2 * h + m2) + c16) * RS +
+                for (int m2 = 0; m2 < HS; m2++)
+                    *reinterpret_cast<f16x4 *>(smem + (16 * (HS * h + m2) + c16) * RS +
                                                ((NB * wave + j) * 16 + g4 * 4) * 2) = x[j][m2];
         __syncthreads();
         constexpr int PR = D / 8;
-        for (int i = tid; i < 32 * PR; i += TT_WAVES * 64) {
-            const int r = 32 * h + i / PR, cc = i % PR;
+        for (int i = tid; i < 16 * HS * PR; i += TT_WAVES * 64) {
+            const int r = 16 * HS * h + i / PR, cc = i % PR;
             if (m0 + r < a.M)
                 *reinterpret_cast<u32x4 *>(a.Y + (size_t)(m0 + r) * D + cc * 8) =
                     *reinterpret_cast<const u32x4 *>(smem + r * RS + cc * 16);
@@ -671,7 +619,6 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
     const int other_h = 1 - half;
     publish(other_h); // the partner finishes that row-half unless it has long gone
     __syncthreads();  // (also: every wave has left the hidden buffers)
-    TT_STAMP(7)
     if (tid == 0) {
         // one round trip: arrive at the other row-half's counter, look at the own one
         misc[0] = __hip_atomic_fetch_add(a.sync + 2 * panel + other_h, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -689,14 +636,12 @@ __global__ void __launch_bounds__(TT_WAVES * 64) tile_tail_pair_kernel(const TtA
         __syncthreads();
         arrived_own = misc[2];
     }
-    TT_STAMP(8)
     if (arrived_own != 0)
         finish(half);
     if (arrived_other != 0) {
         __syncthreads(); // (the statistics area and the broadcast words are free again)
         finish(other_h);
     }
-    TT_STAMP(9)
 }
 
 // ---------------------------------------------------------------------------
@@ -707,7 +652,6 @@ struct TailProgram {
     int nphase[2] = {0, 0}, hb0[2] = {0, 0}, nb1h[2] = {0, 0};
     f16 *d_pairs = nullptr;
     int *d_rec = nullptr, *d_wtab = nullptr, *d_sync = nullptr;
-    size_t lds_bytes = 0;
     size_t npairs = 0; // including padding (for reports)
 };
 
@@ -721,12 +665,10 @@ void tail_program_destroy(TailProgram *p) {
     delete p;
 }
 
-#ifdef TT_TRACE
-long long *g_tt_trace = nullptr;
-#endif
-// et_tuning_set("tile_tail_pair"): 0 never (default: at BERT-base / 80 % / 8192 rows the paired form takes 69 us
-// against 55 us of the one-workgroup form), 1 where there are enough panels, 2 wherever it applies
+// et_tuning_set("tile_tail_pair"): 0 never, 1 where there are enough panels (32-row panels), 2 wherever it
+// applies with 64-row panels, 3 wherever it applies with 32-row panels
 static int g_tail_pair = 0;
+static int tail_ms() { return g_tail_pair == 2 ? 4 : 2; } // 16-row subtiles per panel
 static int g_tail_spin = 1 << 22;    // et_tuning_set("tile_wait_spin"): polls before a bounded LDS wait gives up
 void set_tail_pair(int v) { g_tail_pair = v; }
 bool tail_pair_forced() { return g_tail_pair >= 2; }
@@ -739,6 +681,11 @@ static int tail_geom(int D, int *nb, int *xw) {
     *nb = (D / 16 + TT_WAVES - 1) / TT_WAVES;
     *xw = (D + ((D & 31) ? 0 : 16)) * 2;
     return 1;
+}
+
+// LDS bytes of a workgroup: the rows, the event counters, zeros and broadcast words, the first linear's bias
+static size_t tail_lds_bytes(int xw, int ms, int nb1h) {
+    return (size_t)16 * ms * (xw + 2 * TT_HW) + 2 * TT_MAX_PHASES * 4 + 128 + (size_t)nb1h * TT_BI_BYTES;
 }
 
 // which panel widths the kernel is built for
@@ -757,16 +704,21 @@ bool tail_pair_applies(const et_tile_plan *pO, const et_tile_plan *p1, const et_
     int nb, xw;
     if (!tail_geom(D, &nb, &xw))
         return false;
-    const size_t lds = (size_t)TT_BM * (xw + 2 * TT_HW) + 2 * TT_MAX_PHASES * 4 + 128 + (size_t)per_half * TT_HB * 64;
-    return lds <= 160 * 1024;
+    return tail_lds_bytes(xw, tail_ms(), per_half * TT_HB) <= 160 * 1024;
 }
 
 size_t tail_ws_bytes_for(int D, int rows) {
     int nb, xw;
     if (rows <= 0 || !tail_width_built(D) || !tail_geom(D, &nb, &xw))
         return 0;
-    const size_t npanels = ((size_t)rows + TT_BM - 1) / TT_BM;
-    return npanels * 4 * ((size_t)TT_WAVES * nb * 2 * 64 * 4) * sizeof(float);
+    // per (panel, half, row-half): waves x block-rows x subtiles of the row-half x 64 lanes x 4 floats; enough
+    // for either panel height
+    size_t need = 0;
+    for (int ms = 2; ms <= 4; ms += 2) {
+        const size_t npanels = ((size_t)rows + 16 * ms - 1) / (16 * ms);
+        need = std::max(need, npanels * 4 * ((size_t)TT_WAVES * nb * (ms / 2) * 64 * 4) * sizeof(float));
+    }
+    return need;
 }
 
 size_t tail_pair_ws_bytes(const et_tile_plan *pO, const et_tile_plan *p1, const et_tile_plan *p2, int M) {
@@ -850,7 +802,7 @@ int tail_pair_prepare(const et_tile_plan *pO, const et_tile_plan *p1, et_tile_pl
     const int D = pO->out_feat, Hd = p1->out_feat, nbrD = D / 16, nbr1 = Hd / 16;
     int NB, XW;
     tail_geom(D, &NB, &XW);
-    const int RS = XW + 2 * TT_HW, CT = TT_BM * RS, ZV = CT + 2 * TT_MAX_PHASES * 4, BI = ZV + 128;
+    const int RS = XW + 2 * TT_HW;
     const int nchunk = (Hd + TT_HC - 1) / TT_HC;
     TailProgram *P = new TailProgram();
     P->D = D;
@@ -862,7 +814,6 @@ int tail_pair_prepare(const et_tile_plan *pO, const et_tile_plan *p1, et_tile_pl
         P->hb0[h] = c0[h] * TT_HB;
         P->nb1h[h] = std::min(nbr1, (c0[h] + P->nphase[h]) * TT_HB) - P->hb0[h];
     }
-    P->lds_bytes = (size_t)BI + (size_t)std::max(P->nb1h[0], P->nb1h[1]) * 64;
 
     ProgBuilder B;
     std::vector<int> wtab(2 * TT_WAVES * 8, 0);
@@ -881,7 +832,7 @@ int tail_pair_prepare(const et_tile_plan *pO, const et_tile_plan *p1, et_tile_pl
                     segs.push_back(Segment{(int)(B.npairs() - base), false, j, 0, 0, false, false, 255, -1, 0});
             }
             if (!segs.empty()) {
-                while ((B.npairs() - base) % TT_DEPTH)
+                while ((B.npairs() - base) % TT_PAD)
                     B.add_zero_pair(0);
                 segs.back().end = (int)(B.npairs() - base); // the padding belongs to the last segment
             }
@@ -933,7 +884,7 @@ int tail_pair_prepare(const et_tile_plan *pO, const et_tile_plan *p1, et_tile_pl
                     first(p + 1);
                 second(p);
             }
-            while ((B.npairs() - base) % TT_DEPTH)
+            while ((B.npairs() - base) % TT_PAD)
                 B.add_zero_pair(XW + ((np - 1) & 1) * TT_HW);
             segs.back().end = (int)(B.npairs() - base);
             wt[3] = (int)(B.npairs() - base);
@@ -942,7 +893,7 @@ int tail_pair_prepare(const et_tile_plan *pO, const et_tile_plan *p1, et_tile_pl
             B.seal(base, segs);
         }
     P->npairs = B.npairs();
-    for (int i = 0; i < 2 * TT_DEPTH; i++) // the last stages of a stream request up to TT_DEPTH - 1 pairs past its end
+    for (int i = 0; i < 2 * TT_PAD; i++) // the last stages of a stream request up to depth - 1 pairs past its end
         B.add_zero_pair(0);
     // every offset must address the panel or a hidden buffer of the lane's row
     for (size_t q = 0; q < B.npairs(); q++)
@@ -994,9 +945,9 @@ static hipError_t tt_allow_lds(size_t lds) {
     return e;
 }
 
-template <int D>
+template <int D, int MS>
 static int tt_launch(const TtArgs &a, size_t lds, hipStream_t st) {
-    constexpr auto k = &tile_tail_pair_kernel<D>;
+    constexpr auto k = &tile_tail_pair_kernel<D, MS>;
     ET_HIP(tt_allow_lds<k>(lds));
     hipLaunchKernelGGL(k, dim3(a.per_xcd * 8), dim3(TT_WAVES * 64), lds, st, a);
     return launch_status("layer tail (pairs) launch");
@@ -1008,9 +959,10 @@ int tail_pair_launch(const et_tile_plan *pO, const et_tile_plan *p1, const et_ti
     const TailProgram *P = p2->tail;
     ET_REQUIRE(P && p2->tail_uid[0] == pO->uid && p2->tail_uid[1] == p1->uid, ET_ERR_INVALID_ARG,
                "layer tail (pairs): no program for these plans (et_tile_plan_tail_prepare)");
-    const int npanels = (M + TT_BM - 1) / TT_BM;
+    const int ms = tail_ms(), bm = 16 * ms;
+    const int npanels = (M + bm - 1) / bm;
     ET_REQUIRE(npanels <= TT_MAX_PANELS, ET_ERR_UNSUPPORTED, "layer tail (pairs): %d rows, at most %d", M,
-               TT_MAX_PANELS * TT_BM);
+               TT_MAX_PANELS * bm);
     ET_REQUIRE(ws && aligned16(ws), ET_ERR_INVALID_ARG, "layer tail (pairs): scratch missing or misaligned");
     int *status = wait_status_device();
     ET_REQUIRE(status, ET_ERR_HIP, "layer tail (pairs): no wait-status word");
@@ -1043,19 +995,16 @@ int tail_pair_launch(const et_tile_plan *pO, const et_tile_plan *p1, const et_ti
         a.hb0[h] = P->hb0[h];
         a.nb1h[h] = P->nb1h[h];
     }
-#ifdef TT_TRACE
-    {
-        static long long *trace = nullptr;
-        if (!trace)
-            (void)hipMalloc(&trace, (size_t)4096 * TT_WAVES * 16 * 8);
-        a.trace = trace;
-        g_tt_trace = trace;
-    }
-#endif
-    switch (P->D) {
-    case 768: return tt_launch<768>(a, P->lds_bytes, st);
-    case 512: return tt_launch<512>(a, P->lds_bytes, st);
-    case 256: return tt_launch<256>(a, P->lds_bytes, st);
+    int nb, xw;
+    tail_geom(P->D, &nb, &xw);
+    const size_t lds = tail_lds_bytes(xw, ms, std::max(P->nb1h[0], P->nb1h[1]));
+    switch (P->D * 8 + ms) {
+    case 768 * 8 + 4: return tt_launch<768, 4>(a, lds, st);
+    case 512 * 8 + 4: return tt_launch<512, 4>(a, lds, st);
+    case 256 * 8 + 4: return tt_launch<256, 4>(a, lds, st);
+    case 768 * 8 + 2: return tt_launch<768, 2>(a, lds, st);
+    case 512 * 8 + 2: return tt_launch<512, 2>(a, lds, st);
+    case 256 * 8 + 2: return tt_launch<256, 2>(a, lds, st);
     default: break;
     }
     set_error("layer tail (pairs): width %d is not built", P->D);
@@ -1063,8 +1012,3 @@ int tail_pair_launch(const et_tile_plan *pO, const et_tile_plan *p1, const et_ti
 }
 
 } // namespace et
-#ifdef TT_TRACE
-extern "C" int et_tt_trace_read(long long *host, int nwg) {
-    return hipMemcpy(host, et::g_tt_trace, (size_t)nwg * et::TT_WAVES * 16 * 8, hipMemcpyDeviceToHost) == hipSuccess ? 0 : -1;
-}
-#endif

@@ -275,12 +275,13 @@ int et_tile_plan_run_tail(const et_tile_plan *out, const et_tile_plan *first,
 int et_tile_plan_tail_fusable(const et_tile_plan *out, const et_tile_plan *first,
                               const et_tile_plan *second);
 /* The same five steps with device scratch from the caller, which opens a second
- * form of the launch: PAIRS of workgroups over 64-row panels.  Both workgroups
- * of a pair run the projection and the first LayerNorm on the panel, each takes
- * one half of the hidden columns of the feed-forward block, and their fp32
- * partial sums meet in `ws` (whoever arrives second at a row-half's counter
- * finishes it: no workgroup waits for another).  A CU then streams half the
- * weights per row.  Taken only when switched on (et_tuning_set
+ * form of the launch: PAIRS of workgroups over 64-row or 32-row panels.  Both
+ * workgroups of a pair run the projection and the first LayerNorm on the panel,
+ * each takes one half of the hidden columns of the feed-forward block, and
+ * their fp32 partial sums meet in `ws` (whoever arrives second at a row-half's
+ * counter finishes it: no workgroup waits for another).  With 64-row panels a
+ * CU streams half the weights per row; with 32-row panels two workgroups share
+ * a CU.  Taken only when switched on (et_tuning_set
  * "tile_tail_pair"), where it applies (model width 256, 512 or 768, hidden
  * width a multiple of 16 and at least 384), ws_bytes >=
  * et_tile_plan_tail_ws_bytes(out, first, second, M) and there are enough row
@@ -470,7 +471,8 @@ int et_device_synchronize(void);
  *   "tile_tail_pair"  0 (default): et_tile_plan_run_tail_ws never takes the paired
  *                     form (measured slower than the one-workgroup form on the
  *                     BERT-base shapes); 1: where it applies and there are
- *                     enough row panels; 2: wherever it applies
+ *                     enough row panels (32-row panels); 2: wherever it applies,
+ *                     64-row panels; 3: wherever it applies, 32-row panels
  *   "tile_tail_pair_min_wgs" fewest workgroups (two per 64-row panel) for the
  *                     paired form (default: three quarters of the CUs)
  *   "tile_wait_spin"  polls after which a bounded wait inside a workgroup gives

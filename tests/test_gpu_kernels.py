@@ -303,9 +303,10 @@ PAIR_CASES = [
 ]
 
 
+@pytest.mark.parametrize("mode", [2, 3])
 @pytest.mark.parametrize("M,d,F,sp", PAIR_CASES)
-def test_tile_layer_tail_pairs(K, M, d, F, sp):
-    """the layer tail as pairs of workgroups over 64-row panels (scratch given, mid=None insists on it) == the
+def test_tile_layer_tail_pairs(K, M, d, F, sp, mode):
+    """the layer tail as pairs of workgroups over 64-row (mode 2) or 32-row (mode 3) panels (scratch given, mid=None insists on it) == the
     oracle's chain of five steps; a second run on the same plans (the per-panel counters reset themselves) and a
     run whose output overwrites the attention buffer give the same bits; close to the one-workgroup form"""
     from et_amd.encoder import Linear_tile
@@ -326,13 +327,13 @@ def test_tile_layer_tail_pairs(K, M, d, F, sp):
     from et_amd import lib
     ln = [dev(t) for t in (g1, b1, g2, b2)]
     assert Linear_tile.tail_ws_bytes(to, t1, t2, M) == 0          # the paired form is off by default
-    lib().et_tuning_set(b"tile_tail_pair", 2)
+    lib().et_tuning_set(b"tile_tail_pair", mode)
     try:
         need = Linear_tile.tail_ws_bytes(to, t1, t2, M)
-        assert need == ((M + 63) // 64) * 64 * (-(-d // 192) * 192) * 4 * 2   # twelve waves x block-rows per wave x 16 columns
+        assert need == ((M + 63) // 64) * 64 * (-(-d // 128) * 128) * 4 * 2   # eight waves x block-rows per wave x 16 columns
         Linear_tile.tail_prepare(to, t1, t2)
         ws = torch.full((need,), 0xFF, dtype=torch.uint8, device="cuda")   # NaN patterns: nothing may be read before written
-        print(f"pair tail: M={M} d={d} F={F} sp={sp}", flush=True)
+        print(f"pair tail: M={M} d={d} F={F} sp={sp} mode={mode}", flush=True)
         got = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln, ws=ws))
         check_close(got, want, max_abs=3e-2, mean_rel=2e-3, what="paired layer tail vs oracle chain")
         again = host(Linear_tile.run_tail(to, t1, t2, dev(attn), dev(inp), *ln, ws=ws))
