@@ -262,10 +262,22 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
 
         f32x4 ot[DV][QS];
         float m_run[QS];
+        // What the key-tile loop needs of m_run in every tile, kept as state and touched only where a
+        // maximum is raised (after the first tiles: almost never): the start vector of the score
+        // products, four copies of -m (zero while the row has no maximum yet), and the amount a
+        // tile's maximum has to exceed before the row's is raised (-inf until then, 8 binades after).
+        // Only the plain form keeps them (there they save a dozen vector instructions per tile); with
+        // mask handling they would be ten registers too many for three waves per SIMD, and the masked
+        // forms work both out from m_run in every tile.
+        constexpr bool KEEP_START = PLAIN;
+        f32x4 neg_m4[QS];
+        float raise_over[QS];
         f32x4 l_acc[QS]; // row sums of P, accumulated by the matrix unit (all 16 rows of the tile equal)
 #pragma unroll
         for (int qs = 0; qs < QS; qs++) {
             m_run[qs] = -INFINITY;
+            neg_m4[qs] = f32x4{-0.f, -0.f, -0.f, -0.f};
+            raise_over[qs] = -INFINITY;
             l_acc[qs] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int d = 0; d < DV; d++)
@@ -555,13 +567,17 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
             // ALU one subtraction per score
             f32x4 st[4][QS];
             float m_ref[QS];
-#pragma unroll
-            for (int qs = 0; qs < QS; qs++)
-                m_ref[qs] = (m_run[qs] == -INFINITY) ? 0.f : m_run[qs];
             f32x4 nm4[QS];
 #pragma unroll
-            for (int qs = 0; qs < QS; qs++)
-                nm4[qs] = f32x4{-m_ref[qs], -m_ref[qs], -m_ref[qs], -m_ref[qs]};
+            for (int qs = 0; qs < QS; qs++) {
+                if (KEEP_START) {
+                    nm4[qs] = neg_m4[qs];
+                    m_ref[qs] = -nm4[qs][0]; // (only used where a maximum is raised)
+                } else {
+                    m_ref[qs] = (m_run[qs] == -INFINITY) ? 0.f : m_run[qs];
+                    nm4[qs] = f32x4{-m_ref[qs], -m_ref[qs], -m_ref[qs], -m_ref[qs]};
+                }
+            }
             if (!SHAREDQK) {
                 // K fragments are read one 16-key subtile ahead of the MFMAs that
                 // use them (two subtiles' worth of registers instead of four)
@@ -693,16 +709,25 @@ __device__ __forceinline__ void attention_block(const AttnArgs &a, const int b, 
 #pragma unroll
             for (int qs = 0; qs < QS; qs++) {
                 float mx = pmx[qs];
-                // (a row without a maximum yet, m_run = -inf, takes its first finite one)
-                const bool up_lane = (m_run[qs] == -INFINITY) ? (mx > -INFINITY) : (mx * ls > 8.0f);
+                // (a row without a maximum yet takes its first finite one: raise_over is -inf then)
+                auto raises = [&](float v) {
+                    if (KEEP_START)
+                        return v * ls > raise_over[qs];
+                    return (m_run[qs] == -INFINITY) ? (v > -INFINITY) : (v * ls > 8.0f);
+                };
+                const bool up_lane = raises(mx);
                 if (__builtin_amdgcn_ballot_w64(up_lane) != 0) {
                     mx = xor_max_16_32(mx);
-                    const bool up = (m_run[qs] == -INFINITY) ? (mx > -INFINITY) : (mx * ls > 8.0f);
+                    const bool up = raises(mx);
                     const float m_new = up ? mx + m_ref[qs] : m_run[qs];
                     const float m_fin = (m_new == -INFINITY) ? 0.f : m_new;
                     const float alpha = __builtin_amdgcn_exp2f((m_run[qs] - m_fin) * ls); // 1 where unchanged
                     const float shift = m_fin - m_ref[qs];                                // 0 where unchanged
                     m_run[qs] = m_new;
+                    if (KEEP_START) {
+                        neg_m4[qs] = f32x4{-m_fin, -m_fin, -m_fin, -m_fin};
+                        raise_over[qs] = (m_new == -INFINITY) ? -INFINITY : 8.0f;
+                    }
                     l_acc[qs] *= alpha;
 #pragma unroll
                     for (int d = 0; d < DV; d++)
