@@ -30,7 +30,11 @@ __device__ __forceinline__ f16x8 ln_load(const f16 *row, int chunk) {
 // whose operands exceed the last-level cache (streaming from HBM: 131072 rows
 // of 768 98 -> 85 us); smaller ones are faster with ordinary loads (their
 // operands are usually still cached from the kernel that produced them).
-template <int NCH, int ROWS, bool NT>
+// NTS: the rows are also stored with the non-temporal hint - where the in/out
+// operand alone is well beyond the last-level cache (524288 rows of 768:
+// 440 -> 376 us, 5.5 -> 6.4 TB/s; up to 300 MB per operand the plain store is
+// 2-4 % faster).
+template <int NCH, int ROWS, bool NT, bool NTS = false>
 __global__ void __launch_bounds__(256)
 skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip,
                           const f16 *__restrict__ gamma,
@@ -121,8 +125,12 @@ skip_layernorm_vec_kernel(f16 *__restrict__ in_out, const f16 *__restrict__ skip
 #pragma unroll
             for (int j = 0; j < CW; j++) // ((x - mean) * rstd) * gamma + beta, the first step as one fma
                 y[j] = (f16)(__builtin_fmaf((float)x[i][j], rstd, shift) * (float)gg[i][j] + (float)bb[i][j]);
-            if (i < NCH - 1 || last_ok)
-                a[ci[i]] = y;
+            if (i < NCH - 1 || last_ok) {
+                if (NTS)
+                    __builtin_nontemporal_store(__builtin_bit_cast(u32x4, y), reinterpret_cast<u32x4 *>(a) + ci[i]);
+                else
+                    a[ci[i]] = y;
+            }
         }
     }
 }
@@ -282,11 +290,16 @@ extern "C" int et_skip_layernorm(void *in_out, const void *skip, const void *gam
         // (four rows per wave measured 4-5 % slower from 131072 rows up)
         // both operands together beyond the 256 MB last-level cache: streaming loads, two rows per wave
         const bool nt = g_ln_rows == 0 && (size_t)num * size * 4 > (size_t)256 << 20;
+        // the in/out operand alone well beyond it (measured at 768 halves per row: 302 MB are 4 % faster
+        // with plain stores, 403 MB 17 % faster with non-temporal ones)
+        const bool nts = nt && (size_t)num * size * 2 > (size_t)320 << 20;
         const int rows = nt ? 2 : g_ln_rows > 0 ? g_ln_rows : (num >= 2 * 8192 ? 2 : 1);
         const dim3 grid((num + 4 * rows - 1) / (4 * rows));
 #define ET_LN_CASE(NCH_)                                                                          \
     {                                                                                             \
-    if (nt)                                                                                       \
+    if (nts)                                                                                      \
+        hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 2, true, true>), grid, block, 0, st, a, s, g, b, num, size, inv_n); \
+    else if (nt)                                                                                  \
         hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 2, true>), grid, block, 0, st, a, s, g, b, num, size, inv_n); \
     else if (rows >= 4)                                                                           \
         hipLaunchKernelGGL((skip_layernorm_vec_kernel<NCH_, 4, false>), grid, block, 0, st, a, s, g, b, num, size, inv_n); \
