@@ -445,6 +445,16 @@ def second_targets(torch, K, dev, enc, out, x, B, S, mask_h, lins, ln):
     wsp = torch.empty(Encoder_tile.buffer_size(D, S, H, B) // 2, dtype=torch.float16, device=dev)
     encp = Encoder_tile(D, S, H, wsp, *Lp, *ln, pm, B)
     res["latency_us_padding_mask"] = round(event_time(torch, lambda: encp.run(out, x), reps=50), 1)
+    # ... and checked: its first and last sequence against the oracle with the same mask
+    import oracle.et_oracle as orc          # checker only
+    x_h = x.cpu().numpy()
+    sample = sorted({0, B - 1})
+    srows = np.concatenate([np.arange(b * S, (b + 1) * S) for b in sample])
+    got = out.float().cpu().numpy()[srows]
+    want = orc.encoder_tile_layer(x_h[srows], lins, ln, pm, S, H, len(sample), None, 1.0).astype(np.float32)
+    res["parity_vs_oracle_padding_mask"] = {"max_abs": round(float(np.abs(got - want).max()), 5),
+                                            "mean_rel": round(float(np.abs(got - want).mean() / np.abs(want).mean()), 6),
+                                            "rows": int(srows.size), "sequences": sample}
     # the headline layer replayed from a HIP graph of twenty runs (Encoder_tile::run only launches kernels, so a
     # caller can capture it: a 12-layer model is such a graph); replays repeated with eager work in between
     side = torch.cuda.Stream()

@@ -82,6 +82,31 @@ def test_encoder_tile_layer_config3_full_size():
     assert np.array_equal(host(enc.run(xd, xd)), got)
 
 
+@pytest.mark.parametrize("kind", ["padding", "dense"])
+def test_encoder_tile_layer_config3_full_size_with_a_mask(kind):
+    """the same layer at the same size with masks that the attention launch has to read: a padding mask over the
+    last 64 keys (whole key tiles that end early, the form the benchmark's latency_us_padding_mask times) and a
+    dense random additive mask (every tile read and added); two sequences from across the batch against the
+    oracle"""
+    from et_amd.encoder import Encoder_tile
+    r = rng(561)
+    d, H, dff, S, B = 768, 12, 3072, 512, 16
+    lins, ln = make_layer(r, d, dff, 0.8, seed=906)
+    x = randn_h(r, (B * S, d))
+    if kind == "padding":
+        mask = np.zeros((S, S), np.float16)
+        mask[:, S - 64:] = -30000.0
+    else:
+        mask = randn_h(r, (S, S), 0.5)
+    sample = [0, 11]
+    rows = np.concatenate([np.arange(b * S, (b + 1) * S) for b in sample])
+    want = orc.encoder_tile_layer(x[rows], lins, ln, mask, S, H, len(sample), None, 1.0)
+    enc = Encoder_tile(d, S, H, workspace(Encoder_tile, d, S, H, B), *build_linears(lins, B * S), *ln, mask, B)
+    xd = dev(x)
+    got = host(enc.run(torch.empty_like(xd), xd))
+    check_close(got[rows], want, what=f"Encoder_tile, config 3 full size, {kind} mask")
+
+
 @pytest.mark.parametrize("d,H,dff,S,B,sp", [
     (1024, 16, 4096, 128, 8, 0.8),    # BERT-large widths: K = 1024 needs two panel chunks everywhere
     (1024, 16, 4096, 64, 1, 0.5),     # ... and on few rows
