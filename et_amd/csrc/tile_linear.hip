@@ -2620,7 +2620,10 @@ extern "C" size_t et_tile_plan_tail_ws_bytes(const et_tile_plan *pO, const et_ti
     return et::tail_pair_ws_bytes(pO, p1, p2, M);
 }
 
-extern "C" size_t et_tail_ws_bytes_for(int d_model, int rows) { return et::tail_ws_bytes_for(d_model, rows); }
+extern "C" size_t et_tail_ws_bytes_for(int d_model, int rows) {
+    // (nothing while the paired form is switched off: an encoder's workspace is then the reference's)
+    return et::tail_pair_enabled() ? et::tail_ws_bytes_for(d_model, rows) : 0;
+}
 
 extern "C" int et_tile_plan_tail_prepare(const et_tile_plan *pO, const et_tile_plan *p1,
                                          const et_tile_plan *p2) {

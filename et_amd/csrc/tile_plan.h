@@ -41,6 +41,7 @@ size_t tail_ws_bytes_for(int D, int rows);
 size_t tail_pair_ws_bytes(const et_tile_plan *pO, const et_tile_plan *p1, const et_tile_plan *p2, int M);
 int tail_pair_prepare(const et_tile_plan *pO, const et_tile_plan *p1, et_tile_plan *p2);
 bool tail_pair_forced();
+bool tail_pair_enabled();
 bool tail_pair_applies(const et_tile_plan *pO, const et_tile_plan *p1, const et_tile_plan *p2);
 int tail_pair_launch(const et_tile_plan *pO, const et_tile_plan *p1, const et_tile_plan *p2, f16 *Y,
                      const f16 *attn, const f16 *input, const f16 *gamma1, const f16 *beta1,

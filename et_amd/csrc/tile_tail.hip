@@ -672,6 +672,7 @@ static int tail_ms() { return g_tail_pair == 2 ? 4 : 2; } // 16-row subtiles per
 static int g_tail_spin = 1 << 22;    // et_tuning_set("tile_wait_spin"): polls before a bounded LDS wait gives up
 void set_tail_pair(int v) { g_tail_pair = v; }
 bool tail_pair_forced() { return g_tail_pair >= 2; }
+bool tail_pair_enabled() { return g_tail_pair != 0; }
 void set_tail_spin(int v) { g_tail_spin = v < 0 ? (1 << 22) : v; }
 int tail_spin() { return g_tail_spin; }
 

@@ -302,7 +302,9 @@ int et_tile_plan_tail_prepare(const et_tile_plan *out, const et_tile_plan *first
 /* bytes of scratch the paired form needs for M rows (0 where it does not apply) */
 size_t et_tile_plan_tail_ws_bytes(const et_tile_plan *out, const et_tile_plan *first,
                                   const et_tile_plan *second, int M);
-/* the same figure from the shapes alone (what an encoder adds to its workspace) */
+/* the same figure from the shapes alone (what an encoder adds to its workspace);
+ * 0 while the paired form is switched off (et_tuning_set "tile_tail_pair" 0, the
+ * default), so that Encoder_*::buffer_size is then the reference's five units */
 size_t et_tail_ws_bytes_for(int d_model, int rows);
 /* n (<= 4) planned linears with the same in_feat applied to the same X in ONE
  * launch (the Q/K/V projections, encoder/encoder.cu:22-26, which the

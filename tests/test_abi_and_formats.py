@@ -292,3 +292,27 @@ def test_wait_status_word_is_reported_once_and_cleared():
     assert b"gave up a bounded wait" in l.et_last_error()
     assert l.et_wait_status_take() == 0
 
+
+def test_encoder_workspace_grows_only_while_the_paired_tail_is_switched_on():
+    """Encoder_*::buffer_size is the reference's five units (encoder/encoder.h:51-53; Encoder_length adds its
+    scores) unless the paired layer tail is switched on, whose fp32 exchange area then follows them"""
+    from et_amd.encoder import Encoder_length, Encoder_tile
+    lib = _lib.lib()
+    d, S, H, B = 768, 512, 12, 16
+    units = 5 * B * S * d * 2
+    assert lib.et_tail_ws_bytes_for(d, B * S) == 0
+    assert Encoder_tile.buffer_size(d, S, H, B) == (units + 255) // 256 * 256
+    base_len = Encoder_length.buffer_size(d, S, H, B)
+    assert base_len >= units + B * H * S * S * 2
+    try:
+        for mode in (1, 2, 3):
+            assert lib.et_tuning_set(b"tile_tail_pair", mode) == 0
+            extra = lib.et_tail_ws_bytes_for(d, B * S)
+            assert extra == (B * S) * 768 * 8                      # rows (a multiple of 64) x width x two floats
+            assert Encoder_tile.buffer_size(d, S, H, B) == (units + 255) // 256 * 256 + extra
+            assert Encoder_length.buffer_size(d, S, H, B) == base_len + extra
+        assert lib.et_tail_ws_bytes_for(100, 64) == 0              # a width the paired kernel is not built for
+    finally:
+        lib.et_tuning_set(b"tile_tail_pair", 0)
+    assert Encoder_tile.buffer_size(d, S, H, B) == (units + 255) // 256 * 256
+

@@ -82,6 +82,37 @@ def test_encoder_tile_layer_config3_full_size():
     assert np.array_equal(host(enc.run(xd, xd)), got)
 
 
+@pytest.mark.parametrize("mode", [2, 3])
+def test_encoder_tile_layer_with_the_paired_tail(mode):
+    """an Encoder_tile sized and built while the paired layer tail is switched on runs its tail through
+    et_tile_plan_run_tail_ws with the exchange area behind its workspace units: the oracle's layer, the same bits
+    on a second run, and close to the default encoder's output (fp32 summation order differs)"""
+    from et_amd import lib
+    from et_amd.encoder import Encoder_tile
+    r = rng(577)
+    d, H, dff, S, B = 768, 12, 3072, 128, 10
+    lins, ln = make_layer(r, d, dff, 0.8, seed=911)
+    x = randn_h(r, (B * S, d))
+    mask = randn_h(r, (S, S), 0.3)
+    want = orc.encoder_tile_layer(x, lins, ln, mask, S, H, B, None, 1.0)
+    xd = dev(x)
+    plain = Encoder_tile(d, S, H, workspace(Encoder_tile, d, S, H, B), *build_linears(lins, B * S), *ln, mask, B)
+    base = host(plain.run(torch.empty_like(xd), xd))
+    lib().et_tuning_set(b"tile_tail_pair", mode)
+    try:
+        assert Encoder_tile.buffer_size(d, S, H, B) > 5 * B * S * d * 2
+        enc = Encoder_tile(d, S, H, workspace(Encoder_tile, d, S, H, B), *build_linears(lins, B * S), *ln, mask, B)
+        got = host(enc.run(torch.empty_like(xd), xd))
+        again = host(enc.run(torch.empty_like(xd), xd))
+    finally:
+        lib().et_tuning_set(b"tile_tail_pair", 0)
+    check_close(got, want, what=f"Encoder_tile with the paired tail (mode {mode})")
+    assert np.array_equal(got, again)
+    assert np.abs(got.astype(np.float32) - base.astype(np.float32)).max() <= 3e-2
+    assert (got != base).mean() < 0.05
+    assert (got != base).any()          # (it did take the other kernel: the fp32 sums are added in another order)
+
+
 @pytest.mark.parametrize("kind", ["padding", "dense"])
 def test_encoder_tile_layer_config3_full_size_with_a_mask(kind):
     """the same layer at the same size with masks that the attention launch has to read: a padding mask over the
