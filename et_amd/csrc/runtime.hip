@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <cstdarg>
 #include <cstring>
+#include <mutex>
 
 namespace et {
 
@@ -25,12 +26,9 @@ int hip_fail(hipError_t e, const char *what) {
 // The wait-status word: pinned host memory that the device sees, allocated
 // once per process (by the first plan that is created, never inside a run).
 static int *g_status_host = nullptr, *g_status_dev = nullptr;
-static bool g_status_tried = false;
+static std::once_flag g_status_once;
 static int g_status_local = 0; // stands in where there is no device (the host-side plumbing can still be exercised)
-static void status_init() {
-    if (g_status_tried)
-        return;
-    g_status_tried = true;
+static void status_init_once() {
     void *h = nullptr, *d = nullptr;
     if (hipHostMalloc(&h, 64, hipHostMallocMapped) != hipSuccess) {
         (void)hipGetLastError();
@@ -47,6 +45,7 @@ static void status_init() {
     g_status_host = static_cast<int *>(h);
     g_status_dev = static_cast<int *>(d);
 }
+static void status_init() { std::call_once(g_status_once, status_init_once); } // (plans are created from any thread)
 int *wait_status_device() {
     status_init();
     return g_status_dev;
