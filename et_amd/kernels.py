@@ -5,6 +5,8 @@ torch's current stream.  Names follow the reference launchers.
 """
 from __future__ import annotations
 
+import weakref
+
 import torch
 
 from ._lib import check, lib
@@ -215,16 +217,18 @@ def sharedQK_attention(QK, V, mask, seq_len, nhead, batch=1, seq_lens=None, log2
     return Z
 
 
-_checked_cu = {}   # (address, elements, seq_len, rows) -> tensor version that passed
+_checked_cu = {}   # (address, elements, seq_len, rows) -> (weak reference to the tensor object, version that passed)
 
 
 def _check_cu(cu_seqlens, seq_len, total_rows, what):
     """the packed row offsets must start at 0, rise by at most seq_len per sequence and end at the packed
     tensor's row count: the kernels trust them for every address.  Checking costs one small device-to-host copy,
     which waits for the stream; a tensor that passed is remembered by address and version counter, so only its
-    first use (and the first one after it was written to in place) synchronises."""
+    first use (and the first one after it was written to in place) synchronises.  (The very tensor object: another
+    tensor that the allocator later puts at the same address is checked again.)"""
     key = (cu_seqlens.data_ptr(), cu_seqlens.numel(), seq_len, total_rows)
-    if _checked_cu.get(key) == cu_seqlens._version:
+    hit = _checked_cu.get(key)
+    if hit is not None and hit[0]() is cu_seqlens and hit[1] == cu_seqlens._version:
         return
     cu = cu_seqlens.detach().cpu().numpy().astype("int64")
     if cu.size < 1 or cu[0] != 0 or cu[-1] != total_rows:
@@ -235,7 +239,7 @@ def _check_cu(cu_seqlens, seq_len, total_rows, what):
         raise ValueError(f"{what}: every sequence must hold 0..{seq_len} rows")
     if len(_checked_cu) > 64:
         _checked_cu.clear()
-    _checked_cu[key] = cu_seqlens._version
+    _checked_cu[key] = (weakref.ref(cu_seqlens), cu_seqlens._version)
 
 
 def pack_rows(padded, cu_seqlens, seq_len, total_rows, order=None):
