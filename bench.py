@@ -455,6 +455,32 @@ def second_targets(torch, K, dev, enc, out, x, B, S, mask_h, lins, ln):
     res["parity_vs_oracle_padding_mask"] = {"max_abs": round(float(np.abs(got - want).max()), 5),
                                             "mean_rel": round(float(np.abs(got - want).mean() / np.abs(want).mean()), 6),
                                             "rows": int(srows.size), "sequences": sample}
+    # two batches in flight: the same layer on a second set of buffers, steps alternating between two streams (a
+    # server with more than one request queue).  A launch's start-up and drain then overlap the other stream's
+    # kernel; `value` above stays the one-stream figure.
+    L2_ = [Linear_tile(l["K"], l["N"], T, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], j == 4)
+           for j, l in enumerate(lins)]
+    ws2 = torch.empty(Encoder_tile.buffer_size(D, S, H, B) // 2, dtype=torch.float16, device=dev)
+    enc2 = Encoder_tile(D, S, H, ws2, *L2_, *ln, mask_h, B)
+    x2, out2 = x.clone(), torch.empty_like(x)
+    st = [torch.cuda.Stream(), torch.cuda.Stream()]
+
+    def pair_of_steps():
+        with torch.cuda.stream(st[0]):
+            enc.run(out, x)
+        with torch.cuda.stream(st[1]):
+            enc2.run(out2, x2)
+    torch.cuda.synchronize()
+    spin_up(pair_of_steps)
+    npairs = 100
+    t0 = time.perf_counter()
+    for _ in range(npairs):
+        pair_of_steps()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    res["two_batches_in_flight"] = {"seqs_per_s": round(2 * npairs * B / dt, 1), "us_per_batch": round(dt / (2 * npairs) * 1e6, 1),
+                                    "steps": 2 * npairs, "streams": 2}
+    del enc2, ws2, L2_
     # the headline layer replayed from a HIP graph of twenty runs (Encoder_tile::run only launches kernels, so a
     # caller can capture it: a 12-layer model is such a graph); replays repeated with eager work in between
     side = torch.cuda.Stream()
