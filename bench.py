@@ -121,6 +121,9 @@ def main():
     ap.add_argument("--sparsity", type=float, default=0.8)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--extras", action="store_true", help="also time the other BASELINE configurations")
+    ap.add_argument("--one-stream", action="store_true",
+                    help="skip the two-batches-in-flight figure (for profiler runs: launches that overlap on two "
+                         "streams would mix into the per-kernel averages)")
     ap.add_argument("--micro", action="store_true",
                     help="only run the delivery-path microbenchmarks (LDS reads, weight stream, MFMA / vector-ALU "
                          "co-execution) and print their figures")
@@ -338,7 +341,7 @@ def main():
                              "sequences": sample},
         "roofline": roof, "kernels": kern, "cpu_baseline": cpu, "cpu_baseline_1thread": cpu1,
     }
-    res.update(second_targets(torch, K, dev, enc, out, x, B, S, mask_h, lins, ln))
+    res.update(second_targets(torch, K, dev, enc, out, x, B, S, mask_h, lins, ln, two_streams=not args.one_stream))
     if extras:
         res["extras"] = extras
     print(json.dumps(res))
@@ -406,7 +409,7 @@ def event_time(torch, fn, reps=100, warm=10):
     return a.elapsed_time(b) / reps * 1e3  # us
 
 
-def second_targets(torch, K, dev, enc, out, x, B, S, mask_h, lins, ln):
+def second_targets(torch, K, dev, enc, out, x, B, S, mask_h, lins, ln, two_streams=True):
     """Figures that belong in the default line next to the headline: the stand-alone skip + LayerNorm on
     operands beyond the 256 MB last-level cache (an HBM figure, not a cache figure), BASELINE config 1
     (dense layer, batch 1 x seq 128) and the headline layer with a padding mask instead of the all-zero one."""
@@ -458,29 +461,30 @@ def second_targets(torch, K, dev, enc, out, x, B, S, mask_h, lins, ln):
     # two batches in flight: the same layer on a second set of buffers, steps alternating between two streams (a
     # server with more than one request queue).  A launch's start-up and drain then overlap the other stream's
     # kernel; `value` above stays the one-stream figure.
-    L2_ = [Linear_tile(l["K"], l["N"], T, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], j == 4)
-           for j, l in enumerate(lins)]
-    ws2 = torch.empty(Encoder_tile.buffer_size(D, S, H, B) // 2, dtype=torch.float16, device=dev)
-    enc2 = Encoder_tile(D, S, H, ws2, *L2_, *ln, mask_h, B)
-    x2, out2 = x.clone(), torch.empty_like(x)
-    st = [torch.cuda.Stream(), torch.cuda.Stream()]
+    if two_streams:
+        L2_ = [Linear_tile(l["K"], l["N"], T, l["row_offset"].size, l["data"], l["row_ptr"], l["row_offset"], l["bias"], j == 4)
+               for j, l in enumerate(lins)]
+        ws2 = torch.empty(Encoder_tile.buffer_size(D, S, H, B) // 2, dtype=torch.float16, device=dev)
+        enc2 = Encoder_tile(D, S, H, ws2, *L2_, *ln, mask_h, B)
+        x2, out2 = x.clone(), torch.empty_like(x)
+        st = [torch.cuda.Stream(), torch.cuda.Stream()]
 
-    def pair_of_steps():
-        with torch.cuda.stream(st[0]):
-            enc.run(out, x)
-        with torch.cuda.stream(st[1]):
-            enc2.run(out2, x2)
-    torch.cuda.synchronize()
-    spin_up(pair_of_steps)
-    npairs = 100
-    t0 = time.perf_counter()
-    for _ in range(npairs):
-        pair_of_steps()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    res["two_batches_in_flight"] = {"seqs_per_s": round(2 * npairs * B / dt, 1), "us_per_batch": round(dt / (2 * npairs) * 1e6, 1),
-                                    "steps": 2 * npairs, "streams": 2}
-    del enc2, ws2, L2_
+        def pair_of_steps():
+            with torch.cuda.stream(st[0]):
+                enc.run(out, x)
+            with torch.cuda.stream(st[1]):
+                enc2.run(out2, x2)
+        torch.cuda.synchronize()
+        spin_up(pair_of_steps)
+        npairs = 100
+        t0 = time.perf_counter()
+        for _ in range(npairs):
+            pair_of_steps()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        res["two_batches_in_flight"] = {"seqs_per_s": round(2 * npairs * B / dt, 1),
+                                        "us_per_batch": round(dt / (2 * npairs) * 1e6, 1), "steps": 2 * npairs, "streams": 2}
+        del enc2, ws2, L2_
     # the headline layer replayed from a HIP graph of twenty runs (Encoder_tile::run only launches kernels, so a
     # caller can capture it: a 12-layer model is such a graph); replays repeated with eager work in between
     side = torch.cuda.Stream()
